@@ -1,0 +1,451 @@
+/*
+ * CPU oracle for the gradient-compression hot path (TBQ, TernGrad b-bit
+ * quantiser, GradDrop/"DGC" sparsifier).
+ *
+ * THIS FILE IS TEST INFRASTRUCTURE.  It is a plain-C restatement of the
+ * reference's CPU-runnable algorithm bodies, used only as the checker in
+ * tests, in the smoke test and as the timed CPU baseline of the benchmark.
+ * Nothing in the product library links, loads or calls it.
+ *
+ * Every function cites the reference lines it follows (paths are relative to
+ * the reference checkout).  Build with  -O2 -ffp-contract=off  so that no
+ * multiply-add is fused: the reference's x86-64 CPU build rounds the multiply
+ * and the add separately.
+ *
+ * Parity status of each function (what pins it, beyond this restatement):
+ *   orc_lcg_*            known answers of the ANSI-C LCG + closed-form jumps
+ *   orc_tbq_*            hand-derived known-answer vector, invariants,
+ *                        compiled reference headers (oracle/_ref) where built
+ *   orc_terngrad_*       known-answer payload bytes, decode error bounds,
+ *                        compiled reference headers where built
+ *   orc_gd_*             brute force on small inputs (numpy), invariants,
+ *                        compiled reference functors where built.  The
+ *                        truncation branch's tie order is implementation
+ *                        defined in the reference (unstable sort): PARITY
+ *                        UNPINNED for ties at the cut, by design; tests assert
+ *                        there are none.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define ORC_API __attribute__((visibility("default")))
+
+/* ------------------------------------------------------------------ LCG -- */
+/* ZQ_CPP_LIB/naive_random.hpp:15-33 : x <- a*x + c (mod 2^32), srand() sets
+ * the state and discards one draw. */
+#define LCG_A 1103515245u
+#define LCG_C 12345u
+
+static inline uint32_t lcg_next(uint32_t *x) {
+    *x = LCG_A * (*x) + LCG_C;
+    return *x;
+}
+static inline void lcg_srand(uint32_t *x, uint32_t seed) {
+    *x = seed;
+    (void)lcg_next(x);
+}
+
+/* k-th output (k>=1) after `x = seed`, for tests of the closed-form jump. */
+ORC_API uint32_t orc_lcg_kth(uint32_t seed, int k) {
+    uint32_t x = seed;
+    for (int i = 0; i < k; i++) lcg_next(&x);
+    return x;
+}
+
+/* naive_real_random<float>(0,1)::operator() naive_random.hpp:54-69 :
+ * float(double(rand()) / (4294967295.0 / 1.0f)). */
+static inline float lcg_real01(uint32_t *x) {
+    return (float)((double)lcg_next(x) / 4294967295.0);
+}
+ORC_API float orc_u01_from_u32(uint32_t x) {
+    return (float)((double)x / 4294967295.0);
+}
+
+/* Exhaustive proof obligation used by the GPU kernel: for every 32-bit x,
+ *   float(double(x) / 4294967295.0) == float(double(x) * (2^-32 + 2^-64)).
+ * Returns the number of x in [lo, hi] (inclusive) where they differ. */
+ORC_API uint64_t orc_u01_shortcut_mismatches(uint32_t lo, uint32_t hi) {
+    const double c = 0x1p-32 + 0x1p-64;
+    uint64_t bad = 0;
+    int64_t a = lo, b = hi;
+#pragma omp parallel for reduction(+ : bad) schedule(static)
+    for (int64_t v = a; v <= b; v++) {
+        double d = (double)(uint32_t)v;
+        float ref = (float)(d / 4294967295.0);
+        volatile double prod = d * c;
+        float alt = (float)prod;
+        if (memcmp(&ref, &alt, 4) != 0) bad++;
+    }
+    return bad;
+}
+
+/* ------------------------------------------------------------------ TBQ -- */
+/* One element of the `compress` functor, tbq_body.h:70-84. */
+static inline uint8_t tbq_step(float g, float *r, float thr, int k, uint8_t q) {
+    *r += g;
+    if (*r >= thr) {
+        q ^= (uint8_t)(3 << (k << 1));
+        *r -= thr;
+    } else if (*r <= -thr) {
+        q ^= (uint8_t)(1 << (k << 1));
+        *r += thr;
+    }
+    return q;
+}
+
+/* tbq_body, tbq_body.h:90-158 : full groups of 4 through the functor
+ * (:57-88), the last partial group with the same rule on the host (:114-155),
+ * untouched 2-bit fields stay 01. */
+ORC_API int orc_tbq_encode(const float *g, int32_t n, float *r, uint8_t *out,
+                           float thr) {
+    int32_t groups = n >> 2;
+#pragma omp parallel for schedule(static)
+    for (int32_t i = 0; i < groups; i++) {
+        uint8_t q = 85;
+        int32_t s = i << 2;
+        for (int k = 0; k < 4; k++) q = tbq_step(g[s + k], &r[s + k], thr, k, q);
+        out[i] = q;
+    }
+    int left = n & 3;
+    if (left) {
+        uint8_t q = 85;
+        int32_t s = n - left;
+        for (int j = 0; j < left; j++) q = tbq_step(g[s + j], &r[s + j], thr, j, q);
+        out[n >> 2] = q;
+    }
+    return 0;
+}
+
+/* tbq_r_body, tbq_body.h:160-200 with compressr_write_to / compressr_add_to
+ * (:22-55). */
+ORC_API int orc_tbq_decode(float *out, int32_t n, const uint8_t *in, float thr,
+                           int is_add_to) {
+#pragma omp parallel for schedule(static)
+    for (int32_t i = 0; i < n; i++) {
+        uint8_t q = (in[i >> 2] >> ((i & 3) << 1)) & 3;
+        float v = ((float)q - 1) * thr;
+        out[i] = is_add_to ? v + out[i] : v;
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------- TernGrad -- */
+static const uint8_t k_lg2[9] = {0, 0, 1, 1, 2, 2, 2, 2, 3}; /* terngrad_body.h:202 */
+
+/* thrust::minmax_element semantics (terngrad_body.h:186-190): first smallest
+ * and first largest element under operator<, so the sign of a zero extreme is
+ * that of the first element comparing equal to it. */
+static void first_minmax(const float *x, int32_t n, float *mn, float *mx) {
+    int32_t imin = 0, imax = 0;
+#ifdef _OPENMP
+    int nt = omp_get_max_threads();
+    if (n > (1 << 16) && nt > 1) {
+        int32_t *pmin = (int32_t *)malloc(sizeof(int32_t) * 2 * (size_t)nt);
+        int32_t *pmax = pmin + nt;
+#pragma omp parallel num_threads(nt)
+        {
+            int t = omp_get_thread_num();
+            int64_t lo = (int64_t)n * t / nt, hi = (int64_t)n * (t + 1) / nt;
+            int32_t a = (int32_t)lo, b = (int32_t)lo;
+            for (int64_t i = lo + 1; i < hi; i++) {
+                if (x[i] < x[a]) a = (int32_t)i;
+                if (x[b] < x[i]) b = (int32_t)i;
+            }
+            pmin[t] = a;
+            pmax[t] = b;
+        }
+        imin = pmin[0];
+        imax = pmax[0];
+        for (int t = 1; t < nt; t++) {
+            if (x[pmin[t]] < x[imin]) imin = pmin[t];
+            if (x[imax] < x[pmax[t]]) imax = pmax[t];
+        }
+        free(pmin);
+        *mn = x[imin];
+        *mx = x[imax];
+        return;
+    }
+#endif
+    for (int32_t i = 1; i < n; i++) {
+        if (x[i] < x[imin]) imin = i;
+        if (x[imax] < x[i]) imax = i;
+    }
+    *mn = x[imin];
+    *mx = x[imax];
+}
+
+/* terngrad_body, terngrad_body.h:162-307 for ONE tensor.
+ *   header  :219-224   [0]=bitwidth [1]=tail [2:6]=min [6:10]=max
+ *   scalars :204-206   gap (fp32), gap_inverse = float(1./(double(gap)+1e-8))
+ *   payload :236-269   compress_with_random (:60-99) / compress_without_random
+ *                      (:24-57); RNG seeded per output byte with seed+i
+ *   tail    :275-298   always nearbyint, written at out[out_size-1]
+ * `seed` replaces the wall-clock value the reference captures at :247-251.
+ * Returns -1 for a bitwidth that is not 1, 2, 4 or 8 (:209-212). */
+ORC_API int orc_terngrad_encode(const float *x, int32_t n, uint8_t *out,
+                                int32_t out_size, uint8_t bitwidth,
+                                int32_t enable_random, uint64_t seed) {
+    if (bitwidth > 8) return -1;
+    uint8_t blg2 = k_lg2[bitwidth];
+    if ((1 << blg2) != bitwidth) return -1;
+    float mn = 0.f, mx = 0.f;
+    if (n > 0) first_minmax(x, n, &mn, &mx);
+    float gap = (mx - mn) / ((1 << bitwidth) - 1.0f);
+    float gi = 1. / (gap + 1e-8);
+    uint8_t dlg2 = 3 - blg2;
+    uint8_t dpb = 1 << dlg2;
+    uint8_t tail = n % dpb;
+    tail = tail == 0 ? 0 : dpb - tail;
+    out[0] = bitwidth;
+    out[1] = tail;
+    memcpy(out + 2, &mn, 4);
+    memcpy(out + 6, &mx, 4);
+
+    int32_t nbytes = n >> dlg2;
+    uint8_t *pay = out + 10;
+    if (enable_random) {
+#pragma omp parallel for schedule(static)
+        for (int32_t i = 0; i < nbytes; i++) {
+            uint8_t q = 0;
+            uint32_t st;
+            lcg_srand(&st, (uint32_t)(seed + (uint64_t)(int64_t)i));
+            for (int j = 0; j < dpb; j++) {
+                float th = (x[((int64_t)i << dlg2) + j] - mn) * gi;
+                th += lcg_real01(&st);
+                uint8_t t = (uint8_t)(int32_t)th;
+                q |= (uint8_t)(t << (bitwidth * j));
+            }
+            pay[i] = q;
+        }
+    } else {
+#pragma omp parallel for schedule(static)
+        for (int32_t i = 0; i < nbytes; i++) {
+            uint8_t q = 0;
+            for (int j = 0; j < dpb; j++) {
+                float th = (x[((int64_t)i << dlg2) + j] - mn) * gi;
+                uint8_t t = (uint8_t)(int32_t)nearbyintf(th);
+                q |= (uint8_t)(t << (bitwidth * j));
+            }
+            pay[i] = q;
+        }
+    }
+    if (tail) {
+        uint8_t q = 0;
+        const float *td = x + (n - (dpb - tail));
+        for (int j = 0; j < dpb - tail; j++) {
+            uint8_t t = (uint8_t)(int32_t)nearbyintf((td[j] - mn) * gi);
+            q = q | (uint8_t)(t << (bitwidth * j));
+        }
+        out[out_size - 1] = q;
+    }
+    return 0;
+}
+
+/* terngrad_r_body, terngrad_body.h:309-409 for ONE message, with
+ * decompress_write_to / decompress_add_to (:101-159).  The element count is
+ * ((in_size-10) << lg2(dpb)) - tail (:373, :388). */
+ORC_API int orc_terngrad_decode(float *out, const uint8_t *in, int32_t in_size,
+                                int is_add_to) {
+    float mn, mx;
+    memcpy(&mn, in + 2, 4);
+    memcpy(&mx, in + 6, 4);
+    uint8_t bitwidth = in[0];
+    uint8_t tail = in[1];
+    if (bitwidth > 8) return -1;
+    float gap = (mx - mn) / ((1 << bitwidth) - 1.0f);
+    uint8_t blg2 = k_lg2[bitwidth];
+    if ((1 << blg2) != bitwidth) return -1;
+    uint8_t dlg2 = 3 - blg2;
+    int32_t cnt = ((in_size - 10) << dlg2) - tail;
+    uint8_t mask = (uint8_t)((1 << bitwidth) - 1);
+#pragma omp parallel for schedule(static)
+    for (int32_t i = 0; i < cnt; i++) {
+        uint8_t off = i & ((1 << dlg2) - 1);
+        uint8_t q = (in[(i >> dlg2) + 10] >> (off * bitwidth)) & mask;
+        float prod = q * gap;
+        out[i] = is_add_to ? (float)(prod + mn + out[i]) : (float)(prod + mn);
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------- GradDrop ("DGC") -- */
+static void radix_sort_desc_u32(uint32_t *a, uint32_t *tmp, int64_t n) {
+    /* LSD radix sort on the raw bit pattern, descending.  Used on |x| >= 0
+     * whose IEEE-754 patterns order like unsigned integers. */
+    for (int pass = 0; pass < 4; pass++) {
+        int64_t cnt[256] = {0};
+        int sh = pass * 8;
+        for (int64_t i = 0; i < n; i++) cnt[255 - ((a[i] >> sh) & 255)]++;
+        int64_t pos = 0;
+        for (int d = 0; d < 256; d++) {
+            int64_t c = cnt[d];
+            cnt[d] = pos;
+            pos += c;
+        }
+        for (int64_t i = 0; i < n; i++) tmp[cnt[255 - ((a[i] >> sh) & 255)]++] = a[i];
+        uint32_t *t = a;
+        a = tmp;
+        tmp = t;
+    }
+}
+
+typedef struct {
+    uint32_t key;
+    int32_t idx;
+} kv_t;
+
+static int kv_cmp_desc(const void *pa, const void *pb) {
+    const kv_t *a = (const kv_t *)pa, *b = (const kv_t *)pb;
+    if (a->key != b->key) return a->key > b->key ? -1 : 1;
+    return a->idx < b->idx ? -1 : (a->idx > b->idx);
+}
+
+/* Size arithmetic of gd_body, gd_body.h:112-115 and :153. */
+ORC_API void orc_gd_sizes(int32_t n, double sample_rate, double drop_ratio,
+                          int32_t *sample_cnt, int32_t *expected,
+                          int32_t *thr_index) {
+    double s_percent = 1 - drop_ratio;
+    *sample_cnt = (int32_t)ceil(n * sample_rate);
+    *expected = (int32_t)ceil(n * s_percent);
+    *thr_index = (int32_t)(*sample_cnt * s_percent);
+}
+
+/* The sampled index stream of generate_sample_G, gd_body.h:36-41 :
+ * naive_int_random<uint32_t>(0, N-1) seeded with (uint32)(t+x), one discarded
+ * draw, then rand() % N. */
+ORC_API uint32_t orc_gd_sample_index(uint64_t seed, int32_t x, int32_t n) {
+    uint32_t st;
+    lcg_srand(&st, (uint32_t)(seed + (uint64_t)(int64_t)x));
+    return lcg_next(&st) % (uint32_t)n;
+}
+
+/* gd_body, gd_body.h:102-232 for ONE tensor.
+ *   :121-128  R += G
+ *   :130-142  sample[x] = |R[idx_x]|
+ *   :145-161  sort descending, threshold = sample[int(sample_cnt*s)]
+ *   :165-173  candidates {i : R[i] > thr || R[i] < -thr}, ascending
+ *   :176-187  if more than `expected`: order by |R| descending, keep `expected`
+ *   :193-229  header int32 4+8k, index block, value block, R[idx] = 0
+ * `seed` replaces the wall-clock value captured at :138-140.  Ties in the
+ * truncation order are broken by ascending index (the reference's order among
+ * ties is unspecified).  info[0]=candidates before truncation, info[1]=kept,
+ * info[2]=threshold bits.  Scratch is private: unlike the reference nothing
+ * beyond the 4+8k message bytes of `out` is touched. */
+ORC_API int orc_gd_encode(const float *g, int32_t n, float *r, uint8_t *out,
+                          double sample_rate, double drop_ratio, uint64_t seed,
+                          int32_t *info) {
+    int32_t sample_cnt, expected, thr_index;
+    orc_gd_sizes(n, sample_rate, drop_ratio, &sample_cnt, &expected, &thr_index);
+#pragma omp parallel for schedule(static)
+    for (int32_t i = 0; i < n; i++) r[i] = g[i] + r[i];
+
+    float *sample = (float *)malloc(sizeof(float) * (size_t)(sample_cnt > 0 ? sample_cnt : 1) * 2);
+#pragma omp parallel for schedule(static)
+    for (int32_t x = 0; x < sample_cnt; x++)
+        sample[x] = fabsf(r[orc_gd_sample_index(seed, x, n)]);
+    radix_sort_desc_u32((uint32_t *)sample, (uint32_t *)sample + sample_cnt, sample_cnt);
+    float thr = sample[thr_index];
+    free(sample);
+
+    /* stable compaction, two passes so it can run in parallel */
+    int nt = 1;
+#ifdef _OPENMP
+    nt = omp_get_max_threads();
+#endif
+    int64_t *part = (int64_t *)calloc((size_t)nt + 1, sizeof(int64_t));
+#pragma omp parallel num_threads(nt)
+    {
+        int t = 0;
+#ifdef _OPENMP
+        t = omp_get_thread_num();
+#endif
+        int64_t lo = (int64_t)n * t / nt, hi = (int64_t)n * (t + 1) / nt, c = 0;
+        for (int64_t i = lo; i < hi; i++) c += (r[i] > thr) || (r[i] < -thr);
+        part[t + 1] = c;
+    }
+    for (int t = 0; t < nt; t++) part[t + 1] += part[t];
+    int64_t selected = part[nt];
+    int32_t *cand = (int32_t *)malloc(sizeof(int32_t) * (size_t)(selected > 0 ? selected : 1));
+#pragma omp parallel num_threads(nt)
+    {
+        int t = 0;
+#ifdef _OPENMP
+        t = omp_get_thread_num();
+#endif
+        int64_t lo = (int64_t)n * t / nt, hi = (int64_t)n * (t + 1) / nt, w = part[t];
+        for (int64_t i = lo; i < hi; i++)
+            if ((r[i] > thr) || (r[i] < -thr)) cand[w++] = (int32_t)i;
+    }
+    free(part);
+    if (info) {
+        info[0] = (int32_t)selected;
+        memcpy(&info[2], &thr, 4);
+    }
+    if (selected > expected) {
+        kv_t *kv = (kv_t *)malloc(sizeof(kv_t) * (size_t)selected);
+        for (int64_t i = 0; i < selected; i++) {
+            float a = fabsf(r[cand[i]]);
+            memcpy(&kv[i].key, &a, 4);
+            kv[i].idx = cand[i];
+        }
+        qsort(kv, (size_t)selected, sizeof(kv_t), kv_cmp_desc);
+        for (int32_t i = 0; i < expected; i++) cand[i] = kv[i].idx;
+        free(kv);
+        selected = expected;
+    }
+    if (info) info[1] = (int32_t)selected;
+    int32_t out_size = 4 + (int32_t)selected * 2 * 4;
+    memcpy(out, &out_size, 4);
+    int32_t *oidx = (int32_t *)(out + 4);
+    float *oval = (float *)(out + 4 + 4 * (size_t)selected);
+    for (int64_t i = 0; i < selected; i++) {
+        int32_t ix = cand[i];
+        oidx[i] = ix;
+        oval[i] = r[ix];
+        r[ix] = 0;
+    }
+    free(cand);
+    return 0;
+}
+
+/* gd_r_body, gd_body.h:283-353 for ONE message: header M (:304-306),
+ * k = (M-4)/8 (:315), -1 if in_size < M (:317-325), write mode zero-fills all
+ * out_size elements then scatters (:335-347), add mode accumulates (:328-333). */
+ORC_API int orc_gd_decode(const uint8_t *in, int32_t in_size, float *out,
+                          int32_t out_size, int is_add_to) {
+    int32_t M;
+    memcpy(&M, in, 4);
+    int32_t k = (M - 4) / 8;
+    if (in_size < M) return -1;
+    const int32_t *idx = (const int32_t *)(in + 4);
+    const float *val = (const float *)(in + 4 + 4 * (size_t)k);
+    if (is_add_to) {
+        for (int32_t x = 0; x < k; x++) out[idx[x]] += val[x];
+    } else {
+#pragma omp parallel for schedule(static)
+        for (int32_t x = 0; x < out_size; x++) out[x] = 0;
+        for (int32_t x = 0; x < k; x++) out[idx[x]] = val[x];
+    }
+    return 0;
+}
+
+ORC_API int orc_max_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
+ORC_API void orc_set_threads(int n) {
+#ifdef _OPENMP
+    omp_set_num_threads(n);
+#else
+    (void)n;
+#endif
+}
