@@ -1,0 +1,170 @@
+/*
+ * hpx — MI355X (gfx950) gradient-compression kernels behind a plain C ABI.
+ *
+ * This is the drop-in boundary for the reference extension's kernel-driver
+ * layer: each entry point below replaces one of the nine `hp_cuda_*` free
+ * functions the reference declares in hp_cuda.cpp:18-102 and defines in
+ * hp_cuda_kernel.cu.  The reference passes std::vector<T*>/std::vector<int32_t>
+ * argument lists and a cudaStream_t; here the same lists arrive as `count`
+ * plus parallel arrays of plain pointers and sizes, and the stream as an opaque
+ * hipStream_t.  Argument order and meaning follow the reference function named
+ * in each comment.
+ *
+ * Conventions
+ *   - All tensor pointers are DEVICE pointers into caller-owned memory; the
+ *     pointer/size arrays themselves are HOST arrays read during the call.
+ *   - Calls enqueue work on `stream` and return without waiting, except where a
+ *     comment says otherwise.  The reference's drivers print and continue on a
+ *     body failure; these entry points return the code instead:
+ *       0   success
+ *      -1   the reference body's own failure (bad bitwidth, short message)
+ *      -2   a HIP runtime error (hpx_last_error() has the text)
+ *      -3   an argument the kernels cannot take (null pointer, negative size)
+ *   - The library owns a small grow-only device workspace per (device, stream).
+ *     Entry points may be called from several host threads; calls that share a
+ *     stream are serialised while they enqueue.
+ *   - Sizes are int32 element/byte counts exactly as in the reference.
+ */
+#ifndef HPX_H_
+#define HPX_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* hpx_stream_t; /* a hipStream_t; NULL is the null stream */
+
+#define HPX_OK 0
+#define HPX_ERR_BODY (-1)
+#define HPX_ERR_HIP (-2)
+#define HPX_ERR_ARG (-3)
+
+/* Library version (major*10000 + minor*100 + patch). */
+int hpx_version(void);
+/* Text of the last failure on the calling thread ("" if none). */
+const char* hpx_last_error(void);
+/* Releases every workspace the library allocated (all devices, all streams).
+ * No call may be in flight.  No counterpart in the reference (its scratch is
+ * the caller's output buffer). */
+int hpx_release_workspaces(void);
+
+/* ---- TBQ: threshold quantisation with residual feedback ------------------ */
+
+/* Replaces hp_cuda_tbq (hp_cuda.cpp:52-61, hp_cuda_kernel.cu:120-158; body
+ * tbq_body.h:90-158).  For tensor t: residual += grad; each element becomes a
+ * 2-bit code (1: |r|<thr, 2: r>=thr then r-=thr, 0: r<=-thr then r+=thr), four
+ * codes per byte LSB-first, unused fields of the last byte stay 1.
+ * outs[t] needs (sizes[t]+3)/4 bytes.  grads are read-only.  The reference's
+ * unused size arguments (residual sizes, out sizes) are not part of this ABI.
+ * All tensors go out in one launch sequence; no host synchronisation (the
+ * reference's trailing cudaStreamSynchronize is left to the caller). */
+int hpx_tbq_encode(int count, const float* const* grads, const int32_t* sizes,
+                   float* const* residuals, uint8_t* const* outs,
+                   const float* thresholds, hpx_stream_t stream);
+
+/* Replaces hp_cuda_tbqr (hp_cuda.cpp:41-50, hp_cuda_kernel.cu:161-198; body
+ * tbq_body.h:160-200).  outs[t][i] = (code-1)*thr, added to the existing value
+ * when is_add_tos[t] != 0. */
+int hpx_tbq_decode(int count, float* const* outs, const int32_t* sizes,
+                   const uint8_t* const* ins, const float* thresholds,
+                   const int32_t* is_add_tos, hpx_stream_t stream);
+
+/* ---- TernGrad: b-bit min/max quantiser, b in {1,2,4,8} -------------------- */
+
+/* Replaces hp_cuda_terngrad (hp_cuda.cpp:21-29, hp_cuda_kernel.cu:30-65; body
+ * terngrad_body.h:162-307).  Message layout: [0]=bitwidth, [1]=unused slots in
+ * the last byte, [2:6]=min, [6:10]=max (fp32 LE), [10:] codes LSB-first.
+ * out_sizes[t] must be 10 + ceil(n/(8/b)): a partial last byte is written at
+ * outs[t][out_sizes[t]-1] as in the reference (and always rounds to nearest).
+ * enable_randoms[t] != 0 selects stochastic rounding with the reference's LCG
+ * seeded per output byte from seeds[t] + byte index.  The reference takes that
+ * seed from the wall clock inside the body (terngrad_body.h:247-251); pass
+ * seeds == NULL for that behaviour, or an array of `count` values to fix it.
+ * Returns -1 without launching if any bitwidth is not 1, 2, 4 or 8
+ * (terngrad_body.h:207-212). */
+int hpx_terngrad_encode(int count, const float* const* ins, const int32_t* in_sizes,
+                        uint8_t* const* outs, const int32_t* out_sizes,
+                        const uint8_t* bitwidths, const int32_t* enable_randoms,
+                        const uint64_t* seeds, hpx_stream_t stream);
+
+/* Replaces hp_cuda_terngradr (hp_cuda.cpp:31-38, hp_cuda_kernel.cu:200-230;
+ * body terngrad_body.h:309-409).  The header is parsed on the device, so the
+ * call does not wait for the stream (the reference copies it to the host and
+ * synchronises).  The element count is ((in_size-10)*(8/b)) - tail as in the
+ * reference, and is additionally clamped to out_sizes[t] so a malformed header
+ * cannot write outside the output.  A message whose bitwidth byte is invalid
+ * decodes to nothing and raises the sticky flag hpx_terngrad_decode_status
+ * reports. */
+int hpx_terngrad_decode(int count, float* const* outs, const int32_t* out_sizes,
+                        const uint8_t* const* ins, const int32_t* in_sizes,
+                        const int32_t* is_add_tos, hpx_stream_t stream);
+
+/* Waits for `stream`, then returns -1 if any hpx_terngrad_decode on it since
+ * the last status call met an invalid bitwidth byte (the reference's
+ * terngrad_r_body failure, terngrad_body.h:352-355), else 0. */
+int hpx_terngrad_decode_status(hpx_stream_t stream);
+
+/* ---- GradDrop ("DGC"): sampled-threshold top-k sparsifier ----------------- */
+
+/* Replaces hp_cuda_gd (hp_cuda.cpp:64-73, hp_cuda_kernel.cu:67-94; body
+ * gd_body.h:102-232).  Per tensor: residual += grad; threshold = the
+ * int(sample_cnt*(1-drop))-th largest of sample_cnt = ceil(N*sample_rate)
+ * sampled |residual| values (indices from the reference's LCG seeded with
+ * seeds[t] + sample number); select {i : r[i] > thr || r[i] < -thr}; if more
+ * than ceil(N*(1-drop)) were selected keep that many largest |r|.  Message:
+ * int32 4+8k, k int32 indices, k fp32 values; residual[idx] = 0.  Indices are
+ * ascending when nothing was cut and in descending |r| order when cut (ties:
+ * ascending index).  seeds == NULL takes the wall clock (gd_body.h:138-140).
+ * Unlike the reference, bytes of outs[t] past the message are left untouched
+ * (scratch lives in the library workspace), so outs[t] needs only
+ * 4 + 8*ceil(N*(1-drop)) bytes.  The call waits for the stream once per tensor
+ * (the reference waits three times). */
+int hpx_gd_encode(int count, const float* const* grads, const int32_t* Ns,
+                  float* const* residuals, uint8_t* const* outs,
+                  const double* sample_rates, const double* drop_ratios,
+                  const uint64_t* seeds, hpx_stream_t stream);
+
+/* Replaces hp_cuda_gdr (hp_cuda.cpp:75-82, hp_cuda_kernel.cu:96-118; body
+ * gd_body.h:283-353).  Reads every header first (one wait on the stream, as in
+ * the reference); returns -1 before touching any output if a message is longer
+ * than its in_sizes[t].  is_add_tos[t] == 0 zero-fills out_sizes[t] elements
+ * and then scatters; otherwise accumulates. */
+int hpx_gd_decode(int count, const uint8_t* const* ins, const int32_t* in_sizes,
+                  float* const* outs, const int32_t* out_sizes,
+                  const int32_t* is_add_tos, hpx_stream_t stream);
+
+/* ---- PowerSGD: rank-r factorisation with error feedback ------------------- */
+/* The reference bodies operate on torch tensors (powersgd_body.h); here every
+ * matrix is a row-major fp32 device array: M is n x m, Q is m x r, P is n x r,
+ * grad/residual hold numel <= n*m elements (the flat prefix of M). */
+
+/* Replaces hp_cuda_powersgd_encode1 (hp_cuda.cpp:85-92,
+ * hp_cuda_kernel.cu:232-255; powersgd_body.h:10-31 as its comments state it):
+ * M.flat[:numel] = grad + residual;  P = M * Q. */
+int hpx_powersgd_encode1(int count, const float* const* grads, const int64_t* numels,
+                         const float* const* residuals, const float* const* Qs,
+                         float* const* Ms, float* const* Ps, const int32_t* ns,
+                         const int32_t* ms, const int32_t* rs, hpx_stream_t stream);
+
+/* Replaces hp_cuda_powersgd_encode2 (hp_cuda.cpp:93-98,
+ * hp_cuda_kernel.cu:257-276; powersgd_body.h:33-52): P <- orthonormal basis of
+ * its columns (modified Gram-Schmidt; equals the reference's Householder Q
+ * factor up to the sign of each column), then Q = M^T * P. */
+int hpx_powersgd_encode2(int count, float* const* Ps, const float* const* Ms,
+                         float* const* Qs, const int32_t* ns, const int32_t* ms,
+                         const int32_t* rs, hpx_stream_t stream);
+
+/* Replaces hp_cuda_powersgd_decode (hp_cuda.cpp:99-106,
+ * hp_cuda_kernel.cu:278-301; powersgd_body.h:54-78): M = P * Q^T;
+ * residual = grad - M.flat[:numel];  grad = M.flat[:numel]. */
+int hpx_powersgd_decode(int count, const float* const* Ps, const float* const* Qs,
+                        float* const* Ms, float* const* residuals, float* const* grads,
+                        const int64_t* numels, const int32_t* ns, const int32_t* ms,
+                        const int32_t* rs, hpx_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HPX_H_ */

@@ -1,0 +1,47 @@
+import importlib
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+@pytest.fixture(scope="session")
+def pkg():
+    """The product package (its directory name is not a Python identifier)."""
+    return importlib.import_module("torch-hipress-extension_amd")
+
+
+@pytest.fixture(scope="session")
+def capi(pkg):
+    pkg._capi.load()
+    return pkg._capi
+
+
+@pytest.fixture(scope="session")
+def oracle_cpu():
+    from oracle import cpu
+    cpu.lib()
+    return cpu
+
+
+@pytest.fixture(scope="session")
+def oracle_ref():
+    """The reference's own bodies compiled for the host; optional."""
+    from oracle import ref
+    if not ref.available():
+        try:
+            ref.build()
+        except Exception:
+            pass
+    if not ref.available():
+        pytest.skip("oracle/_ref not built (no reference checkout here)")
+    ref.lib()
+    return ref

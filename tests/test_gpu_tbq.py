@@ -1,0 +1,150 @@
+"""GPU parity: TBQ encode/decode through the C ABI vs the CPU oracle (bit-exact)."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import Tbq, assert_bits_equal, dev, host
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def tbq(capi):
+    assert torch.cuda.is_available()
+    return Tbq(capi)
+
+
+def _roundtrip(tbq, oracle_cpu, gs, rs, thrs, adds, rng):
+    dg = [dev(g) for g in gs]
+    dr = [dev(r) for r in rs]
+    packed = tbq.encode(dg, dr, thrs)
+    torch.cuda.synchronize()
+    for i, (g, r, thr) in enumerate(zip(gs, rs, thrs)):
+        r_ref = r.copy()
+        p_ref = oracle_cpu.tbq_encode(g, r_ref, thr)
+        assert_bits_equal(host(packed[i]), p_ref, f"packed[{i}] n={g.size}")
+        assert_bits_equal(host(dr[i]), r_ref, f"residual[{i}] n={g.size}")
+        assert_bits_equal(host(dg[i]), g, f"gradient[{i}] must be untouched")
+    bases = [rng.normal(0, 1, g.size).astype(np.float32) for g in gs]
+    douts = [dev(b) for b in bases]
+    tbq.decode(packed, douts, thrs, adds)
+    torch.cuda.synchronize()
+    for i, (g, thr, add) in enumerate(zip(gs, thrs, adds)):
+        ref = oracle_cpu.tbq_decode(host(packed[i]), g.size, thr, bases[i].copy(), add)
+        assert_bits_equal(host(douts[i]), ref, f"decoded[{i}] n={g.size} add={add}")
+
+
+def test_known_answer(tbq, oracle_cpu):
+    g = np.array([.003, -.003, .001, -.001, .002, -.002, 0, .0041, .5, -.5], np.float32)
+    dr = dev(np.zeros(10, np.float32))
+    packed = tbq.encode([dev(g)], [dr], [0.002])
+    torch.cuda.synchronize()
+    assert host(packed[0]).tolist() == [82, 146, 82]
+    out = dev(np.zeros(10, np.float32))
+    tbq.decode(packed, [out], [0.002], [0])
+    np.testing.assert_array_equal(host(out), np.array([.002, -.002, 0, 0, .002, -.002, 0, .002, .002, -.002], np.float32))
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 255, 4095, 4096, 4097, 4099, 8191, 1 << 20, (1 << 20) + 1, 3000001])
+def test_single_tensor_sizes(tbq, oracle_cpu, n):
+    rng = np.random.default_rng(n)
+    g = rng.normal(0, 1e-3, n).astype(np.float32)
+    r = rng.normal(0, 1e-3, n).astype(np.float32)
+    for add in (0, 1):
+        _roundtrip(tbq, oracle_cpu, [g], [r], [2e-3], [add], rng)
+
+
+def test_config1_zero_residual(tbq, oracle_cpu):
+    # 1,048,576 elements ~N(0,1e-3), threshold 2e-3, zero residual, seed 0
+    rng = np.random.default_rng(0)
+    g = rng.normal(0, 1e-3, 1 << 20).astype(np.float32)
+    _roundtrip(tbq, oracle_cpu, [g], [np.zeros_like(g)], [2e-3], [0], rng)
+
+
+def test_special_values(tbq, oracle_cpu):
+    rng = np.random.default_rng(5)
+    thr = np.float32(2e-3)
+    g = np.array([thr, -thr, np.nextafter(thr, 0), -np.nextafter(thr, 0), 0.0, -0.0, 1e-45, -1e-45, 1e30, -1e30,
+                  3 * thr, -3 * thr, 1.5e-3, -1.5e-3, 7.0], np.float32)
+    r = np.array([0, 0, 0, 0, thr, -thr, 0, 0, 0, 0, 0, 0, 1e-3, -1e-3, -7.0], np.float32)
+    _roundtrip(tbq, oracle_cpu, [g], [r], [float(thr)], [1], rng)
+    # zero and negative thresholds follow the same comparisons
+    _roundtrip(tbq, oracle_cpu, [g], [r], [0.0], [0], rng)
+    _roundtrip(tbq, oracle_cpu, [g], [r], [-1e-3], [0], rng)
+
+
+def test_unaligned_views(tbq, oracle_cpu):
+    # tensors that start at an odd element / odd byte of their allocation
+    rng = np.random.default_rng(9)
+    n = 10007
+    g = rng.normal(0, 1e-3, n).astype(np.float32)
+    r = rng.normal(0, 1e-3, n).astype(np.float32)
+    gbuf = torch.zeros(n + 3, device="cuda"); rbuf = torch.zeros(n + 3, device="cuda")
+    obuf = torch.zeros((n + 3) // 4 + 3, dtype=torch.uint8, device="cuda")
+    dg, dr, do = gbuf[1:1 + n], rbuf[3:3 + n], obuf[3:3 + (n + 3) // 4]
+    dg.copy_(dev(g)); dr.copy_(dev(r))
+    tbq.encode([dg], [dr], [2e-3], outs=[do])
+    torch.cuda.synchronize()
+    r_ref = r.copy()
+    p_ref = oracle_cpu.tbq_encode(g, r_ref, 2e-3)
+    assert_bits_equal(host(do), p_ref, "packed")
+    assert_bits_equal(host(dr), r_ref, "residual")
+    assert host(obuf[:3]).tolist() == [0, 0, 0] and float(rbuf[:3].abs().sum()) == 0.0
+    out = torch.zeros(n + 1, device="cuda")
+    tbq.decode([do], [out[1:]], [2e-3], [0])
+    assert_bits_equal(host(out[1:]), oracle_cpu.tbq_decode(p_ref, n, 2e-3), "decoded")
+    assert float(out[0]) == 0.0
+
+
+def test_bucket_of_many_tensors(tbq, oracle_cpu):
+    # More tensors than one launch table holds, ragged sizes, per-tensor thresholds,
+    # an empty tensor in the middle; two consecutive steps exercise residual feedback.
+    rng = np.random.default_rng(1)
+    sizes = [int(s) for s in np.exp(rng.uniform(np.log(3), np.log(60000), 230))]
+    sizes[17] = 0
+    gs = [rng.normal(0, 5e-3, n).astype(np.float32) for n in sizes]
+    rs = [np.zeros(n, np.float32) for n in sizes]
+    thrs = [float(np.float32(rng.uniform(5e-3, 2e-2))) for _ in sizes]
+    dg = [dev(g) if g.size else torch.empty(0, device="cuda") for g in gs]
+    dr = [dev(r) if r.size else torch.empty(0, device="cuda") for r in rs]
+    for step in range(2):
+        packed = tbq.encode(dg, dr, thrs)
+        torch.cuda.synchronize()
+        for i, n in enumerate(sizes):
+            p_ref = oracle_cpu.tbq_encode(gs[i], rs[i], thrs[i])
+            assert_bits_equal(host(packed[i]), p_ref, f"step {step} packed[{i}] n={n}")
+            assert_bits_equal(host(dr[i]), rs[i], f"step {step} residual[{i}] n={n}")
+    outs = [torch.zeros(n, device="cuda") for n in sizes]
+    tbq.decode(packed, outs, thrs, [i & 1 for i in range(len(sizes))])
+    torch.cuda.synchronize()
+    for i, n in enumerate(sizes):
+        assert_bits_equal(host(outs[i]), oracle_cpu.tbq_decode(host(packed[i]), n, thrs[i]), f"decoded[{i}]")
+
+
+def test_full_size_bucket_properties(tbq):
+    # 110M-element bucket (BERT-base-like): size-independent properties only.
+    rng = np.random.default_rng(0)
+    sizes = np.exp(rng.uniform(np.log(768), np.log(3e7), 200))
+    sizes = np.clip(np.floor(sizes * 110e6 / sizes.sum()), 768, 3e7).astype(np.int64)
+    sizes[np.argmax(sizes)] += 110_000_000 - sizes.sum()
+    assert sizes.sum() == 110_000_000
+    thr = 1e-2
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    gs = [torch.randn(int(n), device="cuda", generator=gen) * 5e-3 for n in sizes]
+    rs = [torch.zeros(int(n), device="cuda") for n in sizes]
+    g_sum = [float(g.double().sum()) for g in gs[:5]]
+    packed = tbq.encode(gs, rs, [thr] * len(gs))
+    outs = [torch.empty(int(n), device="cuda") for n in sizes]
+    tbq.decode(packed, outs, [thr] * len(gs), [0] * len(gs))
+    torch.cuda.synchronize()
+    t = torch.tensor(thr, dtype=torch.float32, device="cuda")
+    for i in (0, 1, 2, int(np.argmax(sizes)), len(gs) - 1):
+        g, r, o = gs[i], rs[i], outs[i]
+        # decode takes only the values {-thr, 0, thr}; decode + residual == gradient (residual started at 0)
+        assert bool(((o == 0) | (o == t) | (o == -t)).all())
+        assert float((o.double() + r.double() - g.double()).abs().max()) < 1e-9
+        small = g.abs() < 2 * t - 1e-7
+        assert bool((r[small].abs() < t).all())
+        codes = packed[i]
+        assert int(((codes >> 0) & 3 == 3).sum() + ((codes >> 2) & 3 == 3).sum()) == 0
+    assert [float(g.double().sum()) for g in gs[:5]] == g_sum  # gradients untouched

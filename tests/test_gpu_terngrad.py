@@ -1,0 +1,169 @@
+"""GPU parity: TernGrad b-bit quantiser through the C ABI vs the CPU oracle (bit-exact)."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import Terngrad, assert_bits_equal, dev, host
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def tg(capi):
+    assert torch.cuda.is_available()
+    return Terngrad(capi)
+
+
+def _check(tg, oracle_cpu, xs, bws, rnds, seeds, adds, rng):
+    dx = [dev(x) for x in xs]
+    outs = tg.encode(dx, bws, rnds, seeds)
+    torch.cuda.synchronize()
+    for i, x in enumerate(xs):
+        rc, ref = oracle_cpu.terngrad_encode(x, bws[i], rnds[i], seeds[i])
+        assert rc == 0
+        assert_bits_equal(host(outs[i])[:10], ref[:10], f"header[{i}] n={x.size} b={bws[i]}")
+        assert_bits_equal(host(outs[i]), ref, f"message[{i}] n={x.size} b={bws[i]} rnd={rnds[i]}")
+        assert_bits_equal(host(dx[i]), x, "input untouched")
+    bases = [rng.normal(0, 1, x.size).astype(np.float32) for x in xs]
+    douts = [dev(b) for b in bases]
+    tg.decode(outs, douts, adds)
+    torch.cuda.synchronize()
+    for i, x in enumerate(xs):
+        rc, ref = oracle_cpu.terngrad_decode(host(outs[i]), x.size, bases[i].copy(), adds[i])
+        assert rc == 0
+        assert_bits_equal(host(douts[i]), ref, f"decoded[{i}] n={x.size} b={bws[i]} add={adds[i]}")
+    assert tg.status() == 0
+
+
+def test_known_answers(tg):
+    x = (np.array([(7 * i % 11) - 5 for i in range(40)], np.float32) * np.float32(0.01)).astype(np.float32)
+    out = tg.encode([dev(x)], [2], [1], [12345])[0]
+    assert host(out)[10:15].tobytes().hex() == "c8b22cb72d"
+    out = tg.encode([dev(x[:22].copy())], [2], [0], [0])[0]
+    assert host(out).tobytes().hex() == "0202cccc4cbdcccc4c3dd87618b61d06"
+
+
+@pytest.mark.parametrize("b", [1, 2, 4, 8])
+@pytest.mark.parametrize("rnd", [0, 1])
+def test_sizes_and_tails(tg, oracle_cpu, b, rnd):
+    rng = np.random.default_rng(100 * b + rnd)
+    sizes = [1, 2, 3, 4, 5, 7, 8, 9, 15, 16, 17, 1023, 4095, 4096, 4097, 8191, 8192, 8193, 8199, 32768 + 5, 300007]
+    xs = [rng.normal(0, 1e-2, n).astype(np.float32) for n in sizes]
+    seeds = [int(s) for s in rng.integers(0, 2**63, len(sizes))]
+    _check(tg, oracle_cpu, xs, [b] * len(sizes), [rnd] * len(sizes), seeds, [i & 1 for i in range(len(sizes))], rng)
+
+
+def test_more_tensors_than_one_table(tg, oracle_cpu):
+    rng = np.random.default_rng(21)
+    sizes = [int(s) for s in np.exp(rng.uniform(np.log(2), np.log(40000), 150))]
+    xs = [rng.normal(0, 1e-2, n).astype(np.float32) for n in sizes]
+    bws = [int(b) for b in rng.choice([1, 2, 4, 8], len(sizes))]
+    rnds = [int(r) for r in rng.integers(0, 2, len(sizes))]
+    seeds = [int(s) for s in rng.integers(0, 2**64 - 1, len(sizes), dtype=np.uint64)]
+    _check(tg, oracle_cpu, xs, bws, rnds, seeds, [int(a) for a in rng.integers(0, 2, len(sizes))], rng)
+
+
+def test_seed_edges(tg, oracle_cpu):
+    rng = np.random.default_rng(4)
+    x = rng.normal(0, 1e-2, 70001).astype(np.float32)
+    seeds = [0, 1, 2**32 - 1, 2**32, 2**32 - 70001 // 4 + 5, 2**63, 2**64 - 1, 1700000000123456789]
+    _check(tg, oracle_cpu, [x] * len(seeds), [2] * len(seeds), [1] * len(seeds), seeds, [0] * len(seeds), rng)
+
+
+def test_scalar_preparation_many_ranges(tg, oracle_cpu):
+    # gap (fp32 divide) and 1/(gap+1e-8) (fp64) are computed on the device: sweep min/max over many magnitudes
+    rng = np.random.default_rng(8)
+    xs, bws = [], []
+    for k in range(240):
+        lo = np.float32(rng.normal() * 10.0 ** rng.uniform(-30, 20))
+        hi = np.float32(lo + abs(np.float32(rng.normal() * 10.0 ** rng.uniform(-38, 20))))
+        n = int(rng.integers(2, 40))
+        x = rng.uniform(lo, hi, n).astype(np.float32)
+        x[0], x[-1] = lo, hi
+        xs.append(x)
+        bws.append(int(rng.choice([1, 2, 4, 8])))
+    seeds = [int(s) for s in rng.integers(0, 2**63, len(xs))]
+    for rnd in (0, 1):
+        _check(tg, oracle_cpu, xs, bws, [rnd] * len(xs), seeds, [0] * len(xs), rng)
+
+
+def test_constant_and_zero_tensors(tg, oracle_cpu):
+    rng = np.random.default_rng(2)
+    xs = [np.zeros(1000, np.float32), np.full(1003, -0.0, np.float32), np.full(4097, 0.125, np.float32),
+          np.array([0.5, -0.0, 0.0, 0.25, 0.0], np.float32), np.array([-0.5, 0.0, -0.0, -0.25], np.float32),
+          np.concatenate([np.full(20000, 0.5, np.float32), [-0.0], np.full(9000, 0.25, np.float32), [0.0]]).astype(np.float32),
+          np.array([1e-45, 0, 3e-45, 2e-45] * 50, np.float32)]
+    for rnd in (0, 1):
+        _check(tg, oracle_cpu, xs, [2] * len(xs), [rnd] * len(xs), [77] * len(xs), [0] * len(xs), rng)
+
+
+def test_outliers_config_shape_small(tg, oracle_cpu):
+    # the config-2 distribution at a size the oracle finishes quickly
+    rng = np.random.default_rng(0)
+    n = 2_000_003
+    x = rng.normal(0, 1e-2, n).astype(np.float32)
+    pos = rng.choice(n, n // 1000, replace=False)
+    x[pos] = np.where(rng.random(pos.size) < 0.5, 0.5, -0.5).astype(np.float32)
+    _check(tg, oracle_cpu, [x], [2], [1], [0], [0], rng)
+    _check(tg, oracle_cpu, [x], [2], [0], [0], [1], rng)
+
+
+def test_unaligned_views(tg, oracle_cpu):
+    rng = np.random.default_rng(12)
+    n = 30011
+    x = rng.normal(0, 1e-2, n).astype(np.float32)
+    xbuf = torch.zeros(n + 3, device="cuda")
+    dx = xbuf[3:3 + n]; dx.copy_(dev(x))
+    size = tg.packed_size(n, 2)
+    obuf = torch.zeros(size + 5, dtype=torch.uint8, device="cuda")
+    out = obuf[1:1 + size]
+    tg.encode([dx], [2], [1], [5], outs=[out])
+    rc, ref = oracle_cpu.terngrad_encode(x, 2, 1, 5)
+    assert_bits_equal(host(out), ref, "message")
+    assert host(obuf[:1]).tolist() == [0] and host(obuf[1 + size:]).tolist() == [0, 0, 0, 0]
+    dbuf = torch.zeros(n + 1, device="cuda")
+    tg.decode([out], [dbuf[1:]], [0])
+    rc, dref = oracle_cpu.terngrad_decode(ref, n)
+    assert_bits_equal(host(dbuf[1:]), dref, "decoded")
+
+
+def test_invalid_bitwidth_paths(tg):
+    x = dev(np.arange(16, dtype=np.float32))
+    out = torch.zeros(26, dtype=torch.uint8, device="cuda")
+    tg.encode([x], [3], [0], [0], outs=[out], expect_rc=-1)       # terngrad_body.h:207-212
+    assert int(out.sum()) == 0
+    # a header whose bitwidth byte is invalid decodes to nothing and is reported
+    bad = torch.zeros(14, dtype=torch.uint8, device="cuda"); bad[0] = 3
+    dst = torch.full((16,), 7.0, device="cuda")
+    tg.decode([bad], [dst], [0])
+    assert tg.status() == -1
+    assert bool((dst == 7.0).all())
+    assert tg.status() == 0   # the flag is cleared once reported
+
+
+def test_full_size_config2_properties(tg):
+    # 25,557,032 elements (ResNet-50), 0.1% outliers at +-50 sigma: size-independent properties
+    n = 25_557_032
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    x = torch.randn(n, device="cuda", generator=gen) * 1e-2
+    pos = torch.randperm(n, device="cuda", generator=gen)[: n // 1000]
+    x[pos] = torch.where(torch.rand(pos.numel(), device="cuda", generator=gen) < 0.5, 0.5, -0.5)
+    out = tg.encode([x], [2], [1], [0])[0]
+    dec = torch.empty(n, device="cuda")
+    tg.decode([out], [dec], [0])
+    torch.cuda.synchronize()
+    hdr = host(out[:10])
+    assert hdr[0] == 2 and hdr[1] == 0
+    mn, mx = hdr[2:6].view(np.float32)[0], hdr[6:10].view(np.float32)[0]
+    assert mn == float(x.min()) and mx == float(x.max())
+    gap = (float(mx) - float(mn)) / 3
+    err = (dec.double() - x.double()).abs()
+    assert float(err.max()) <= gap * (1 + 1e-4) + 1e-7        # stochastic rounding moves at most one level
+    assert abs(float((dec.double() - x.double()).mean())) < gap * 2e-3   # and is unbiased
+    levels = torch.unique(dec)
+    assert levels.numel() <= 4
+    # idempotence: re-encoding the decoded tensor deterministically returns the same codes
+    out2 = tg.encode([dec], [2], [0], [0])[0]
+    torch.cuda.synchronize()
+    same = (out2[10:] == out[10:]).float().mean()
+    assert float(same) == 1.0

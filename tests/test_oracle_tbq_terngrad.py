@@ -1,0 +1,231 @@
+"""Pins the plain-C oracle for the LCG, TBQ and TernGrad (CPU only).
+
+Checks that do not retype the oracle's formula: published/hand-derived known
+answers, closed-form LCG jumps, algebraic invariants, and (where oracle/_ref is
+built) the reference's own header bodies on the same seeded inputs.
+"""
+import numpy as np
+import pytest
+
+A, C_ = 1103515245, 12345
+M32 = 0xFFFFFFFF
+
+
+# ---- LCG (naive_random.hpp:15-33) ------------------------------------------
+def test_lcg_known_answers(oracle_cpu):
+    # ANSI-C LCG from seed 0: 12345, then a*x+c repeatedly
+    assert [oracle_cpu.lcg_kth(0, k) for k in range(1, 6)] == [12345, 3554416254, 2802067423, 3596950572, 229283573]
+
+
+def test_lcg_closed_form_jumps(oracle_cpu):
+    # x_k = A_k * s + C_k with the jump constants the GPU kernels rely on
+    jumps = {1: (1103515245, 12345), 2: (3265436265, 3554416254), 3: (2155723957, 2802067423),
+             4: (3993403153, 3596950572), 5: (3953215549, 229283573)}
+    rng = np.random.default_rng(0)
+    for s in [0, 1, M32, 0x80000000] + rng.integers(0, 2**32, 50).tolist():
+        for k, (ak, ck) in jumps.items():
+            assert oracle_cpu.lcg_kth(s, k) == (ak * s + ck) & M32
+    # and the constants follow from the recurrence itself
+    a, c = 1, 0
+    for k in range(1, 6):
+        a, c = (a * A) & M32, (c * A + C_) & M32
+        assert (a, c) == jumps[k]
+
+
+def test_u01_matches_python_float_division(oracle_cpu):
+    for x in [0, 1, 2, 0x7FFFFFFF, 0x80000000, 0x80000080, 0xFFFFFF7F, 0xFFFFFD7F, 0xFFFFFFFE, 0xFFFFFFFF]:
+        assert oracle_cpu.u01_from_u32(x) == np.float32(x / 4294967295.0)
+    assert oracle_cpu.u01_from_u32(0xFFFFFFFF) == np.float32(1.0)  # u can be exactly 1
+
+
+def test_u01_multiply_shortcut_is_exact_for_all_inputs(oracle_cpu):
+    # The GPU evaluates float(double(x)/4294967295.0) as float(double(x)*0x1.00000001p-32).
+    assert oracle_cpu.u01_shortcut_mismatches(0, 0xFFFFFFFF) == 0
+
+
+# ---- TBQ (tbq_body.h) ------------------------------------------------------
+def test_tbq_known_answer(oracle_cpu):
+    g = np.array([.003, -.003, .001, -.001, .002, -.002, 0, .0041, .5, -.5], np.float32)
+    r = np.zeros(10, np.float32)
+    packed = oracle_cpu.tbq_encode(g, r, 0.002)
+    assert packed.tolist() == [82, 146, 82]
+    np.testing.assert_allclose(r, [.001, -.001, .001, -.001, 0, 0, 0, .0021, .498, -.498], atol=1e-7)
+    dec = oracle_cpu.tbq_decode(packed, 10, 0.002)
+    np.testing.assert_array_equal(dec, np.array([.002, -.002, 0, 0, .002, -.002, 0, .002, .002, -.002], np.float32))
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 1023, 4096, 100003])
+def test_tbq_invariants(oracle_cpu, n):
+    rng = np.random.default_rng(n)
+    thr = np.float32(2e-3)
+    g = rng.normal(0, 1e-3, n).astype(np.float32)
+    r0 = rng.normal(0, 1e-3, n).astype(np.float32)
+    g_copy, r = g.copy(), r0.copy()
+    packed = oracle_cpu.tbq_encode(g, r, thr)
+    assert np.array_equal(g, g_copy)                      # gradient is read-only
+    assert packed.size == (n + 3) // 4
+    codes = (packed[:, None] >> (2 * np.arange(4))) & 3
+    codes = codes.ravel()
+    assert np.all(codes[n:] == 1)                         # padding fields stay 01
+    assert np.all(codes[:n] != 3)                         # code 3 is never produced
+    dec = oracle_cpu.tbq_decode(packed, n, thr)
+    acc = g.astype(np.float64) + r0.astype(np.float64)
+    np.testing.assert_allclose(dec.astype(np.float64) + r, acc, atol=4e-10)  # decode + residual == r + g
+    small = np.abs(acc) < 2 * thr - 1e-7
+    assert np.all(np.abs(r[small]) < thr)
+    # add mode adds the same values
+    base = rng.normal(0, 1, n).astype(np.float32)
+    added = oracle_cpu.tbq_decode(packed, n, thr, base.copy(), 1)
+    np.testing.assert_array_equal(added, dec + base)
+
+
+def test_tbq_code3_decodes_to_twice_threshold(oracle_cpu):
+    dec = oracle_cpu.tbq_decode(np.array([0b11100100], np.uint8), 4, 0.5)
+    np.testing.assert_array_equal(dec, np.array([-0.5, 0, 0.5, 1.0], np.float32))
+
+
+@pytest.mark.parametrize("policy", [0, 1])
+def test_tbq_against_reference_bodies(oracle_cpu, oracle_ref, policy):
+    rng = np.random.default_rng(7)
+    for n in [1, 2, 3, 4, 5, 7, 8, 1000, 1001, 1002, 1003, 262147]:
+        g = rng.normal(0, 1e-3, n).astype(np.float32)
+        r0 = rng.normal(0, 1e-3, n).astype(np.float32)
+        ra, rb = r0.copy(), r0.copy()
+        pa = oracle_cpu.tbq_encode(g, ra, 2e-3)
+        pb = oracle_ref.tbq_encode(g.copy(), rb, 2e-3, policy)
+        assert np.array_equal(pa, pb) and np.array_equal(ra.view(np.uint32), rb.view(np.uint32))
+        for add in (0, 1):
+            base = rng.normal(0, 1, n).astype(np.float32)
+            da = oracle_cpu.tbq_decode(pa, n, 2e-3, base.copy(), add)
+            db = oracle_ref.tbq_decode(pa, n, 2e-3, base.copy(), add, policy)
+            assert np.array_equal(da.view(np.uint32), db.view(np.uint32))
+
+
+# ---- TernGrad (terngrad_body.h) --------------------------------------------
+def _kat_x(n):
+    return (np.array([(7 * i % 11) - 5 for i in range(n)], np.float32) * np.float32(0.01)).astype(np.float32)
+
+
+def test_terngrad_known_answer_random(oracle_cpu):
+    rc, out = oracle_cpu.terngrad_encode(_kat_x(40), 2, 1, 12345)
+    assert rc == 0
+    assert out[10:15].tobytes().hex() == "c8b22cb72d"
+    assert out[0] == 2 and out[1] == 0
+    assert out[2:6].view(np.float32)[0] == np.float32(-5) * np.float32(0.01)
+    assert out[6:10].view(np.float32)[0] == np.float32(5) * np.float32(0.01)
+
+
+def test_terngrad_known_answer_deterministic_with_tail(oracle_cpu):
+    rc, out = oracle_cpu.terngrad_encode(_kat_x(22), 2, 0, 0)
+    assert rc == 0 and out.tobytes().hex() == "0202cccc4cbdcccc4c3dd87618b61d06"
+
+
+def test_terngrad_rejects_bad_bitwidth(oracle_cpu):
+    for b in (0, 3, 5, 6, 7, 9, 16):
+        rc, _ = oracle_cpu.terngrad_encode(_kat_x(8), b, 0, 0)
+        assert rc == -1
+
+
+def test_terngrad_independent_numpy_model_of_payload(oracle_cpu):
+    # An independent vectorised statement (numpy fp32 arithmetic, python-int LCG).
+    rng = np.random.default_rng(3)
+    n, seed = 4096 + 3, 2**40 + 77
+    x = rng.normal(0, 1e-2, n).astype(np.float32)
+    rc, out = oracle_cpu.terngrad_encode(x, 2, 1, seed)
+    mn, mx = x.min(), x.max()
+    gap = np.float32((mx - mn) / np.float32(3.0))
+    gi = np.float32(1.0 / (np.float64(gap) + 1e-8))
+    nb = n // 4
+    th = ((x[:nb * 4] - mn) * gi).astype(np.float32).reshape(nb, 4)
+    u = np.empty((nb, 4), np.float32)
+    for i in range(nb):
+        s = (seed + i) & M32
+        s = (A * s + C_) & M32
+        for j in range(4):
+            s = (A * s + C_) & M32
+            u[i, j] = np.float32(s / 4294967295.0)
+    t = (th + u).astype(np.float32).astype(np.int32).astype(np.uint8).astype(np.uint32)
+    byte = (t[:, 0] | (t[:, 1] << 2) | (t[:, 2] << 4) | (t[:, 3] << 6)) & 0xFF
+    assert np.array_equal(out[10:10 + nb], byte.astype(np.uint8))
+    tail = np.rint(((x[nb * 4:] - mn) * gi).astype(np.float32)).astype(np.uint32)
+    assert out[-1] == (tail[0] | (tail[1] << 2) | (tail[2] << 4))
+    assert out[1] == 1
+
+
+@pytest.mark.parametrize("b", [1, 2, 4, 8])
+def test_terngrad_decode_error_bounds_and_header(oracle_cpu, b):
+    rng = np.random.default_rng(b)
+    for n in (8 // b * 37 + 1, 4099, 65536):
+        x = rng.normal(0, 1e-2, n).astype(np.float32)
+        mn, mx = x.min(), x.max()
+        gap = (np.float64(mx) - np.float64(mn)) / ((1 << b) - 1)
+        for rnd, bound in ((0, 0.5), (1, 1.0)):
+            rc, out = oracle_cpu.terngrad_encode(x, b, rnd, 99)
+            assert rc == 0 and out.size == 10 + -(-n // (8 // b))
+            assert out[0] == b and out[1] == (-n) % (8 // b)
+            assert out[2:6].view(np.float32)[0] == mn and out[6:10].view(np.float32)[0] == mx
+            rc, dec = oracle_cpu.terngrad_decode(out, n)
+            assert rc == 0
+            assert np.max(np.abs(dec.astype(np.float64) - x)) <= bound * gap * (1 + 1e-4) + (1 << b) * 1e-8 + 1e-9  # gi = 1/(gap+1e-8)
+
+
+def test_terngrad_stochastic_rounding_is_unbiased(oracle_cpu):
+    x = np.full(200000, 0.3, np.float32)
+    x[0], x[1] = 0.0, 1.0
+    rc, out = oracle_cpu.terngrad_encode(x, 2, 1, 4242)
+    rc, dec = oracle_cpu.terngrad_decode(out, x.size)
+    assert abs(dec[2:].mean() - 0.3) < 2e-3            # E[decode] = x
+    assert {round(float(v), 3) for v in np.unique(dec[2:])} == {0.0, 0.333}  # the two neighbouring levels
+
+
+def test_terngrad_zero_extreme_takes_sign_of_first_zero(oracle_cpu):
+    x = np.array([0.5, -0.0, 0.0, 0.25, 0.0], np.float32)
+    rc, out = oracle_cpu.terngrad_encode(x, 2, 0, 0)
+    assert out[2:6].view(np.uint32)[0] == 0x80000000   # min is the first zero: -0.0
+    x = np.array([-0.5, 0.0, -0.0, -0.25], np.float32)
+    rc, out = oracle_cpu.terngrad_encode(x, 2, 0, 0)
+    assert out[6:10].view(np.uint32)[0] == 0x00000000  # max is the first zero: +0.0
+
+
+@pytest.mark.parametrize("policy", [0, 1])
+def test_terngrad_against_reference_bodies(oracle_cpu, oracle_ref, policy):
+    rng = np.random.default_rng(11)
+    for b in (1, 2, 4, 8):
+        for n in [1, 2, 3, 5, 8, 9, 1000, 1001, 1003, 1007, 262147]:
+            x = rng.normal(0, 1e-2, n).astype(np.float32)
+            if n > 100:
+                x[rng.integers(0, n, 3)] = 0.5
+            rc1, a = oracle_cpu.terngrad_encode(x, b, 0, 0)
+            rc2, r = oracle_ref.terngrad_encode_det(x.copy(), b, policy)
+            assert rc1 == rc2 == 0 and np.array_equal(a, r), (b, n)
+            dpb = 8 // b
+            nb = n // dpb
+            mn = a[2:6].view(np.float32)[0]
+            mx = a[6:10].view(np.float32)[0]
+            gap = np.float32((mx - mn) / np.float32((1 << b) - 1.0))
+            gi = np.float32(1.0 / (np.float64(gap) + 1e-8))
+            for seed in (0, 12345, 2**63 + 12345, 2**64 - 3):
+                rc1, a = oracle_cpu.terngrad_encode(x, b, 1, seed)
+                pay = oracle_ref.terngrad_payload_random(x.copy(), nb, b, mn, gi, seed, policy)
+                assert np.array_equal(a[10:10 + nb], pay), (b, n, seed)
+            for add in (0, 1):
+                base = rng.normal(0, 1, n).astype(np.float32)
+                r1, d1 = oracle_cpu.terngrad_decode(a, n, base.copy(), add)
+                r2, d2 = oracle_ref.terngrad_decode(a, n, base.copy(), add, policy)
+                assert r1 == r2 == 0 and np.array_equal(d1.view(np.uint32), d2.view(np.uint32))
+
+
+def test_terngrad_zero_sign_against_reference(oracle_cpu, oracle_ref):
+    for x in ([0.5, -0.0, 0.0, 0.25, 0.0], [-0.5, 0.0, -0.0, -0.25], [0.0, -0.0, 0.0, 0.0], [-0.0, 0.0, 0.0, 0.0]):
+        x = np.array(x, np.float32)
+        for pol in (0, 1):
+            _, a = oracle_cpu.terngrad_encode(x, 2, 0, 0)
+            _, r = oracle_ref.terngrad_encode_det(x.copy(), 2, pol)
+            assert np.array_equal(a, r), (x, pol)
+
+
+def test_lcg_against_reference_generators(oracle_cpu, oracle_ref):
+    for s in (0, 1, 12345, 0xFFFFFFFF, 0x80000000):
+        for k in (2, 3, 4, 5):
+            assert oracle_ref.lcg_kth(s, k) == oracle_cpu.lcg_kth(s, k)
+            assert oracle_ref.real01(s, k) == oracle_cpu.u01_from_u32(oracle_cpu.lcg_kth(s, k))

@@ -1,0 +1,99 @@
+"""ctypes binding of libhpx.so, the C-ABI kernel library (include/hpx.h).
+
+The library is the product: if it has not been built this module raises, it
+never falls back to another implementation.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libhpx.so")
+
+# every symbol include/hpx.h declares
+SYMBOLS = (
+    "hpx_version",
+    "hpx_last_error",
+    "hpx_release_workspaces",
+    "hpx_tbq_encode",
+    "hpx_tbq_decode",
+    "hpx_terngrad_encode",
+    "hpx_terngrad_decode",
+    "hpx_terngrad_decode_status",
+    "hpx_gd_encode",
+    "hpx_gd_decode",
+    "hpx_powersgd_encode1",
+    "hpx_powersgd_encode2",
+    "hpx_powersgd_decode",
+)
+
+_lib = None
+
+
+class HpxError(RuntimeError):
+    def __init__(self, code, text):
+        super().__init__(f"hpx call failed with code {code}: {text}")
+        self.code = code
+        self.text = text
+
+
+def load():
+    """Load libhpx.so (built by `make -C csrc`); raises if it is missing."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build the HIP kernel library first "
+            "(python -c 'import __graft_entry__ as g; g.build()' or make -C csrc)")
+    L = C.CDLL(LIB_PATH)
+    pp, p, i32 = C.c_void_p, C.c_void_p, C.c_int
+    L.hpx_version.restype = C.c_int
+    L.hpx_last_error.restype = C.c_char_p
+    L.hpx_release_workspaces.restype = C.c_int
+    L.hpx_tbq_encode.argtypes = [i32, pp, p, pp, pp, p, p]
+    L.hpx_tbq_decode.argtypes = [i32, pp, p, pp, p, p, p]
+    L.hpx_terngrad_encode.argtypes = [i32, pp, p, pp, p, p, p, p, p]
+    L.hpx_terngrad_decode.argtypes = [i32, pp, p, pp, p, p, p]
+    L.hpx_terngrad_decode_status.argtypes = [p]
+    L.hpx_gd_encode.argtypes = [i32, pp, p, pp, pp, p, p, p, p]
+    L.hpx_gd_decode.argtypes = [i32, pp, p, pp, p, p, p]
+    L.hpx_powersgd_encode1.argtypes = [i32, pp, p, pp, pp, pp, pp, p, p, p, p]
+    L.hpx_powersgd_encode2.argtypes = [i32, pp, pp, pp, p, p, p, p]
+    L.hpx_powersgd_decode.argtypes = [i32, pp, pp, pp, pp, pp, p, p, p, p, p]
+    for name in SYMBOLS:
+        getattr(L, name)  # AttributeError if the build lost an entry point
+    _lib = L
+    return L
+
+
+def last_error():
+    return load().hpx_last_error().decode()
+
+
+# ---- marshalling helpers: host arrays of pointers / scalars -----------------
+def ptr_array(ptrs):
+    return (C.c_void_p * len(ptrs))(*[C.c_void_p(int(x)) for x in ptrs])
+
+
+def i32_array(vals):
+    return (C.c_int32 * len(vals))(*[int(v) for v in vals])
+
+
+def i64_array(vals):
+    return (C.c_int64 * len(vals))(*[int(v) for v in vals])
+
+
+def u8_array(vals):
+    return (C.c_uint8 * len(vals))(*[int(v) & 0xFF for v in vals])
+
+
+def u64_array(vals):
+    return (C.c_uint64 * len(vals))(*[int(v) & 0xFFFFFFFFFFFFFFFF for v in vals])
+
+
+def f32_array(vals):
+    return (C.c_float * len(vals))(*[float(v) for v in vals])
+
+
+def f64_array(vals):
+    return (C.c_double * len(vals))(*[float(v) for v in vals])

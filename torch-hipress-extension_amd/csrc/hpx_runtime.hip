@@ -1,0 +1,89 @@
+// Library state that is not a kernel: error text, workspaces, seeds.
+#include <chrono>
+#include <cstdarg>
+#include <cstdio>
+#include <map>
+#include <memory>
+#include <utility>
+
+#include "hpx_common.h"
+
+namespace hpx {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+void clear_error() { g_err[0] = 0; }
+
+static std::mutex g_ws_mu;
+static std::map<std::pair<int, hipStream_t>, std::unique_ptr<Workspace>> g_ws;
+
+Workspace* workspace_record(hipStream_t stream) {
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) {
+    set_error("hipGetDevice failed");
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> g(g_ws_mu);
+  auto& slot = g_ws[{device, stream}];
+  if (!slot) {
+    slot.reset(new Workspace());
+    slot->device = device;
+    slot->stream = stream;
+  }
+  return slot.get();
+}
+
+int ensure_workspace(Workspace* ws, size_t dev_bytes) {
+  if (!ws->state) {
+    HPX_HIP(hipMalloc(reinterpret_cast<void**>(&ws->state), kStateWords * sizeof(uint32_t)));
+    HPX_HIP(hipMemset(ws->state, 0, kStateWords * sizeof(uint32_t)));
+    HPX_HIP(hipHostMalloc(reinterpret_cast<void**>(&ws->pinned), kPinnedBytes, hipHostMallocDefault));
+  }
+  if (dev_bytes > ws->dev_bytes) {
+    // Work already queued on this stream may still use the old block.
+    HPX_HIP(hipStreamSynchronize(ws->stream));
+    if (ws->dev) HPX_HIP(hipFree(ws->dev));
+    ws->dev = nullptr;
+    ws->dev_bytes = 0;
+    size_t want = dev_bytes + dev_bytes / 8 + (1 << 20);
+    want = (want + 255) & ~size_t(255);
+    HPX_HIP(hipMalloc(reinterpret_cast<void**>(&ws->dev), want));
+    ws->dev_bytes = want;
+  }
+  return HPX_OK;
+}
+
+uint64_t clock_seed() {
+  return static_cast<uint64_t>(
+      std::chrono::high_resolution_clock::now().time_since_epoch().count());
+}
+
+}  // namespace hpx
+
+HPX_API int hpx_version(void) { return 100; }
+
+HPX_API const char* hpx_last_error(void) { return hpx::g_err; }
+
+HPX_API int hpx_release_workspaces(void) {
+  std::lock_guard<std::mutex> g(hpx::g_ws_mu);
+  int rc = HPX_OK;
+  int cur = 0;
+  if (hipGetDevice(&cur) != hipSuccess) cur = -1;
+  for (auto& kv : hpx::g_ws) {
+    hpx::Workspace* ws = kv.second.get();
+    std::lock_guard<std::mutex> g2(ws->mu);
+    if (hipSetDevice(ws->device) != hipSuccess) { rc = HPX_ERR_HIP; continue; }
+    if (ws->dev && hipFree(ws->dev) != hipSuccess) rc = HPX_ERR_HIP;
+    if (ws->state && hipFree(ws->state) != hipSuccess) rc = HPX_ERR_HIP;
+    if (ws->pinned && hipHostFree(ws->pinned) != hipSuccess) rc = HPX_ERR_HIP;
+  }
+  hpx::g_ws.clear();
+  if (cur >= 0) (void)hipSetDevice(cur);
+  return rc;
+}

@@ -1,0 +1,535 @@
+// TernGrad path: b-bit uniform min/max quantiser (b in {1,2,4,8}) with optional
+// stochastic rounding, 10-byte header, codes packed LSB-first.
+//
+// Semantics follow terngrad_body.h:162-307 (encode) and :309-409 (decode).
+// Encode is two launches with no host round trip: a min/max reduction whose
+// last-arriving workgroup per tensor folds the partial results, derives the
+// scalars (gap, 1/gap) on the device and writes the header; then the
+// quantise-and-pack stream.  Decode parses the header on the device.
+//
+// Bit-exactness notes
+//   * (x - min) * gi + u is three separately rounded fp32 operations (the
+//     library is built with -ffp-contract=off).
+//   * gi = float(1.0 / (double(gap) + 1e-8)), terngrad_body.h:206.
+//   * The reference seeds its LCG per output byte with seed + byte index and
+//     draws once per slot after one discarded draw (terngrad_body.h:88-96), so
+//     slot j of byte i uses x = A_{j+2} * (seed + i) + C_{j+2}: a lane stepping
+//     through bytes at a fixed stride advances each draw by a constant.
+//   * u = float(double(x) / 4294967295.0) is evaluated as
+//     float(double(x) * 0x1.00000001p-32); the two agree for all 2^32 inputs
+//     (checked exhaustively on the CPU), and the product needs no division.
+//   * min and max are the FIRST smallest / largest element as
+//     thrust::minmax_element returns them, which only matters for the sign of
+//     a zero extreme; it is recovered from the first zero of the tensor.
+#include "hpx_common.h"
+
+namespace {
+using namespace hpx;
+
+constexpr int kThreads = 256;
+constexpr int kMaxSeg = 64;
+constexpr int kRedIters = 8;                                 // float4 loads per lane
+constexpr int kRedTile = kThreads * kRedIters * 4;           // 8192 elements
+constexpr int kQIters = 4;                                   // units per lane
+constexpr int kDecTile = kThreads * kQIters * 4;             // 4096 elements
+
+struct Partial {
+  float mn, mx;
+  uint32_t has_zero;
+};
+struct Scalars {
+  float mn, gi;
+};
+
+struct EncSeg {
+  const float* x;
+  uint8_t* out;
+  int32_t n;
+  int32_t out_size;
+  uint32_t seed;  // only the low 32 bits of seed + byte index reach the LCG
+  uint8_t bits;
+  uint8_t random;
+  uint16_t pad;
+};
+struct EncArgs {
+  int32_t nseg;
+  int32_t tile_start[kMaxSeg + 1];
+  EncSeg seg[kMaxSeg];
+  Partial* partials;    // one per reduction tile of this launch
+  Scalars* scalars;     // one per segment
+  uint32_t* counters;   // one per segment, zero on entry and on exit
+};
+struct DecSeg {
+  float* out;
+  const uint8_t* in;
+  int32_t out_size;
+  int32_t in_size;
+  int32_t add;
+  int32_t pad;
+};
+struct DecArgs {
+  int32_t nseg;
+  int32_t tile_start[kMaxSeg + 1];
+  DecSeg seg[kMaxSeg];
+  uint32_t* status;
+};
+static_assert(sizeof(EncArgs) <= 4096 && sizeof(DecArgs) <= 4096, "kernarg limit");
+
+__device__ __forceinline__ float wave_min(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) { float t = __shfl_xor(v, o, 64); v = t < v ? t : v; }
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) { float t = __shfl_xor(v, o, 64); v = t > v ? t : v; }
+  return v;
+}
+__device__ __forceinline__ uint32_t wave_min_u32(uint32_t v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) { uint32_t t = __shfl_xor(v, o, 64); v = t < v ? t : v; }
+  return v;
+}
+
+// Block-wide (min, max, min-u32) over 4 waves.  Result valid in every thread.
+__device__ __forceinline__ void block_reduce(float& mn, float& mx, uint32_t& z) {
+  __shared__ float s_mn[kThreads / kWave], s_mx[kThreads / kWave];
+  __shared__ uint32_t s_z[kThreads / kWave];
+  mn = wave_min(mn);
+  mx = wave_max(mx);
+  z = wave_min_u32(z);
+  const int w = threadIdx.x / kWave;
+  __syncthreads();  // protects reuse of the shared arrays between calls
+  if ((threadIdx.x & (kWave - 1)) == 0) { s_mn[w] = mn; s_mx[w] = mx; s_z[w] = z; }
+  __syncthreads();
+  mn = s_mn[0]; mx = s_mx[0]; z = s_z[0];
+#pragma unroll
+  for (int i = 1; i < kThreads / kWave; i++) {
+    mn = s_mn[i] < mn ? s_mn[i] : mn;
+    mx = s_mx[i] > mx ? s_mx[i] : mx;
+    z = s_z[i] < z ? s_z[i] : z;
+  }
+}
+
+__device__ __forceinline__ void acc3(float v, float& mn, float& mx, float& am) {
+  mn = v < mn ? v : mn;
+  mx = v > mx ? v : mx;
+  const float a = __builtin_fabsf(v);
+  am = a < am ? a : am;
+}
+
+__global__ __launch_bounds__(kThreads) void terngrad_minmax_kernel(const EncArgs a) {
+  const int tile = blockIdx.x;
+  const int s = find_segment<kMaxSeg>(a.tile_start, a.nseg, tile);
+  const float* __restrict__ xp = a.seg[s].x;
+  const uint32_t n = static_cast<uint32_t>(a.seg[s].n);
+  const int ntiles = a.tile_start[s + 1] - a.tile_start[s];
+  const uint32_t t = static_cast<uint32_t>(tile - a.tile_start[s]);
+  const uint32_t e0 = t * uint32_t(kRedTile);
+
+  float mn = __builtin_inff(), mx = -__builtin_inff(), am = __builtin_inff();
+  if (n - e0 >= uint32_t(kRedTile)) {
+    float4 v[kRedIters];
+#pragma unroll
+    for (int k = 0; k < kRedIters; k++) v[k] = ld4(xp + size_t(e0) + size_t(k * kThreads + threadIdx.x) * 4);
+#pragma unroll
+    for (int k = 0; k < kRedIters; k++) {
+      acc3(v[k].x, mn, mx, am); acc3(v[k].y, mn, mx, am);
+      acc3(v[k].z, mn, mx, am); acc3(v[k].w, mn, mx, am);
+    }
+  } else {
+    for (uint32_t e = e0 + threadIdx.x; e < n; e += kThreads) acc3(xp[e], mn, mx, am);
+  }
+  uint32_t z = (am == 0.0f) ? 0u : 1u;  // 0 when this tile holds a zero
+  block_reduce(mn, mx, z);
+
+  __shared__ uint32_t s_last;
+  if (threadIdx.x == 0) {
+    Partial p{mn, mx, z == 0u ? 1u : 0u};
+    a.partials[tile] = p;
+    __threadfence();
+    const uint32_t prev = atomicAdd(&a.counters[s], 1u);
+    s_last = (prev == uint32_t(ntiles - 1));
+  }
+  __syncthreads();
+  if (!s_last) return;
+  __threadfence();
+
+  // Last workgroup of this tensor: fold the partials.
+  const Partial* pp = a.partials + a.tile_start[s];
+  mn = __builtin_inff(); mx = -__builtin_inff();
+  uint32_t first_zero_tile = 0xFFFFFFFFu;
+  for (int i = threadIdx.x; i < ntiles; i += kThreads) {
+    const float pmn = __hip_atomic_load(&pp[i].mn, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const float pmx = __hip_atomic_load(&pp[i].mx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const uint32_t hz = __hip_atomic_load(&pp[i].has_zero, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    mn = pmn < mn ? pmn : mn;
+    mx = pmx > mx ? pmx : mx;
+    if (hz && uint32_t(i) < first_zero_tile) first_zero_tile = uint32_t(i);
+  }
+  block_reduce(mn, mx, first_zero_tile);
+  if ((mn == 0.0f || mx == 0.0f) && first_zero_tile != 0xFFFFFFFFu) {
+    // A zero extreme takes the sign of the first zero element of the tensor.
+    const uint32_t b0 = first_zero_tile * uint32_t(kRedTile);
+    const uint32_t b1 = (n - b0 < uint32_t(kRedTile)) ? n : b0 + uint32_t(kRedTile);
+    uint32_t first = 0xFFFFFFFFu;
+    for (uint32_t e = b0 + threadIdx.x; e < b1; e += kThreads)
+      if (xp[e] == 0.0f && e < first) first = e;
+    float d0 = 0.f, d1 = 0.f;
+    block_reduce(d0, d1, first);
+    if (first != 0xFFFFFFFFu) {
+      const float zv = xp[first];
+      if (mn == 0.0f) mn = zv;
+      if (mx == 0.0f) mx = zv;
+    }
+  }
+  if (threadIdx.x == 0) {
+    const uint32_t bits = a.seg[s].bits;
+    const float gap = (mx - mn) / (float(1 << bits) - 1.0f);
+    const float gi = static_cast<float>(1.0 / (static_cast<double>(gap) + 1e-8));
+    const uint32_t dpb = 8u / bits;
+    uint32_t tail = n % dpb;
+    tail = tail == 0 ? 0 : dpb - tail;
+    uint8_t* o = a.seg[s].out;
+    const uint32_t mb = __float_as_uint(mn), xb = __float_as_uint(mx);
+    o[0] = uint8_t(bits);
+    o[1] = uint8_t(tail);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      o[2 + i] = uint8_t(mb >> (8 * i));
+      o[6 + i] = uint8_t(xb >> (8 * i));
+    }
+    a.scalars[s] = Scalars{mn, gi};
+    a.counters[s] = 0;  // ready for the next call
+  }
+}
+
+// float(double(x) / 4294967295.0) without the division (see the file header).
+__device__ __forceinline__ float u01(uint32_t x) {
+  return static_cast<float>(static_cast<double>(x) * 0x1.00000001p-32);
+}
+
+template <int B, bool RANDOM>
+__device__ __forceinline__ uint32_t quant_one(float x, float mn, float gi, uint32_t draw) {
+  float th = (x - mn) * gi;
+  int32_t t;
+  if (RANDOM) {
+    th += u01(draw);
+    t = static_cast<int32_t>(th);  // truncation, terngrad_body.h:94
+  } else {
+    t = static_cast<int32_t>(__builtin_rintf(th));  // nearbyint, terngrad_body.h:53
+  }
+  return static_cast<uint32_t>(t) & 0xFFu;
+}
+
+// One tile of the quantise stream.  A unit is UNIT = max(4, 8/B) consecutive
+// elements owned by one lane per step; it packs into BPU = UNIT*B/8 bytes.
+template <int B, bool RANDOM>
+__device__ __forceinline__ void quant_tile(const EncSeg& sg, const Scalars sc, uint32_t tile_in_seg) {
+  constexpr int DPB = 8 / B;
+  constexpr int UNIT = DPB > 4 ? DPB : 4;
+  constexpr int BPU = UNIT / DPB;
+  constexpr uint32_t kStrideBytes = uint32_t(kThreads) * BPU;
+  const float* __restrict__ xp = sg.x;
+  uint8_t* __restrict__ pay = sg.out + 10;
+  const uint32_t n = static_cast<uint32_t>(sg.n);
+  const uint32_t nbytes = n / DPB;  // bytes the reference's transform covers
+  const float mn = sc.mn, gi = sc.gi;
+  const uint32_t u0 = tile_in_seg * uint32_t(kThreads * kQIters) + threadIdx.x;
+
+  // Draw for slot j of byte (u*BPU + jb): A_{j+2} * (seed + byte) + C_{j+2}.
+  uint32_t draw[UNIT];
+  if (RANDOM) {
+    const uint32_t x0 = sg.seed + u0 * BPU;
+#pragma unroll
+    for (int q = 0; q < UNIT; q++) {
+      const int jb = q / DPB, j = q % DPB;
+      draw[q] = lcg_mul(j + 2) * (x0 + jb) + lcg_add(j + 2);
+    }
+  }
+
+  const uint32_t units_total = (n + UNIT - 1) / UNIT;
+  const uint32_t tile_u0 = u0 - threadIdx.x;
+  if (uint64_t(tile_u0 + kThreads * kQIters) * UNIT <= n) {
+    float4 v[kQIters][UNIT / 4];
+#pragma unroll
+    for (int k = 0; k < kQIters; k++)
+#pragma unroll
+      for (int h = 0; h < UNIT / 4; h++)
+        v[k][h] = ld4(xp + size_t(u0 + k * kThreads) * UNIT + h * 4);
+#pragma unroll
+    for (int k = 0; k < kQIters; k++) {
+      const uint32_t u = u0 + k * kThreads;
+      uint32_t packed = 0;
+#pragma unroll
+      for (int q = 0; q < UNIT; q++) {
+        const float4 f = v[k][q / 4];
+        const float x = (q & 3) == 0 ? f.x : (q & 3) == 1 ? f.y : (q & 3) == 2 ? f.z : f.w;
+        const uint32_t t = quant_one<B, RANDOM>(x, mn, gi, RANDOM ? draw[q] : 0u);
+        // Within a byte codes are OR-ed without masking (terngrad_body.h:95):
+        // a code that reaches 1<<B spills into the next slot of the SAME byte.
+        const int jb = q / DPB, j = q % DPB;
+        packed |= ((t << (B * j)) & 0xFFu) << (8 * jb);
+        if (RANDOM) draw[q] += lcg_mul(j + 2) * kStrideBytes;
+      }
+#pragma unroll
+      for (int jb = 0; jb < BPU; jb++) pay[size_t(u) * BPU + jb] = uint8_t(packed >> (8 * jb));
+    }
+    return;
+  }
+  // Tile holding the end of the tensor.
+  for (int k = 0; k < kQIters; k++) {
+    const uint32_t u = u0 + k * kThreads;
+    if (u < units_total) {
+      for (int jb = 0; jb < BPU; jb++) {
+        const uint32_t byte = u * BPU + jb;
+        const size_t e = size_t(byte) * DPB;
+        if (byte < nbytes) {
+          uint32_t qv = 0;
+          for (int j = 0; j < DPB; j++) {
+            const uint32_t t = quant_one<B, RANDOM>(xp[e + j], mn, gi, RANDOM ? draw[jb * DPB + j] : 0u);
+            qv |= t << (B * j);
+          }
+          pay[byte] = uint8_t(qv);
+        } else if (byte == nbytes && (n % DPB)) {
+          // Partial last byte: always round-to-nearest, stored at the last byte
+          // of the caller's buffer (terngrad_body.h:288-296).
+          uint32_t qv = 0;
+          for (uint32_t j = 0; j < n % DPB; j++) qv |= quant_one<B, false>(xp[e + j], mn, gi, 0u) << (B * j);
+          sg.out[sg.out_size - 1] = uint8_t(qv);
+        }
+      }
+    }
+    if (RANDOM) {
+#pragma unroll
+      for (int q = 0; q < UNIT; q++) draw[q] += lcg_mul(q % DPB + 2) * kStrideBytes;
+    }
+  }
+}
+
+template <int B>
+__device__ __forceinline__ void quant_dispatch(const EncSeg& sg, const Scalars sc, uint32_t t) {
+  if (sg.random) quant_tile<B, true>(sg, sc, t); else quant_tile<B, false>(sg, sc, t);
+}
+
+// tile_start here counts quantise tiles (kThreads*kQIters units each).
+__global__ __launch_bounds__(kThreads) void terngrad_quant_kernel(const EncArgs a) {
+  const int tile = blockIdx.x;
+  const int s = find_segment<kMaxSeg>(a.tile_start, a.nseg, tile);
+  const Scalars sc = a.scalars[s];
+  const uint32_t t = static_cast<uint32_t>(tile - a.tile_start[s]);
+  switch (a.seg[s].bits) {
+    case 1: quant_dispatch<1>(a.seg[s], sc, t); break;
+    case 2: quant_dispatch<2>(a.seg[s], sc, t); break;
+    case 4: quant_dispatch<4>(a.seg[s], sc, t); break;
+    default: quant_dispatch<8>(a.seg[s], sc, t); break;
+  }
+}
+
+template <int B, bool ADD>
+__device__ __forceinline__ void decode_tile(const DecSeg& sg, float mn, float gap, uint32_t cnt, uint32_t tile_in_seg) {
+  constexpr int DPB = 8 / B;
+  constexpr uint32_t MASK = (1u << B) - 1u;
+  float* __restrict__ op = sg.out;
+  const uint8_t* __restrict__ pay = sg.in + 10;
+  const uint32_t g0 = tile_in_seg * uint32_t(kThreads * kQIters) + threadIdx.x;  // groups of 4 elements
+#pragma unroll
+  for (int k = 0; k < kQIters; k++) {
+    const uint32_t grp = g0 + k * kThreads;
+    const size_t e = size_t(grp) * 4;
+    if (e + 4 <= cnt) {
+      uint32_t bits;  // the 4*B bits holding this group's codes
+      if (B == 1) bits = (pay[e >> 3] >> (e & 4)) & 0xFu;
+      else if (B == 2) bits = pay[e >> 2];
+      else if (B == 4) bits = uint32_t(pay[e >> 1]) | (uint32_t(pay[(e >> 1) + 1]) << 8);
+      else bits = uint32_t(pay[e]) | (uint32_t(pay[e + 1]) << 8) | (uint32_t(pay[e + 2]) << 16) | (uint32_t(pay[e + 3]) << 24);
+      float4 v;
+      // static_cast<float>(qval*gap + min_f), terngrad_body.h:127
+      v.x = float(int((bits >> (0 * B)) & MASK)) * gap + mn;
+      v.y = float(int((bits >> (1 * B)) & MASK)) * gap + mn;
+      v.z = float(int((bits >> (2 * B)) & MASK)) * gap + mn;
+      v.w = float(int((bits >> (3 * B)) & MASK)) * gap + mn;
+      if (ADD) {
+        const float4 o = ld4(op + e);
+        v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w;
+      }
+      st4(op + e, v);
+    } else {
+      for (size_t i = e; i < cnt && i < e + 4; i++) {
+        const uint32_t q = (pay[i / DPB] >> ((i % DPB) * B)) & MASK;
+        const float v = float(int(q)) * gap + mn;
+        op[i] = ADD ? v + op[i] : v;
+      }
+    }
+  }
+}
+
+template <int B>
+__device__ __forceinline__ void decode_dispatch(const DecSeg& sg, float mn, float gap, uint32_t cnt, uint32_t t) {
+  if (sg.add) decode_tile<B, true>(sg, mn, gap, cnt, t); else decode_tile<B, false>(sg, mn, gap, cnt, t);
+}
+
+__global__ __launch_bounds__(kThreads) void terngrad_decode_kernel(const DecArgs a) {
+  const int tile = blockIdx.x;
+  const int s = find_segment<kMaxSeg>(a.tile_start, a.nseg, tile);
+  const uint8_t* __restrict__ in = a.seg[s].in;
+  const uint32_t bits = in[0];
+  const uint32_t tail = in[1];
+  uint32_t mb = 0, xb = 0;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    mb |= uint32_t(in[2 + i]) << (8 * i);
+    xb |= uint32_t(in[6 + i]) << (8 * i);
+  }
+  if (bits != 1 && bits != 2 && bits != 4 && bits != 8) {
+    if (threadIdx.x == 0 && tile == a.tile_start[s]) atomicOr(a.status, 1u);
+    return;
+  }
+  const float mn = __uint_as_float(mb), mx = __uint_as_float(xb);
+  const float gap = (mx - mn) / (float(1 << bits) - 1.0f);
+  // ((in_size-10) << lg2(dpb)) - tail, terngrad_body.h:373; clamped to the output.
+  int64_t c = int64_t(a.seg[s].in_size - 10) * int64_t(8 / bits) - int64_t(tail);
+  if (c > a.seg[s].out_size) c = a.seg[s].out_size;
+  if (c <= 0) return;
+  const uint32_t cnt = static_cast<uint32_t>(c);
+  const uint32_t t = static_cast<uint32_t>(tile - a.tile_start[s]);
+  switch (bits) {
+    case 1: decode_dispatch<1>(a.seg[s], mn, gap, cnt, t); break;
+    case 2: decode_dispatch<2>(a.seg[s], mn, gap, cnt, t); break;
+    case 4: decode_dispatch<4>(a.seg[s], mn, gap, cnt, t); break;
+    default: decode_dispatch<8>(a.seg[s], mn, gap, cnt, t); break;
+  }
+}
+
+inline int32_t ceil_div(int64_t a, int64_t b) { return static_cast<int32_t>((a + b - 1) / b); }
+
+}  // namespace
+
+HPX_API int hpx_terngrad_encode(int count, const float* const* ins, const int32_t* in_sizes,
+                                uint8_t* const* outs, const int32_t* out_sizes,
+                                const uint8_t* bitwidths, const int32_t* enable_randoms,
+                                const uint64_t* seeds, hpx_stream_t stream) {
+  hpx::clear_error();
+  HPX_ARG(count >= 0, "hpx_terngrad_encode: negative count");
+  if (count == 0) return HPX_OK;
+  HPX_ARG(ins && in_sizes && outs && out_sizes && bitwidths && enable_randoms,
+          "hpx_terngrad_encode: null argument array");
+  int64_t red_tiles_total = 0;
+  for (int i = 0; i < count; i++) {
+    const uint8_t b = bitwidths[i];
+    if (!(b == 1 || b == 2 || b == 4 || b == 8)) {
+      hpx::set_error("Invalid value of bitwidth, check value: bitwidth=%d", int(b));
+      return HPX_ERR_BODY;
+    }
+    HPX_ARG(in_sizes[i] > 0, "hpx_terngrad_encode: tensor %d has size %d (must be positive)", i, in_sizes[i]);
+    HPX_ARG(ins[i] && outs[i], "hpx_terngrad_encode: tensor %d has a null pointer", i);
+    const int64_t need = 10 + (int64_t(in_sizes[i]) + 8 / b - 1) / (8 / b);
+    HPX_ARG(out_sizes[i] >= need, "hpx_terngrad_encode: tensor %d needs %lld output bytes, got %d", i,
+            static_cast<long long>(need), out_sizes[i]);
+    red_tiles_total += ceil_div(in_sizes[i], kRedTile);
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  hpx::Workspace* ws = hpx::workspace_record(st);
+  if (!ws) return HPX_ERR_HIP;
+  std::lock_guard<std::mutex> lock(ws->mu);
+  const size_t scal_bytes = (size_t(count) * sizeof(Scalars) + 255) & ~size_t(255);
+  int rc = hpx::ensure_workspace(ws, scal_bytes + size_t(red_tiles_total) * sizeof(Partial));
+  if (rc != HPX_OK) return rc;
+  Scalars* scal_base = reinterpret_cast<Scalars*>(ws->dev);
+  Partial* part_base = reinterpret_cast<Partial*>(ws->dev + scal_bytes);
+
+  EncArgs a;
+  int i = 0;
+  size_t part_off = 0;
+  while (i < count) {
+    const int first = i;
+    a.nseg = 0;
+    a.tile_start[0] = 0;
+    a.partials = part_base + part_off;
+    a.scalars = scal_base + first;
+    a.counters = ws->state;  // launches are stream-ordered and each leaves them zero
+    int32_t qstart[kMaxSeg + 1];
+    qstart[0] = 0;
+    while (i < count && a.nseg < kMaxSeg) {
+      const int32_t n = in_sizes[i];
+      const int b = bitwidths[i];
+      const int unit = (8 / b) > 4 ? (8 / b) : 4;
+      const int32_t rt = ceil_div(n, kRedTile);
+      const int32_t qt = ceil_div(ceil_div(n, unit), kThreads * kQIters);
+      if (int64_t(a.tile_start[a.nseg]) + rt > INT32_MAX || int64_t(qstart[a.nseg]) + qt > INT32_MAX) break;
+      const uint64_t seed = seeds ? seeds[i] : hpx::clock_seed();
+      a.seg[a.nseg] = EncSeg{ins[i], outs[i], n, out_sizes[i], static_cast<uint32_t>(seed),
+                             static_cast<uint8_t>(b), static_cast<uint8_t>(enable_randoms[i] != 0), 0};
+      a.tile_start[a.nseg + 1] = a.tile_start[a.nseg] + rt;
+      qstart[a.nseg + 1] = qstart[a.nseg] + qt;
+      a.nseg++;
+      i++;
+    }
+    hipLaunchKernelGGL(terngrad_minmax_kernel, dim3(a.tile_start[a.nseg]), dim3(kThreads), 0, st, a);
+    HPX_HIP(hipGetLastError());
+    part_off += size_t(a.tile_start[a.nseg]);
+    for (int k = 0; k <= a.nseg; k++) a.tile_start[k] = qstart[k];
+    hipLaunchKernelGGL(terngrad_quant_kernel, dim3(a.tile_start[a.nseg]), dim3(kThreads), 0, st, a);
+    HPX_HIP(hipGetLastError());
+  }
+  return HPX_OK;
+}
+
+HPX_API int hpx_terngrad_decode(int count, float* const* outs, const int32_t* out_sizes,
+                                const uint8_t* const* ins, const int32_t* in_sizes,
+                                const int32_t* is_add_tos, hpx_stream_t stream) {
+  hpx::clear_error();
+  HPX_ARG(count >= 0, "hpx_terngrad_decode: negative count");
+  if (count == 0) return HPX_OK;
+  HPX_ARG(outs && out_sizes && ins && in_sizes && is_add_tos, "hpx_terngrad_decode: null argument array");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  hpx::Workspace* ws = hpx::workspace_record(st);
+  if (!ws) return HPX_ERR_HIP;
+  std::lock_guard<std::mutex> lock(ws->mu);
+  int rc = hpx::ensure_workspace(ws, 0);
+  if (rc != HPX_OK) return rc;
+  DecArgs a;
+  a.status = ws->state + hpx::kStatusWord;
+  int i = 0;
+  while (i < count) {
+    a.nseg = 0;
+    a.tile_start[0] = 0;
+    while (i < count && a.nseg < kMaxSeg) {
+      HPX_ARG(out_sizes[i] >= 0 && in_sizes[i] >= 10, "hpx_terngrad_decode: message %d: out_size %d, in_size %d", i,
+              out_sizes[i], in_sizes[i]);
+      if (out_sizes[i] > 0) {
+        HPX_ARG(outs[i] && ins[i], "hpx_terngrad_decode: message %d has a null pointer", i);
+        const int32_t t = ceil_div(out_sizes[i], kDecTile);
+        if (int64_t(a.tile_start[a.nseg]) + t > INT32_MAX) break;
+        a.seg[a.nseg] = DecSeg{outs[i], ins[i], out_sizes[i], in_sizes[i], is_add_tos[i] != 0, 0};
+        a.tile_start[a.nseg + 1] = a.tile_start[a.nseg] + t;
+        a.nseg++;
+      }
+      i++;
+    }
+    if (a.nseg == 0) continue;
+    hipLaunchKernelGGL(terngrad_decode_kernel, dim3(a.tile_start[a.nseg]), dim3(kThreads), 0, st, a);
+    HPX_HIP(hipGetLastError());
+  }
+  return HPX_OK;
+}
+
+HPX_API int hpx_terngrad_decode_status(hpx_stream_t stream) {
+  hpx::clear_error();
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  hpx::Workspace* ws = hpx::workspace_record(st);
+  if (!ws) return HPX_ERR_HIP;
+  std::lock_guard<std::mutex> lock(ws->mu);
+  int rc = hpx::ensure_workspace(ws, 0);
+  if (rc != HPX_OK) return rc;
+  uint32_t* flag = ws->state + hpx::kStatusWord;
+  uint32_t* host = reinterpret_cast<uint32_t*>(ws->pinned);
+  HPX_HIP(hipMemcpyAsync(host, flag, sizeof(uint32_t), hipMemcpyDeviceToHost, st));
+  HPX_HIP(hipStreamSynchronize(st));
+  if (*host & 1u) {
+    HPX_HIP(hipMemsetAsync(flag, 0, sizeof(uint32_t), st));
+    hpx::set_error("bitwidth is invalid");
+    return HPX_ERR_BODY;
+  }
+  return HPX_OK;
+}
