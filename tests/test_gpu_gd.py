@@ -1,0 +1,210 @@
+"""GPU parity: GradDrop ("DGC") encode/decode through the C ABI vs the CPU oracle.
+
+Bit-exact: message bytes (header, index block, value block), residual after
+encode, decoded tensors.  In the cut branch the order among equal |r| is
+unspecified in the reference; the oracle and the kernels both keep ascending
+index order among ties.
+"""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import assert_bits_equal, dev, host, stream_ptr
+
+pytestmark = pytest.mark.gpu
+
+
+class Gd:
+    def __init__(self, capi):
+        self.c = capi
+        self.L = capi.load()
+
+    def encode(self, gs, rs, outs, srs, drs, seeds, expect_rc=0):
+        c = self.c
+        rc = self.L.hpx_gd_encode(len(gs), c.ptr_array([g.data_ptr() for g in gs]), c.i32_array([g.numel() for g in gs]),
+                                  c.ptr_array([r.data_ptr() for r in rs]), c.ptr_array([o.data_ptr() for o in outs]),
+                                  c.f64_array(srs), c.f64_array(drs), c.u64_array(seeds) if seeds is not None else None,
+                                  stream_ptr())
+        assert rc == expect_rc, (rc, c.last_error())
+
+    def decode(self, msgs, in_sizes, outs, adds, expect_rc=0):
+        c = self.c
+        rc = self.L.hpx_gd_decode(len(msgs), c.ptr_array([m.data_ptr() for m in msgs]), c.i32_array(in_sizes),
+                                  c.ptr_array([o.data_ptr() for o in outs]), c.i32_array([o.numel() for o in outs]),
+                                  c.i32_array(adds), stream_ptr())
+        assert rc == expect_rc, (rc, c.last_error())
+
+
+@pytest.fixture(scope="module")
+def gd(capi):
+    assert torch.cuda.is_available()
+    return Gd(capi)
+
+
+_BRANCHES = set()
+
+
+def _out_bytes(n, dr):
+    return 4 + 8 * int(np.ceil(n * (1 - dr)))
+
+
+def _check_encode(gd, oracle_cpu, g, r0, sr, dr, seed, guard=64):
+    n = g.size
+    dg, dr_ = dev(g), dev(r0)
+    size = _out_bytes(n, dr)
+    out = torch.full((size + guard,), 0xEE, dtype=torch.uint8, device="cuda")
+    gd.encode([dg], [dr_], [out], [sr], [dr], [seed])
+    torch.cuda.synchronize()
+    r_ref = r0.copy()
+    msg, info = oracle_cpu.gd_encode(g, r_ref, sr, dr, seed)
+    got = host(out)
+    m = int(got[:4].view(np.int32)[0])
+    assert m == msg.size, (m, msg.size, info)
+    # In the cut branch equal |r| keep ascending index order on both sides (the
+    # reference leaves that order unspecified), so ties need no special care here.
+    assert_bits_equal(got[:m], msg, f"message n={n} seed={seed} info={info}")
+    assert np.all(got[size:] == 0xEE), "wrote past 4 + 8*expected bytes"
+    assert_bits_equal(host(dr_), r_ref, "residual")
+    assert_bits_equal(host(dg), g, "gradient untouched")
+    return out, msg, info
+
+
+@pytest.mark.parametrize("n,sr,dr", [(1000, 0.05, 0.99), (4095, 0.05, 0.99), (4096, 0.01, 0.999), (4097, 0.1, 0.9),
+                                     (10007, 0.1, 0.9), (65536, 0.5, 0.5), (100003, 0.01, 0.999), (300007, 0.02, 0.97),
+                                     (1_000_003, 0.01, 0.999), (5_000_011, 0.01, 0.999)])
+def test_encode_decode_sizes(gd, oracle_cpu, n, sr, dr):
+    rng = np.random.default_rng(n)
+    branches = set()
+    for seed in (0, 1, 12345, 2**40 + 5, 2**64 - 2, 77):
+        g = rng.laplace(0, 1e-3, n).astype(np.float32)
+        r0 = rng.normal(0, 1e-4, n).astype(np.float32)
+        out, msg, info = _check_encode(gd, oracle_cpu, g, r0, sr, dr, seed)
+        branches.add(info["candidates"] > info["kept"])
+        for add in (0, 1):
+            base = rng.normal(0, 1, n).astype(np.float32)
+            dout = dev(base)
+            gd.decode([out], [msg.size], [dout], [add])
+            torch.cuda.synchronize()
+            ref = base.copy()
+            assert oracle_cpu.gd_decode(msg, ref, add) == 0
+            assert_bits_equal(host(dout), ref, f"decode add={add}")
+    _BRANCHES.update(branches)
+
+
+def test_both_branches_were_exercised():
+    # runs after the size sweep above: the sweep met tensors that were cut and tensors that were not
+    assert _BRANCHES == {True, False}, _BRANCHES
+
+
+def test_cut_branch_small_sample(gd, oracle_cpu):
+    # threshold = 2nd largest of 1000 samples: about twice as many candidates as `expected`
+    rng = np.random.default_rng(3)
+    n = 200_000
+    g = rng.laplace(0, 1e-3, n).astype(np.float32)
+    r0 = rng.normal(0, 1e-4, n).astype(np.float32)
+    cuts = 0
+    for seed in range(8):
+        out, msg, info = _check_encode(gd, oracle_cpu, g, r0, 0.005, 0.999, seed)
+        cuts += info["candidates"] > info["kept"]
+    assert cuts >= 2
+
+
+def test_far_more_candidates_than_reserved(gd, oracle_cpu):
+    # The sampled positions (a known function of the seed) hold tiny values, everything else is
+    # large: the threshold comes out tiny and nearly the whole tensor is a candidate.
+    rng = np.random.default_rng(4)
+    n, sr, dr, seed = 400_000, 0.01, 0.999, 9
+    g = rng.laplace(0, 1e-3, n).astype(np.float32)
+    g[np.abs(g) < 1e-5] = 1e-5
+    sampled = np.array([oracle_cpu.gd_sample_index(seed, x, n) for x in range(4000)])
+    g[sampled] = (1e-7 * (1 + np.arange(4000) / 4000.0)).astype(np.float32)
+    out, msg, info = _check_encode(gd, oracle_cpu, g, np.zeros(n, np.float32), sr, dr, seed)
+    assert info["threshold"] < 3e-7 and info["candidates"] > 390_000 and info["kept"] == oracle_cpu.gd_sizes(n, sr, dr)[1]
+
+
+def test_nothing_selected(gd, oracle_cpu):
+    n = 50_000
+    _check_encode(gd, oracle_cpu, np.zeros(n, np.float32), np.zeros(n, np.float32), 0.05, 0.99, 0)
+
+
+def test_several_tensors_and_messages(gd, oracle_cpu):
+    rng = np.random.default_rng(6)
+    sizes = [1000, 70001, 4096, 250_003]
+    gs = [rng.laplace(0, 1e-3, n).astype(np.float32) for n in sizes]
+    rs = [rng.normal(0, 1e-4, n).astype(np.float32) for n in sizes]
+    dgs, drs_ = [dev(g) for g in gs], [dev(r) for r in rs]
+    outs = [torch.zeros(_out_bytes(n, 0.99), dtype=torch.uint8, device="cuda") for n in sizes]
+    seeds = [3, 4, 5, 6]
+    gd.encode(dgs, drs_, outs, [0.05] * 4, [0.99] * 4, seeds)
+    torch.cuda.synchronize()
+    msgs = []
+    for i, n in enumerate(sizes):
+        r_ref = rs[i].copy()
+        msg, _ = oracle_cpu.gd_encode(gs[i], r_ref, 0.05, 0.99, seeds[i])
+        assert_bits_equal(host(outs[i])[: msg.size], msg, f"message[{i}]")
+        assert_bits_equal(host(drs_[i]), r_ref, f"residual[{i}]")
+        msgs.append(msg)
+    # several messages accumulate into ONE tensor sequentially (the root's gather-decode, hp_cuda.cpp:241-259)
+    n = 70001
+    m2 = []
+    for seed in (11, 12, 13):
+        r = np.zeros(n, np.float32)
+        m, _ = oracle_cpu.gd_encode(rng.laplace(0, 1e-3, n).astype(np.float32), r, 0.05, 0.99, seed)
+        m2.append(m)
+    base = rng.normal(0, 1, n).astype(np.float32)
+    dout = dev(base)
+    dm = [dev(m) for m in m2]
+    gd.decode(dm, [m.size for m in m2], [dout] * 3, [1, 1, 1])
+    ref = base.copy()
+    for m in m2:
+        oracle_cpu.gd_decode(m, ref, 1)
+    assert_bits_equal(host(dout), ref, "accumulated decode")
+
+
+def test_decode_errors(gd, oracle_cpu):
+    n = 5000
+    rng = np.random.default_rng(1)
+    r = np.zeros(n, np.float32)
+    msg, _ = oracle_cpu.gd_encode(rng.laplace(0, 1e-3, n).astype(np.float32), r, 0.05, 0.99, 3)
+    good = dev(np.array([4, 0, 0, 0], np.uint8))
+    o1 = torch.ones(n, device="cuda"); o2 = torch.ones(n, device="cuda")
+    # a short message fails the whole call before any output is touched (gd_body.h:317-325)
+    gd.decode([good, dev(msg)], [4, msg.size - 1], [o1, o2], [0, 0], expect_rc=-1)
+    torch.cuda.synchronize()
+    assert bool((o1 == 1).all()) and bool((o2 == 1).all())
+    gd.decode([good], [4], [o1], [0])      # k == 0: write mode still zero-fills
+    assert bool((o1 == 0).all())
+
+
+def test_encode_argument_errors(gd):
+    g = torch.zeros(100, device="cuda"); r = torch.zeros(100, device="cuda")
+    out = torch.zeros(64, dtype=torch.uint8, device="cuda")
+    gd.encode([g], [r], [out], [0.05], [0.0], [0], expect_rc=-3)   # threshold index == sample_cnt (out of range in the reference)
+    gd.encode([g], [r], [out[1:]], [0.05], [0.9], [0], expect_rc=-3)  # misaligned output
+
+
+def test_full_size_config3(gd):
+    # 138,357,544 elements (VGG-16), Laplace(0,1e-3) + residual N(0,1e-4), sample 1 %, keep 0.1 %, seed 0
+    from oracle import cpu
+    n, sr, dr, seed = 138_357_544, 0.01, 0.999, 0
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    u = torch.rand(n, device="cuda", generator=gen) - 0.5
+    g = (-1e-3 * torch.sign(u) * torch.log1p(-2 * u.abs())).float()
+    del u
+    r = torch.randn(n, device="cuda", generator=gen) * 1e-4
+    gh, rh = host(g), host(r)
+    out = torch.zeros(_out_bytes(n, dr), dtype=torch.uint8, device="cuda")
+    gd.encode([g], [r], [out], [sr], [dr], [seed])
+    torch.cuda.synchronize()
+    msg, info = cpu.gd_encode(gh, rh, sr, dr, seed)
+    got = host(out)
+    assert int(got[:4].view(np.int32)[0]) == msg.size, info
+    assert_bits_equal(got[: msg.size], msg, f"full-size message {info}")
+    assert_bits_equal(host(r), rh, "full-size residual")
+    # size-independent property: R_after + scatter(idx, val) == R_before + G, via decode(add) on the device
+    dec = r.clone()
+    gd.decode([out], [msg.size], [dec], [1])
+    idx, val = cpu.gd_split(msg)
+    decoded = host(dec)
+    rh2 = rh.copy(); rh2[idx] += val
+    assert_bits_equal(decoded, rh2, "decode(add) restores the accumulated tensor")

@@ -148,3 +148,12 @@ def test_full_size_bucket_properties(tbq):
         codes = packed[i]
         assert int(((codes >> 0) & 3 == 3).sum() + ((codes >> 2) & 3 == 3).sum()) == 0
     assert [float(g.double().sum()) for g in gs[:5]] == g_sum  # gradients untouched
+    # bit-exact against the oracle on the largest and a few other tensors of the bucket
+    from oracle import cpu
+    for i in (0, 7, int(np.argmax(sizes)), len(gs) - 1):
+        gh = host(gs[i])
+        rh = np.zeros_like(gh)
+        p_ref = cpu.tbq_encode(gh, rh, thr)
+        assert_bits_equal(host(packed[i]), p_ref, f"bucket packed[{i}]")
+        assert_bits_equal(host(rs[i]), rh, f"bucket residual[{i}]")
+        assert_bits_equal(host(outs[i]), cpu.tbq_decode(p_ref, gh.size, thr), f"bucket decoded[{i}]")

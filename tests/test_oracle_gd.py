@@ -1,0 +1,148 @@
+"""Pins the plain-C GradDrop ("DGC") oracle (CPU only): brute force on small
+inputs with numpy's full sort, the closed-form sample index stream, the
+invariants gd_body.h implies, and the reference's own functors where built."""
+import numpy as np
+import pytest
+
+A2, C2 = 3265436265, 3554416254   # two LCG steps: x2 = A2*s + C2 (mod 2^32)
+
+
+def _brute_force(g, r0, sample_rate, drop_ratio, seed):
+    """Independent numpy statement of gd_body.h:102-232 (sorts instead of selects)."""
+    n = g.size
+    s = 1 - drop_ratio
+    sample_cnt = int(np.ceil(n * sample_rate))
+    expected = int(np.ceil(n * s))
+    r = (g + r0).astype(np.float32)
+    x = (seed + np.arange(sample_cnt, dtype=np.uint64)) & np.uint64(0xFFFFFFFF)
+    idx = ((x * np.uint64(A2) + np.uint64(C2)) & np.uint64(0xFFFFFFFF)) % np.uint64(n)
+    sample = np.sort(np.abs(r[idx.astype(np.int64)]))[::-1]
+    thr = sample[int(sample_cnt * s)]
+    cand = np.flatnonzero((r > thr) | (r < -thr))
+    total = cand.size
+    if total > expected:
+        order = np.lexsort((cand, -np.abs(r[cand]).astype(np.float64)))  # |r| descending, ties by index
+        cand = cand[order][:expected]
+    vals = r[cand].copy()
+    r[cand] = 0
+    return cand.astype(np.int32), vals, r, thr, total
+
+
+@pytest.mark.parametrize("n,sr,dr", [(1000, 0.05, 0.99), (4096, 0.01, 0.999), (10007, 0.1, 0.9), (100003, 0.01, 0.999),
+                                     (65536, 0.5, 0.5), (300007, 0.02, 0.97), (5000, 1.0, 0.999)])
+def test_gd_encode_matches_brute_force(oracle_cpu, n, sr, dr):
+    rng = np.random.default_rng(n)
+    for seed in (0, 1, 12345, 2**40 + 5, 2**64 - 2):
+        g = rng.laplace(0, 1e-3, n).astype(np.float32)
+        r0 = rng.normal(0, 1e-4, n).astype(np.float32)
+        g_copy, r = g.copy(), r0.copy()
+        msg, info = oracle_cpu.gd_encode(g, r, sr, dr, seed)
+        idx, val, r_ref, thr, total = _brute_force(g, r0, sr, dr, seed)
+        assert np.array_equal(g, g_copy)
+        assert info["candidates"] == total and info["threshold"] == thr
+        oi, ov = oracle_cpu.gd_split(msg)
+        assert msg[:4].view(np.int32)[0] == 4 + 8 * idx.size == msg.size
+        assert np.array_equal(oi, idx) and np.array_equal(ov.view(np.uint32), val.view(np.uint32))
+        assert np.array_equal(r.view(np.uint32), r_ref.view(np.uint32))
+
+
+def test_gd_sizes_and_index_stream(oracle_cpu):
+    # config 3: N = 138,357,544, sample 1 %, drop 99.9 %
+    assert oracle_cpu.gd_sizes(138_357_544, 0.01, 0.999) == (1_383_576, 138_358, 1383)
+    for seed in (0, 7, 2**32 - 1, 2**50):
+        for x in (0, 1, 99, 1_000_000):
+            for n in (1000, 138_357_544):
+                s = (seed + x) & 0xFFFFFFFF
+                assert oracle_cpu.gd_sample_index(seed, x, n) == ((A2 * s + C2) & 0xFFFFFFFF) % n
+
+
+def test_gd_invariants(oracle_cpu):
+    rng = np.random.default_rng(5)
+    n, sr, dr = 200003, 0.02, 0.995
+    g = rng.laplace(0, 1e-3, n).astype(np.float32)
+    r0 = rng.normal(0, 1e-4, n).astype(np.float32)
+    for seed in range(6):
+        r = r0.copy()
+        msg, info = oracle_cpu.gd_encode(g, r, sr, dr, seed)
+        idx, val = oracle_cpu.gd_split(msg)
+        acc = (g + r0).astype(np.float32)
+        _, expected, _ = oracle_cpu.gd_sizes(n, sr, dr)
+        assert idx.size == min(info["candidates"], expected) == info["kept"]
+        assert np.unique(idx).size == idx.size                      # indices unique
+        assert np.all(np.abs(val) > info["threshold"])              # every selected |v| > thr
+        rebuilt = r.copy(); rebuilt[idx] += val                     # R_after + scatter == R_before + G, exactly
+        assert np.array_equal(rebuilt.view(np.uint32), acc.view(np.uint32))
+        assert np.all(r[idx] == 0)
+        if info["candidates"] > expected:                           # cut: kept dominate the rejected candidates
+            rejected = np.setdiff1d(np.flatnonzero(np.abs(acc) > info["threshold"]), idx)
+            assert np.abs(val).min() >= np.abs(acc[rejected]).max()
+            assert np.all(np.diff(np.abs(val)) <= 0)                # descending |v|
+        else:
+            assert np.all(np.diff(idx) > 0)                         # ascending index
+        # decode (write) of the message is the masked accumulated tensor
+        out = np.full(n, 3.0, np.float32)
+        assert oracle_cpu.gd_decode(msg, out, 0) == 0
+        mask = np.zeros(n, bool); mask[idx] = True
+        assert np.array_equal(out, np.where(mask, acc, 0).astype(np.float32))
+        base = rng.normal(0, 1, n).astype(np.float32)
+        out = base.copy()
+        assert oracle_cpu.gd_decode(msg, out, 1) == 0
+        exp = base.copy(); exp[idx] += val
+        assert np.array_equal(out, exp)
+
+
+def test_gd_decode_short_message_and_empty(oracle_cpu):
+    n = 5000
+    rng = np.random.default_rng(1)
+    g = rng.laplace(0, 1e-3, n).astype(np.float32); r = np.zeros(n, np.float32)
+    msg, _ = oracle_cpu.gd_encode(g, r, 0.05, 0.99, 3)
+    out = np.ones(n, np.float32)
+    assert oracle_cpu.gd_decode(msg, out, 0, in_size=msg.size - 1) == -1     # gd_body.h:317-325
+    assert np.all(out == 1)
+    empty = np.array([4, 0, 0, 0], np.uint8)                                   # k == 0: header only
+    assert oracle_cpu.gd_decode(empty, out, 0) == 0 and np.all(out == 0)
+
+
+def test_gd_all_zero_gradient_selects_nothing(oracle_cpu):
+    n = 4096
+    g = np.zeros(n, np.float32); r = np.zeros(n, np.float32)
+    msg, info = oracle_cpu.gd_encode(g, r, 0.05, 0.99, 0)
+    assert msg.size == 4 and info["kept"] == 0
+
+
+@pytest.mark.parametrize("policy", [0, 1])
+def test_gd_against_reference_functors(oracle_cpu, oracle_ref, policy):
+    rng = np.random.default_rng(1)
+    cut = kept = 0
+    for n in [1000, 4096, 10007, 100003, 1000003]:
+        for sr, dr in [(0.01, 0.999), (0.05, 0.99), (0.1, 0.9), (0.5, 0.5)]:
+            for seed in (0, 1, 7, 2**40 + 5, 2**64 - 2):
+                g = rng.laplace(0, 1e-3, n).astype(np.float32)
+                r0 = rng.normal(0, 1e-4, n).astype(np.float32)
+                ra, rb = r0.copy(), r0.copy()
+                ma, ia = oracle_cpu.gd_encode(g, ra, sr, dr, seed)
+                mb, ib = oracle_ref.gd_encode_seeded(g.copy(), rb, sr, dr, seed, policy)
+                assert ia == ib, (n, sr, dr, seed)
+                assert np.array_equal(ra.view(np.uint32), rb.view(np.uint32))
+                # continuous random data: no |r| ties, so even the cut branch agrees byte for byte
+                assert np.array_equal(ma, mb)
+                if ia["candidates"] > ia["kept"]:
+                    cut += 1
+                else:
+                    kept += 1
+    assert cut > 5 and kept > 5      # both branches were exercised
+    s = oracle_ref.gd_sample(np.arange(1000, dtype=np.float32), 50, 12345)
+    assert s.astype(np.int64).tolist() == [oracle_cpu.gd_sample_index(12345, x, 1000) for x in range(50)]
+
+
+def test_gd_decode_against_reference(oracle_cpu, oracle_ref):
+    rng = np.random.default_rng(3)
+    for n in (1000, 100003):
+        g = rng.laplace(0, 1e-3, n).astype(np.float32); r = np.zeros(n, np.float32)
+        m, _ = oracle_cpu.gd_encode(g, r, 0.05, 0.99, 3)
+        for add in (0, 1):
+            base = rng.normal(0, 1, n).astype(np.float32)
+            a, b = base.copy(), base.copy()
+            assert oracle_cpu.gd_decode(m, a, add) == 0 and oracle_ref.gd_decode(m, b, add) == 0
+            assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+        assert oracle_ref.gd_decode(m, b, 0, in_size=m.size - 1) == -1

@@ -2,8 +2,8 @@
 // stochastic rounding, 10-byte header, codes packed LSB-first.
 //
 // Semantics follow terngrad_body.h:162-307 (encode) and :309-409 (decode).
-// Encode is two launches with no host round trip: a min/max reduction whose
-// last-arriving workgroup per tensor folds the partial results, derives the
+// Encode is three launches with no host round trip: a min/max reduction to
+// per-tile partials; one workgroup per tensor that folds them, derives the
 // scalars (gap, 1/gap) on the device and writes the header; then the
 // quantise-and-pack stream.  Decode parses the header on the device.
 //
@@ -57,7 +57,6 @@ struct EncArgs {
   EncSeg seg[kMaxSeg];
   Partial* partials;    // one per reduction tile of this launch
   Scalars* scalars;     // one per segment
-  uint32_t* counters;   // one per segment, zero on entry and on exit
 };
 struct DecSeg {
   float* out;
@@ -123,7 +122,6 @@ __global__ __launch_bounds__(kThreads) void terngrad_minmax_kernel(const EncArgs
   const int s = find_segment<kMaxSeg>(a.tile_start, a.nseg, tile);
   const float* __restrict__ xp = a.seg[s].x;
   const uint32_t n = static_cast<uint32_t>(a.seg[s].n);
-  const int ntiles = a.tile_start[s + 1] - a.tile_start[s];
   const uint32_t t = static_cast<uint32_t>(tile - a.tile_start[s]);
   const uint32_t e0 = t * uint32_t(kRedTile);
 
@@ -142,27 +140,25 @@ __global__ __launch_bounds__(kThreads) void terngrad_minmax_kernel(const EncArgs
   }
   uint32_t z = (am == 0.0f) ? 0u : 1u;  // 0 when this tile holds a zero
   block_reduce(mn, mx, z);
+  if (threadIdx.x == 0) a.partials[tile] = Partial{mn, mx, z == 0u ? 1u : 0u};
+}
 
-  __shared__ uint32_t s_last;
-  if (threadIdx.x == 0) {
-    Partial p{mn, mx, z == 0u ? 1u : 0u};
-    a.partials[tile] = p;
-    __threadfence();
-    const uint32_t prev = atomicAdd(&a.counters[s], 1u);
-    s_last = (prev == uint32_t(ntiles - 1));
-  }
-  __syncthreads();
-  if (!s_last) return;
-  __threadfence();
-
-  // Last workgroup of this tensor: fold the partials.
+// One workgroup per tensor folds that tensor's partials, derives the scalars
+// and writes the header.  (A last-arriving-workgroup scheme inside the
+// reduction kernel would save this launch, but thousands of workgroups bumping
+// one arrival counter serialise at ~40 ns each across the XCDs.)
+__global__ __launch_bounds__(kThreads) void terngrad_finalize_kernel(const EncArgs a) {
+  const int s = blockIdx.x;
+  const float* __restrict__ xp = a.seg[s].x;
+  const uint32_t n = static_cast<uint32_t>(a.seg[s].n);
+  const int ntiles = a.tile_start[s + 1] - a.tile_start[s];
+  float mn, mx;
   const Partial* pp = a.partials + a.tile_start[s];
   mn = __builtin_inff(); mx = -__builtin_inff();
   uint32_t first_zero_tile = 0xFFFFFFFFu;
   for (int i = threadIdx.x; i < ntiles; i += kThreads) {
-    const float pmn = __hip_atomic_load(&pp[i].mn, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const float pmx = __hip_atomic_load(&pp[i].mx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const uint32_t hz = __hip_atomic_load(&pp[i].has_zero, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const float pmn = pp[i].mn, pmx = pp[i].mx;
+    const uint32_t hz = pp[i].has_zero;
     mn = pmn < mn ? pmn : mn;
     mx = pmx > mx ? pmx : mx;
     if (hz && uint32_t(i) < first_zero_tile) first_zero_tile = uint32_t(i);
@@ -200,7 +196,6 @@ __global__ __launch_bounds__(kThreads) void terngrad_minmax_kernel(const EncArgs
       o[6 + i] = uint8_t(xb >> (8 * i));
     }
     a.scalars[s] = Scalars{mn, gi};
-    a.counters[s] = 0;  // ready for the next call
   }
 }
 
@@ -447,7 +442,6 @@ HPX_API int hpx_terngrad_encode(int count, const float* const* ins, const int32_
     a.tile_start[0] = 0;
     a.partials = part_base + part_off;
     a.scalars = scal_base + first;
-    a.counters = ws->state;  // launches are stream-ordered and each leaves them zero
     int32_t qstart[kMaxSeg + 1];
     qstart[0] = 0;
     while (i < count && a.nseg < kMaxSeg) {
@@ -466,6 +460,8 @@ HPX_API int hpx_terngrad_encode(int count, const float* const* ins, const int32_
       i++;
     }
     hipLaunchKernelGGL(terngrad_minmax_kernel, dim3(a.tile_start[a.nseg]), dim3(kThreads), 0, st, a);
+    HPX_HIP(hipGetLastError());
+    hipLaunchKernelGGL(terngrad_finalize_kernel, dim3(a.nseg), dim3(kThreads), 0, st, a);
     HPX_HIP(hipGetLastError());
     part_off += size_t(a.tile_start[a.nseg]);
     for (int k = 0; k <= a.nseg; k++) a.tile_start[k] = qstart[k];
