@@ -1,0 +1,511 @@
+// PowerSGD rank-r phases over a batch of row-major fp32 matrices.
+//
+// Semantics are the ones the reference's comments state (powersgd_body.h:20-29,
+// :41-50, :64-76); its literal copy_ calls have source and destination
+// swapped:
+//   encode1  M.flat[:N] = grad + residual ;  P = M Q        (n x m)(m x r)
+//   encode2  P <- orthonormal columns     ;  Q = M^T P      (m x n)(n x r)
+//   decode   M = P Q^T ; residual = grad - M.flat[:N] ; grad = M.flat[:N]
+//
+// Every phase is one streaming pass over the n x m data, so all three are bound
+// by HBM; the rank-r contractions ride along on the matrix cores with
+// v_mfma_f32_4x4x1_16b_f32: sixteen independent 4x4 outer-product blocks per
+// instruction, so four columns of a rank-4 factor fill the N dimension exactly.
+// Operand layout of that instruction: A[blk][i] in lane 4*blk+i, B[blk][j] in
+// lane 4*blk+j, D[blk][i][j] in lane 4*blk+j, register i.
+//
+// Ranks up to 16 are handled as up to four column groups of four.
+#include "hpx_common.h"
+
+namespace {
+using namespace hpx;
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / kWave;
+constexpr int kMaxSeg = 40;
+constexpr int kMaxCG = 4;                 // column groups of 4 -> rank <= 16
+constexpr int kStrip = 256;               // columns per wave step in encode2 / decode
+constexpr int kE2RowsPerBlock = 128;      // rows folded into one partial of Q
+constexpr int kDecRowsPerBlock = 128;
+
+struct Seg {
+  const float* grad;   // encode1: in.  decode: in/out (as float*)
+  const float* res;    // encode1: in.  decode: out
+  const float* Q;
+  float* M;
+  float* P;
+  float* Qout;         // encode2: Q to write;  partials live in the workspace
+  int64_t numel;
+  int32_t n, m, r;
+  int32_t part_off;    // encode2: offset (in floats / 4) of this matrix's partials
+};
+struct Args {
+  int32_t nseg;
+  int32_t tile_start[kMaxSeg + 1];
+  Seg seg[kMaxSeg];
+  float* partials;
+};
+static_assert(sizeof(Args) <= 4096, "kernarg limit");
+
+__device__ __forceinline__ f32x4 mfma4(float a, float b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_4x4x1f32(a, b, c, 0, 0, 0);
+}
+
+// ---- encode1: M = G + R (flat prefix), P = M Q -------------------------------
+// One workgroup per group of 4 rows; its 4 waves split the columns and meet in
+// LDS.  Lane 4b+i of a wave owns row i and the 4 columns k0+4b..k0+4b+3 of each
+// 64-column step, which is one 128-bit load of G and of R and one store of M.
+template <int CG>
+__global__ __launch_bounds__(kThreads) void psgd_encode1_kernel(const Args a) {
+  const int tile = blockIdx.x;
+  const int s = find_segment<kMaxSeg>(a.tile_start, a.nseg, tile);
+  const Seg& sg = a.seg[s];
+  const float* __restrict__ G = sg.grad;
+  const float* __restrict__ R = sg.res;
+  const float* __restrict__ Q = sg.Q;
+  float* __restrict__ M = sg.M;
+  const int n = sg.n, m = sg.m, r = sg.r;
+  const int64_t N = sg.numel;
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int row0 = (tile - a.tile_start[s]) * 4;
+  const int i = lane & 3, b = lane >> 2;
+  const int row = row0 + i;
+  // columns of this wave: a contiguous quarter, in whole 64-column steps
+  const int steps = (m + 63) / 64;
+  const int per = (steps + kWaves - 1) / kWaves;
+  const int kbeg = wave * per * 64;
+  int kend = kbeg + per * 64;
+  if (kend > m) kend = m;
+
+  f32x4 acc[CG];
+#pragma unroll
+  for (int c = 0; c < CG; c++) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const bool rows_full = (row0 + 3 < n) && (int64_t(row0 + 4) * m <= N);
+  for (int k0 = kbeg; k0 < kend; k0 += 64) {
+    const int kk = k0 + 4 * b;
+    float v[4];
+    if (rows_full && k0 + 64 <= m) {
+      const int64_t f = int64_t(row) * m + kk;
+      const float4 g4 = ld4(G + f), r4 = ld4(R + f);
+      const float4 m4 = make_float4(g4.x + r4.x, g4.y + r4.y, g4.z + r4.z, g4.w + r4.w);
+      st4(M + f, m4);
+      v[0] = m4.x; v[1] = m4.y; v[2] = m4.z; v[3] = m4.w;
+    } else {
+#pragma unroll
+      for (int t = 0; t < 4; t++) {
+        const int k = kk + t;
+        float x = 0.f;
+        if (row < n && k < m) {
+          const int64_t f = int64_t(row) * m + k;
+          if (f < N) {
+            x = G[f] + R[f];
+            M[f] = x;
+          } else {
+            x = M[f];  // beyond the gradient: whatever the caller left in M takes part in P = M Q
+          }
+        }
+        v[t] = x;
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+      const int k = kk + t;
+#pragma unroll
+      for (int c = 0; c < CG; c++) {
+        const int col = c * 4 + i;  // B operand: lane 4b+j holds Q[k][j]
+        const float q = (k < m && col < r) ? Q[int64_t(k) * r + col] : 0.f;
+        acc[c] = mfma4(v[t], q, acc[c]);
+      }
+    }
+  }
+  // acc[c][ii] in lane 4b+j is the part of P[row0+ii][4c+j] from this lane's columns: fold the 16 blocks
+  __shared__ float s_p[kWaves][CG][4][4];
+#pragma unroll
+  for (int c = 0; c < CG; c++)
+#pragma unroll
+    for (int ii = 0; ii < 4; ii++) {
+      float x = acc[c][ii];
+#pragma unroll
+      for (int o = 4; o < kWave; o <<= 1) x += __shfl_xor(x, o, kWave);
+      if (lane < 4) s_p[wave][c][ii][lane] = x;
+    }
+  __syncthreads();
+  if (threadIdx.x < CG * 16) {
+    const int c = threadIdx.x / 16, ii = (threadIdx.x / 4) & 3, j = threadIdx.x & 3;
+    const int col = c * 4 + j;
+    if (row0 + ii < n && col < r) {
+      float x = s_p[0][c][ii][j];
+#pragma unroll
+      for (int w = 1; w < kWaves; w++) x += s_p[w][c][ii][j];
+      sg.P[int64_t(row0 + ii) * r + col] = x;
+    }
+  }
+}
+
+// ---- encode2, step 1: orthonormalise the columns of P -------------------------
+// Modified Gram-Schmidt, two sweeps (the second restores orthogonality lost to
+// cancellation), reductions in fp64.  One workgroup per matrix; P is n x r <= 16.
+constexpr int kOrthThreads = 1024;
+
+__device__ __forceinline__ double block_sum(double v, double* s_red) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  const int w = threadIdx.x / kWave;
+  __syncthreads();
+  if ((threadIdx.x & (kWave - 1)) == 0) s_red[w] = v;
+  __syncthreads();
+  double t = 0;
+#pragma unroll
+  for (int k = 0; k < kOrthThreads / kWave; k++) t += s_red[k];
+  return t;
+}
+
+__global__ __launch_bounds__(kOrthThreads) void psgd_orth_kernel(const Args a) {
+  __shared__ double s_red[kOrthThreads / kWave];
+  const Seg& sg = a.seg[blockIdx.x];
+  float* __restrict__ P = sg.P;
+  const int n = sg.n, r = sg.r;
+  for (int sweep = 0; sweep < 2; sweep++) {
+    for (int c = 0; c < r; c++) {
+      double ss = 0;
+      for (int row = threadIdx.x; row < n; row += kOrthThreads) {
+        const double x = P[int64_t(row) * r + c];
+        ss += x * x;
+      }
+      ss = block_sum(ss, s_red);
+      const float inv = ss > 0 ? static_cast<float>(1.0 / sqrt(ss)) : 0.f;
+      for (int row = threadIdx.x; row < n; row += kOrthThreads) P[int64_t(row) * r + c] *= inv;
+      for (int c2 = c + 1; c2 < r; c2++) {
+        double d = 0;
+        for (int row = threadIdx.x; row < n; row += kOrthThreads)
+          d += double(P[int64_t(row) * r + c]) * double(P[int64_t(row) * r + c2]);
+        d = block_sum(d, s_red);
+        const float df = static_cast<float>(d);
+        for (int row = threadIdx.x; row < n; row += kOrthThreads)
+          P[int64_t(row) * r + c2] -= df * P[int64_t(row) * r + c];
+      }
+    }
+  }
+}
+
+// ---- encode2, step 2: Q = M^T P ------------------------------------------------
+// A workgroup takes a strip of 256 columns and 128 rows (32 per wave).  Per row a
+// lane loads its 4 columns of M with one 128-bit load; register t of that load
+// is the A operand of MFMA t, whose block b / row-of-block i' is column
+// k0 + 16b + 4i' + t; the B operand is P[row][j] in every block.  The waves meet
+// in LDS and the workgroup writes one partial of Q; a second kernel adds the
+// partials in a fixed order.
+template <int CG>
+__global__ __launch_bounds__(kThreads) void psgd_mtp_kernel(const Args a) {
+  const int tile = blockIdx.x;
+  const int s = find_segment<kMaxSeg>(a.tile_start, a.nseg, tile);
+  const Seg& sg = a.seg[s];
+  const float* __restrict__ M = sg.M;
+  const float* __restrict__ P = sg.P;
+  const int n = sg.n, m = sg.m, r = sg.r;
+  const int strips = (m + kStrip - 1) / kStrip;
+  const int t_in = tile - a.tile_start[s];
+  const int strip = t_in % strips, rblk = t_in / strips;
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int k0 = strip * kStrip;
+  const int kk = k0 + 4 * lane;
+  const int rbeg = rblk * kE2RowsPerBlock + wave * (kE2RowsPerBlock / kWaves);
+  int rend = rbeg + kE2RowsPerBlock / kWaves;
+  if (rend > n) rend = n;
+
+  f32x4 acc[CG][4];
+#pragma unroll
+  for (int c = 0; c < CG; c++)
+#pragma unroll
+    for (int t = 0; t < 4; t++) acc[c][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const bool cols_full = k0 + kStrip <= m;
+  const int j = lane & 3;
+  for (int row = rbeg; row < rend; row++) {
+    float v[4];
+    if (cols_full) {
+      const float4 m4 = ld4(M + int64_t(row) * m + kk);
+      v[0] = m4.x; v[1] = m4.y; v[2] = m4.z; v[3] = m4.w;
+    } else {
+#pragma unroll
+      for (int t = 0; t < 4; t++) v[t] = (kk + t < m) ? M[int64_t(row) * m + kk + t] : 0.f;
+    }
+#pragma unroll
+    for (int c = 0; c < CG; c++) {
+      const int col = c * 4 + j;
+      const float p = col < r ? P[int64_t(row) * r + col] : 0.f;
+#pragma unroll
+      for (int t = 0; t < 4; t++) acc[c][t] = mfma4(v[t], p, acc[c][t]);
+    }
+  }
+  // acc[c][t][i'] in lane 4b+j  ->  Q[k0 + 16b + 4i' + t][4c + j]
+  __shared__ float s_q[kWaves][CG][kStrip][4];
+#pragma unroll
+  for (int c = 0; c < CG; c++)
+#pragma unroll
+    for (int t = 0; t < 4; t++)
+#pragma unroll
+      for (int ii = 0; ii < 4; ii++) s_q[wave][c][16 * (lane >> 2) + 4 * ii + t][j] = acc[c][t][ii];
+  __syncthreads();
+  float* part = a.partials + (int64_t(sg.part_off) * 4) + int64_t(rblk) * m * r;
+  for (int e = threadIdx.x; e < CG * kStrip * 4; e += kThreads) {
+    const int c = e / (kStrip * 4), kl = (e / 4) % kStrip, jj = e & 3;
+    const int k = k0 + kl, col = c * 4 + jj;
+    if (k < m && col < r) {
+      float x = s_q[0][c][kl][jj];
+#pragma unroll
+      for (int w = 1; w < kWaves; w++) x += s_q[w][c][kl][jj];
+      part[int64_t(k) * r + col] = x;
+    }
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void psgd_qreduce_kernel(const Args a) {
+  const int tile = blockIdx.x;
+  const int s = find_segment<kMaxSeg>(a.tile_start, a.nseg, tile);
+  const Seg& sg = a.seg[s];
+  const int64_t mr = int64_t(sg.m) * sg.r;
+  const int nparts = (sg.n + kE2RowsPerBlock - 1) / kE2RowsPerBlock;
+  const float* part = a.partials + int64_t(sg.part_off) * 4;
+  const int64_t e = int64_t(tile - a.tile_start[s]) * kThreads + threadIdx.x;
+  if (e < mr) {
+    float x = 0.f;
+    for (int p = 0; p < nparts; p++) x += part[int64_t(p) * mr + e];
+    sg.Qout[e] = x;
+  }
+}
+
+// ---- decode: M = P Q^T, residual = grad - M, grad = M ---------------------------
+// A workgroup takes a strip of 256 columns and 128 rows (32 per wave).  MFMA
+// (t, j) has A = P[row0+i'][j] and B = Q[k0+4*lane+t][j], so after the sum over
+// j register i' of accumulator t is M[row0+i'][k0+4*lane+t]: the four
+// accumulators give each lane 4 consecutive columns of 4 rows, i.e. 128-bit
+// loads of grad and 128-bit stores of M, residual and grad.
+template <int CG>
+__global__ __launch_bounds__(kThreads) void psgd_decode_kernel(const Args a) {
+  const int tile = blockIdx.x;
+  const int s = find_segment<kMaxSeg>(a.tile_start, a.nseg, tile);
+  const Seg& sg = a.seg[s];
+  const float* __restrict__ P = sg.P;
+  const float* __restrict__ Q = sg.Q;
+  float* __restrict__ M = sg.M;
+  float* __restrict__ G = const_cast<float*>(sg.grad);
+  float* __restrict__ R = const_cast<float*>(sg.res);
+  const int n = sg.n, m = sg.m, r = sg.r;
+  const int64_t N = sg.numel;
+  const int strips = (m + kStrip - 1) / kStrip;
+  const int t_in = tile - a.tile_start[s];
+  const int strip = t_in % strips, rblk = t_in / strips;
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int k0 = strip * kStrip;
+  const int kk = k0 + 4 * lane;
+  const int rbeg = rblk * kDecRowsPerBlock + wave * (kDecRowsPerBlock / kWaves);
+  int rend = rbeg + kDecRowsPerBlock / kWaves;
+  if (rend > n) rend = n;
+  const int i = lane & 3;
+
+  float q[4][CG * 4];  // Q[kk+t][col]
+#pragma unroll
+  for (int t = 0; t < 4; t++)
+#pragma unroll
+    for (int col = 0; col < CG * 4; col++) q[t][col] = (kk + t < m && col < r) ? Q[int64_t(kk + t) * r + col] : 0.f;
+
+  const bool cols_full = k0 + kStrip <= m;
+  for (int row0 = rbeg; row0 < rend; row0 += 4) {
+    f32x4 acc[4];
+#pragma unroll
+    for (int t = 0; t < 4; t++) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int col = 0; col < CG * 4; col++) {
+      const float p = (row0 + i < n && col < r) ? P[int64_t(row0 + i) * r + col] : 0.f;
+#pragma unroll
+      for (int t = 0; t < 4; t++) acc[t] = mfma4(p, q[t][col], acc[t]);
+    }
+#pragma unroll
+    for (int ii = 0; ii < 4; ii++) {
+      const int row = row0 + ii;
+      if (row >= rend) break;
+      const int64_t f = int64_t(row) * m + kk;
+      const float4 m4 = make_float4(acc[0][ii], acc[1][ii], acc[2][ii], acc[3][ii]);
+      if (cols_full && f + 4 <= N) {
+        const float4 g4 = ld4(G + f);
+        st4(R + f, make_float4(g4.x - m4.x, g4.y - m4.y, g4.z - m4.z, g4.w - m4.w));
+        st4(G + f, m4);
+        st4(M + f, m4);
+      } else {
+        const float mv[4] = {m4.x, m4.y, m4.z, m4.w};
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+          if (kk + t < m) {
+            if (f + t < N) {
+              R[f + t] = G[f + t] - mv[t];
+              G[f + t] = mv[t];
+            }
+            M[f + t] = mv[t];
+          }
+        }
+      }
+    }
+  }
+}
+
+inline int32_t cdiv(int64_t x, int64_t y) { return static_cast<int32_t>((x + y - 1) / y); }
+
+struct Batch {
+  int count;
+  const int32_t *ns, *ms, *rs;
+};
+
+int check_dims(const char* who, const Batch& b, int* max_cg) {
+  *max_cg = 1;
+  for (int i = 0; i < b.count; i++) {
+    HPX_ARG(b.ns[i] > 0 && b.ms[i] > 0 && b.rs[i] > 0, "%s: matrix %d has dims %d x %d rank %d", who, i, b.ns[i], b.ms[i],
+            b.rs[i]);
+    HPX_ARG(b.rs[i] <= 4 * kMaxCG, "%s: matrix %d has rank %d; ranks above %d are not supported", who, i, b.rs[i],
+            4 * kMaxCG);
+    const int cg = (b.rs[i] + 3) / 4;
+    if (cg > *max_cg) *max_cg = cg;
+  }
+  return HPX_OK;
+}
+
+#define PSGD_LAUNCH_CG(KERNEL, cg, grid, st, args)                                              \
+  switch (cg) {                                                                                 \
+    case 1: hipLaunchKernelGGL(KERNEL<1>, dim3(grid), dim3(kThreads), 0, st, args); break;      \
+    case 2: hipLaunchKernelGGL(KERNEL<2>, dim3(grid), dim3(kThreads), 0, st, args); break;      \
+    case 3: hipLaunchKernelGGL(KERNEL<3>, dim3(grid), dim3(kThreads), 0, st, args); break;      \
+    default: hipLaunchKernelGGL(KERNEL<4>, dim3(grid), dim3(kThreads), 0, st, args); break;     \
+  }
+
+}  // namespace
+
+HPX_API int hpx_powersgd_encode1(int count, const float* const* grads, const int64_t* numels,
+                                 const float* const* residuals, const float* const* Qs, float* const* Ms,
+                                 float* const* Ps, const int32_t* ns, const int32_t* ms, const int32_t* rs,
+                                 hpx_stream_t stream) {
+  hpx::clear_error();
+  HPX_ARG(count >= 0, "hpx_powersgd_encode1: negative count");
+  if (count == 0) return HPX_OK;
+  HPX_ARG(grads && numels && residuals && Qs && Ms && Ps && ns && ms && rs, "hpx_powersgd_encode1: null argument array");
+  int cg = 1;
+  int rc = check_dims("hpx_powersgd_encode1", Batch{count, ns, ms, rs}, &cg);
+  if (rc != HPX_OK) return rc;
+  for (int i = 0; i < count; i++) {
+    HPX_ARG(grads[i] && residuals[i] && Qs[i] && Ms[i] && Ps[i], "hpx_powersgd_encode1: matrix %d has a null pointer", i);
+    HPX_ARG(numels[i] >= 0 && numels[i] <= int64_t(ns[i]) * ms[i], "hpx_powersgd_encode1: matrix %d: numel %lld exceeds n*m", i,
+            static_cast<long long>(numels[i]));
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  Args a;
+  a.partials = nullptr;
+  int i = 0;
+  while (i < count) {
+    a.nseg = 0;
+    a.tile_start[0] = 0;
+    while (i < count && a.nseg < kMaxSeg) {
+      const int32_t t = cdiv(ns[i], 4);
+      if (int64_t(a.tile_start[a.nseg]) + t > INT32_MAX) break;
+      a.seg[a.nseg] = Seg{grads[i], residuals[i], Qs[i], Ms[i], Ps[i], nullptr, numels[i], ns[i], ms[i], rs[i], 0};
+      a.tile_start[a.nseg + 1] = a.tile_start[a.nseg] + t;
+      a.nseg++;
+      i++;
+    }
+    PSGD_LAUNCH_CG(psgd_encode1_kernel, cg, a.tile_start[a.nseg], st, a);
+    HPX_HIP(hipGetLastError());
+  }
+  return HPX_OK;
+}
+
+HPX_API int hpx_powersgd_encode2(int count, float* const* Ps, const float* const* Ms, float* const* Qs,
+                                 const int32_t* ns, const int32_t* ms, const int32_t* rs, hpx_stream_t stream) {
+  hpx::clear_error();
+  HPX_ARG(count >= 0, "hpx_powersgd_encode2: negative count");
+  if (count == 0) return HPX_OK;
+  HPX_ARG(Ps && Ms && Qs && ns && ms && rs, "hpx_powersgd_encode2: null argument array");
+  int cg = 1;
+  int rc = check_dims("hpx_powersgd_encode2", Batch{count, ns, ms, rs}, &cg);
+  if (rc != HPX_OK) return rc;
+  int64_t part_quads = 0;  // partial storage in units of 4 floats
+  for (int i = 0; i < count; i++) {
+    HPX_ARG(Ps[i] && Ms[i] && Qs[i], "hpx_powersgd_encode2: matrix %d has a null pointer", i);
+    part_quads += (int64_t(cdiv(ns[i], kE2RowsPerBlock)) * ms[i] * rs[i] + 3) / 4;
+  }
+  HPX_ARG(part_quads <= INT32_MAX, "hpx_powersgd_encode2: batch too large for one call");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  hpx::Workspace* ws = hpx::workspace_record(st);
+  if (!ws) return HPX_ERR_HIP;
+  std::lock_guard<std::mutex> lock(ws->mu);
+  rc = hpx::ensure_workspace(ws, size_t(part_quads) * 16);
+  if (rc != HPX_OK) return rc;
+  Args a;
+  a.partials = reinterpret_cast<float*>(ws->dev);
+  int i = 0;
+  int64_t poff = 0;
+  while (i < count) {
+    const int first = i;
+    a.nseg = 0;
+    a.tile_start[0] = 0;
+    int32_t red_start[kMaxSeg + 1];
+    red_start[0] = 0;
+    while (i < count && a.nseg < kMaxSeg) {
+      const int32_t t = cdiv(ms[i], kStrip) * cdiv(ns[i], kE2RowsPerBlock);
+      const int32_t tr = cdiv(int64_t(ms[i]) * rs[i], kThreads);
+      if (int64_t(a.tile_start[a.nseg]) + t > INT32_MAX || int64_t(red_start[a.nseg]) + tr > INT32_MAX) break;
+      a.seg[a.nseg] = Seg{nullptr, nullptr, nullptr, const_cast<float*>(Ms[i]), Ps[i], Qs[i], 0, ns[i], ms[i], rs[i],
+                          static_cast<int32_t>(poff)};
+      poff += (int64_t(cdiv(ns[i], kE2RowsPerBlock)) * ms[i] * rs[i] + 3) / 4;
+      a.tile_start[a.nseg + 1] = a.tile_start[a.nseg] + t;
+      red_start[a.nseg + 1] = red_start[a.nseg] + tr;
+      a.nseg++;
+      i++;
+    }
+    (void)first;
+    hipLaunchKernelGGL(psgd_orth_kernel, dim3(a.nseg), dim3(kOrthThreads), 0, st, a);
+    PSGD_LAUNCH_CG(psgd_mtp_kernel, cg, a.tile_start[a.nseg], st, a);
+    HPX_HIP(hipGetLastError());
+    for (int k = 0; k <= a.nseg; k++) a.tile_start[k] = red_start[k];
+    hipLaunchKernelGGL(psgd_qreduce_kernel, dim3(a.tile_start[a.nseg]), dim3(kThreads), 0, st, a);
+    HPX_HIP(hipGetLastError());
+  }
+  return HPX_OK;
+}
+
+HPX_API int hpx_powersgd_decode(int count, const float* const* Ps, const float* const* Qs, float* const* Ms,
+                                float* const* residuals, float* const* grads, const int64_t* numels,
+                                const int32_t* ns, const int32_t* ms, const int32_t* rs, hpx_stream_t stream) {
+  hpx::clear_error();
+  HPX_ARG(count >= 0, "hpx_powersgd_decode: negative count");
+  if (count == 0) return HPX_OK;
+  HPX_ARG(Ps && Qs && Ms && residuals && grads && numels && ns && ms && rs, "hpx_powersgd_decode: null argument array");
+  int cg = 1;
+  int rc = check_dims("hpx_powersgd_decode", Batch{count, ns, ms, rs}, &cg);
+  if (rc != HPX_OK) return rc;
+  for (int i = 0; i < count; i++) {
+    HPX_ARG(Ps[i] && Qs[i] && Ms[i] && residuals[i] && grads[i], "hpx_powersgd_decode: matrix %d has a null pointer", i);
+    HPX_ARG(numels[i] >= 0 && numels[i] <= int64_t(ns[i]) * ms[i], "hpx_powersgd_decode: matrix %d: numel %lld exceeds n*m", i,
+            static_cast<long long>(numels[i]));
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  Args a;
+  a.partials = nullptr;
+  int i = 0;
+  while (i < count) {
+    a.nseg = 0;
+    a.tile_start[0] = 0;
+    while (i < count && a.nseg < kMaxSeg) {
+      const int32_t t = cdiv(ms[i], kStrip) * cdiv(ns[i], kDecRowsPerBlock);
+      if (int64_t(a.tile_start[a.nseg]) + t > INT32_MAX) break;
+      a.seg[a.nseg] = Seg{grads[i], residuals[i], Qs[i], Ms[i], const_cast<float*>(Ps[i]), nullptr, numels[i], ns[i], ms[i],
+                          rs[i], 0};
+      a.tile_start[a.nseg + 1] = a.tile_start[a.nseg] + t;
+      a.nseg++;
+      i++;
+    }
+    PSGD_LAUNCH_CG(psgd_decode_kernel, cg, a.tile_start[a.nseg], st, a);
+    HPX_HIP(hipGetLastError());
+  }
+  return HPX_OK;
+}
