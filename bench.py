@@ -1,0 +1,329 @@
+#!/usr/bin/env python3
+"""Benchmark of the gradient-compression hot path on ONE MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one encode + decode pass of the headline workload through the C ABI:
+the TernGrad 2-bit quantiser on a ResNet-50-sized fp32 gradient (25,557,032
+elements ~N(0,1e-2) with 0.1 % outliers at +-50 sigma, stochastic rounding with a
+fixed seed, decode back to fp32).  Inputs are resident in HBM before the clock
+starts.  Buffers rotate over several distinct sets so that a step never finds
+its input in the 256 MB Infinity Cache from the step before.
+
+Prints ONE JSON line:  value = GB/s of fp32 gradient (4*N bytes per step) over
+the whole timed region; "roofline" prices the dominant kernel against the HBM
+peak with its duration measured by HIP events on the launch stream;
+"cpu_baseline" is the plain-C oracle (a port of the reference's CPU bodies)
+timed on the host cores of the same box; "extra" carries the other codecs of
+the path at their configuration sizes.
+"""
+import argparse
+import ctypes as C
+import importlib
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
+FP32_MFMA_PEAK_TF = 157.3   # MI355X dense fp32 matrix, published
+N_TERNGRAD = 25_557_032
+N_DGC = 138_357_544
+
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+# (scaled by a copy kernel of known size); None until such a run has been summarised under profiles/.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--sets", type=int, default=4, help="distinct buffer sets rotated between steps")
+    ap.add_argument("--cpu-seconds", type=float, default=10.0, help="time budget of the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the TBQ / DGC / PowerSGD side measurements")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    return ap.parse_args()
+
+
+class Call:
+    """A C-ABI call with its argument arrays marshalled once."""
+
+    def __init__(self, fn, *args):
+        self.fn, self.args = fn, args
+
+    def __call__(self):
+        rc = self.fn(*self.args)
+        if rc:
+            raise RuntimeError(f"{self.fn.__name__} returned {rc}")
+
+
+def timed(torch, fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def kernel_times(torch, capi, fn, names, reps=10):
+    """Average duration (s) of each named kernel, HIP events on the launch stream."""
+    L = capi.load()
+    torch.cuda.synchronize()
+    L.hpx_profile_reset()
+    L.hpx_profile_enable(1)
+    for _ in range(reps):
+        fn()
+    torch.cuda.synchronize()
+    L.hpx_profile_enable(0)
+    out = {}
+    for k in names:
+        ms, n = capi.profile_query(k)
+        out[k] = (ms / n) * 1e-3 if n else None
+    L.hpx_profile_reset()
+    return out
+
+
+def outlier_gradient(torch, n, gen):
+    x = torch.randn(n, device="cuda", generator=gen) * 1e-2
+    pos = torch.randint(0, n, (n // 1000,), device="cuda", generator=gen)
+    x[pos] = torch.where(torch.rand(pos.numel(), device="cuda", generator=gen) < 0.5, 0.5, -0.5)
+    return x
+
+
+def main():
+    args = parse()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: this path has no inter-GPU communication; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import numpy as np
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    torch.cuda.set_device(0)
+    pkg = importlib.import_module("torch-hipress-extension_amd")
+    capi = pkg._capi
+    L = capi.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    gen = torch.Generator(device="cuda").manual_seed(0)
+
+    # ---- headline: TernGrad 2-bit encode + decode, N = 25,557,032 --------------------------
+    n = N_TERNGRAD
+    msg_bytes = 10 + (n + 3) // 4
+    sets = []
+    for s in range(max(1, args.sets)):
+        x = outlier_gradient(torch, n, gen)
+        msg = torch.zeros(msg_bytes, dtype=torch.uint8, device="cuda")
+        dec = torch.empty(n, device="cuda")
+        enc = Call(L.hpx_terngrad_encode, 1, capi.ptr_array([x.data_ptr()]), capi.i32_array([n]),
+                   capi.ptr_array([msg.data_ptr()]), capi.i32_array([msg_bytes]), capi.u8_array([2]),
+                   capi.i32_array([1]), capi.u64_array([0]), stream)
+        dcd = Call(L.hpx_terngrad_decode, 1, capi.ptr_array([dec.data_ptr()]), capi.i32_array([n]),
+                   capi.ptr_array([msg.data_ptr()]), capi.i32_array([msg_bytes]), capi.i32_array([0]), stream)
+        sets.append((x, msg, dec, enc, dcd))
+    state = {"i": 0}
+
+    def step():
+        _, _, _, enc, dcd = sets[state["i"] % len(sets)]
+        state["i"] += 1
+        enc()
+        dcd()
+
+    sec = timed(torch, step, args.steps, args.warmup)
+    value = 4.0 * n / sec / 1e9
+
+    def warm_step():
+        sets[0][3]()
+        sets[0][4]()
+
+    sec_warm = timed(torch, warm_step, max(20, args.steps // 4), 5)
+    def only(which):
+        def f():
+            state["i"] += 1
+            sets[state["i"] % len(sets)][which]()
+        return f
+
+    sec_enc = timed(torch, only(3), max(20, args.steps // 4), 5)
+    sec_dec = timed(torch, only(4), max(20, args.steps // 4), 5)
+
+    kt = kernel_times(torch, capi, step,
+                      ["terngrad_minmax_kernel", "terngrad_finalize_kernel", "terngrad_quant_kernel", "terngrad_decode_kernel"])
+    alg_bytes = {  # algorithmic bytes per launch: every distinct input byte once, every output byte once
+        "terngrad_minmax_kernel": 4.0 * n,
+        "terngrad_quant_kernel": 4.0 * n + msg_bytes,
+        "terngrad_decode_kernel": msg_bytes + 4.0 * n,
+    }
+    dom = max(alg_bytes, key=lambda k: kt[k] or 0.0)
+    achieved = alg_bytes[dom] / kt[dom] / 1e9
+    roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(dom),
+                "algorithmic_bytes_per_launch": alg_bytes[dom], "avg_launch_us": round(kt[dom] * 1e6, 2),
+                "kernel_us": {k: (round(v * 1e6, 2) if v else None) for k, v in kt.items()}}
+    path_alg = 8.5 * n  # x once in, codes out; codes in, fp32 out
+    path = {"algorithmic_bytes_per_step": path_alg, "achieved_GBps": round(path_alg / sec / 1e9, 1),
+            "frac_of_hbm_peak": round(path_alg / sec / 1e9 / HBM_PEAK_GBS, 4),
+            "warm_cache_ms_per_step": round(sec_warm * 1e3, 4), "encode_ms": round(sec_enc * 1e3, 4),
+            "decode_ms": round(sec_dec * 1e3, 4), "buffer_sets": len(sets)}
+
+    result = {
+        "metric": "encode+decode GB/s of fp32 gradient (TernGrad 2-bit, 1 GPU)", "value": round(value, 2), "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(sec * 1e3, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "terngrad_2bit_resnet50", "elements": n, "bitwidth": 2, "enable_random": 1, "seed": 0,
+                   "outliers": "0.1% at +-50 sigma", "decode": "write"},
+        "roofline": roofline, "path_roofline": path,
+    }
+
+    del sets
+    torch.cuda.empty_cache()
+
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(np, n, args.cpu_seconds)
+    if not args.no_extra:
+        result["extra"] = extra(torch, np, capi, L, stream, gen)
+    print(json.dumps(result), flush=True)
+
+
+def cpu_baseline(np, n, budget_s):
+    """The plain-C oracle (port of the reference's CPU bodies, OpenMP) on the same workload."""
+    from oracle import cpu
+    threads = cpu.max_threads()
+    rng = np.random.default_rng(0)
+    x = rng.normal(0, 1e-2, n).astype(np.float32)
+    pos = rng.integers(0, n, n // 1000)
+    x[pos] = np.where(rng.random(pos.size) < 0.5, 0.5, -0.5).astype(np.float32)
+    out = np.zeros(n, np.float32)
+
+    def one():
+        rc, msg = cpu.terngrad_encode(x, 2, 1, 0)
+        cpu.terngrad_decode(msg, n, out)
+
+    one()
+    one()
+    t0 = time.perf_counter()
+    reps = 0
+    while reps < 3 or (time.perf_counter() - t0 < budget_s and reps < 200):
+        one()
+        reps += 1
+    sec = (time.perf_counter() - t0) / reps
+    return {"value": round(4.0 * n / sec / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"{reps} full encode+decode passes of the same {n}-element workload, OpenMP over {threads} threads "
+                      f"(os.cpu_count()={os.cpu_count()})", "ms_per_step": round(sec * 1e3, 2)}
+
+
+def extra(torch, np, capi, L, stream, gen):
+    """Other codecs of the path at their configuration sizes (GPU only, short runs)."""
+    res = {}
+    # ---- TBQ fused bucket: 110M elements in 200 tensors, thr = 2 sigma ----------------------
+    rng = np.random.default_rng(0)
+    sizes = np.exp(rng.uniform(np.log(768), np.log(3e7), 200))
+    sizes = np.clip(np.floor(sizes * 110e6 / sizes.sum()), 768, 3e7).astype(np.int64)
+    sizes[np.argmax(sizes)] += 110_000_000 - sizes.sum()
+    tot = int(sizes.sum())
+    gs = [torch.randn(int(s), device="cuda", generator=gen) * 5e-3 for s in sizes]
+    rs = [torch.zeros(int(s), device="cuda") for s in sizes]
+    ps = [torch.zeros((int(s) + 3) // 4, dtype=torch.uint8, device="cuda") for s in sizes]
+    os_ = [torch.empty(int(s), device="cuda") for s in sizes]
+    thr = capi.f32_array([1e-2] * len(sizes))
+    szs = capi.i32_array([int(s) for s in sizes])
+    enc = Call(L.hpx_tbq_encode, len(sizes), capi.ptr_array([g.data_ptr() for g in gs]), szs,
+               capi.ptr_array([r.data_ptr() for r in rs]), capi.ptr_array([p.data_ptr() for p in ps]), thr, stream)
+    dec = Call(L.hpx_tbq_decode, len(sizes), capi.ptr_array([o.data_ptr() for o in os_]), szs,
+               capi.ptr_array([p.data_ptr() for p in ps]), thr, capi.i32_array([0] * len(sizes)), stream)
+
+    def tbq_step():
+        enc()
+        dec()
+
+    sec = timed(torch, tbq_step, 30, 5)
+    kt = kernel_times(torch, capi, tbq_step, ["tbq_encode_kernel", "tbq_decode_kernel"], reps=5)
+    # both kernels run several launches per call when the bucket exceeds one table: total per call = avg * launches
+    res["tbq_bucket_110M_200_tensors"] = {
+        "ms_per_step": round(sec * 1e3, 4), "GBps_of_gradient": round(4.0 * tot / sec / 1e9, 1),
+        "algorithmic_bytes": 16.5 * tot, "frac_of_hbm_peak": round(16.5 * tot / sec / 1e9 / HBM_PEAK_GBS, 4),
+        "kernel_us_per_launch": {k: round(v * 1e6, 1) for k, v in kt.items() if v}}
+    del gs, rs, ps, os_
+    torch.cuda.empty_cache()
+
+    # ---- DGC / GradDrop top-0.1 %: 138,357,544 elements --------------------------------------
+    n = N_DGC
+    u = torch.rand(n, device="cuda", generator=gen) - 0.5
+    g = (-1e-3 * torch.sign(u) * torch.log1p(-2 * u.abs())).float()
+    del u
+    r0 = torch.randn(n, device="cuda", generator=gen) * 1e-4
+    r = r0.clone()
+    out = torch.zeros(4 + 8 * int(np.ceil(n * (1 - 0.999))), dtype=torch.uint8, device="cuda")
+    gd = Call(L.hpx_gd_encode, 1, capi.ptr_array([g.data_ptr()]), capi.i32_array([n]), capi.ptr_array([r.data_ptr()]),
+              capi.ptr_array([out.data_ptr()]), capi.f64_array([0.01]), capi.f64_array([0.999]), capi.u64_array([0]), stream)
+    times = []
+    for it in range(12):
+        r.copy_(r0)                      # every repetition sees the configuration's residual
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        gd()
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+    sec = float(np.median(times[2:]))
+    k = (int(out[:4].cpu().numpy().view(np.int32)[0]) - 4) // 8
+    r.copy_(r0)
+    kt = kernel_times(torch, capi, gd, ["gd_select_kernel", "gd_threshold_kernel", "gd_stream_kernel", "gd_scan_kernel",
+                                        "gd_expand_kernel", "gd_gather_kernel", "gd_sort_scatter_kernel"], reps=1)
+    dout = torch.zeros(n, device="cuda")
+    gdr = Call(L.hpx_gd_decode, 1, capi.ptr_array([out.data_ptr()]), capi.i32_array([out.numel()]),
+               capi.ptr_array([dout.data_ptr()]), capi.i32_array([n]), capi.i32_array([1]), stream)
+    sec_dec = timed(torch, gdr, 20, 3)
+    res["dgc_top0.1pct_138M"] = {
+        "encode_ms": round(sec * 1e3, 4), "encode_GBps_of_gradient": round(4.0 * n / sec / 1e9, 1), "selected": k,
+        "algorithmic_bytes": 12.0 * n + 8 * k + 4, "frac_of_hbm_peak": round((12.0 * n + 8 * k + 4) / sec / 1e9 / HBM_PEAK_GBS, 4),
+        "stream_kernel_frac_of_hbm_peak": round(12.0 * n / kt["gd_stream_kernel"] / 1e9 / HBM_PEAK_GBS, 4) if kt["gd_stream_kernel"] else None,
+        "decode_add_ms": round(sec_dec * 1e3, 4), "kernel_us_per_launch": {k_: round(v * 1e6, 1) for k_, v in kt.items() if v}}
+    del g, r, r0, out, dout
+    torch.cuda.empty_cache()
+
+    # ---- PowerSGD rank 4 over the 36-matrix layer set ------------------------------------------
+    shapes = [(4096, 4096)] * 12 + [(1024, 4096)] * 12 + [(4096, 1024)] * 12
+    rk = 4
+    G = [torch.randn(a * b, device="cuda", generator=gen) * 1e-2 for a, b in shapes]
+    R = [torch.zeros(a * b, device="cuda") for a, b in shapes]
+    Q = [torch.randn(b, rk, device="cuda", generator=gen) for a, b in shapes]
+    M = [torch.zeros(a, b, device="cuda") for a, b in shapes]
+    P = [torch.zeros(a, rk, device="cuda") for a, b in shapes]
+    ns, ms, rs_ = capi.i32_array([a for a, b in shapes]), capi.i32_array([b for a, b in shapes]), capi.i32_array([rk] * 36)
+    numels = capi.i64_array([a * b for a, b in shapes])
+    pa = lambda ts: capi.ptr_array([t.data_ptr() for t in ts])
+    e1 = Call(L.hpx_powersgd_encode1, 36, pa(G), numels, pa(R), pa(Q), pa(M), pa(P), ns, ms, rs_, stream)
+    e2 = Call(L.hpx_powersgd_encode2, 36, pa(P), pa(M), pa(Q), ns, ms, rs_, stream)
+    dc = Call(L.hpx_powersgd_decode, 36, pa(P), pa(Q), pa(M), pa(R), pa(G), numels, ns, ms, rs_, stream)
+
+    def psgd_step():
+        e1()
+        e2()
+        dc()
+
+    sec = timed(torch, psgd_step, 10, 2)
+    kt = kernel_times(torch, capi, psgd_step, ["psgd_encode1_kernel", "psgd_orth_kernel", "psgd_mtp_kernel",
+                                               "psgd_qreduce_kernel", "psgd_decode_kernel"], reps=3)
+    elems = sum(a * b for a, b in shapes)
+    flops = 24.0 * elems
+    res["powersgd_rank4_36_matrices"] = {
+        "ms_per_iteration": round(sec * 1e3, 4), "GBps_of_gradient": round(4.0 * elems / sec / 1e9, 1),
+        "algorithmic_bytes": 16.0 * elems, "frac_of_hbm_peak": round(16.0 * elems / sec / 1e9 / HBM_PEAK_GBS, 4),
+        "bytes_moved_by_three_phase_api": 32.0 * elems,
+        "frac_of_hbm_peak_three_phase_bytes": round(32.0 * elems / sec / 1e9 / HBM_PEAK_GBS, 4),
+        "mfma_frac_of_fp32_peak": round(flops / sec / 1e12 / FP32_MFMA_PEAK_TF, 5),
+        "kernel_us_per_launch": {k_: round(v * 1e6, 1) for k_, v in kt.items() if v}}
+    return res
+
+
+if __name__ == "__main__":
+    main()

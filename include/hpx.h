@@ -50,6 +50,17 @@ const char* hpx_last_error(void);
  * the caller's output buffer). */
 int hpx_release_workspaces(void);
 
+/* ---- measurement aid ------------------------------------------------------
+ * No counterpart in the reference.  While enabled, every kernel the library
+ * launches is bracketed by a pair of HIP events recorded on the stream of the
+ * launch; hpx_profile_query waits for them and returns the summed duration and
+ * the number of launches of the kernel with that name (e.g.
+ * "terngrad_decode_kernel").  hpx_profile_reset forgets what was recorded.
+ * Off by default; enabling it inserts events between kernels. */
+int hpx_profile_enable(int on);
+int hpx_profile_reset(void);
+int hpx_profile_query(const char* kernel, double* total_ms, int64_t* launches);
+
 /* ---- TBQ: threshold quantisation with residual feedback ------------------ */
 
 /* Replaces hp_cuda_tbq (hp_cuda.cpp:52-61, hp_cuda_kernel.cu:120-158; body

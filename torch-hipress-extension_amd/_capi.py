@@ -14,6 +14,9 @@ SYMBOLS = (
     "hpx_version",
     "hpx_last_error",
     "hpx_release_workspaces",
+    "hpx_profile_enable",
+    "hpx_profile_reset",
+    "hpx_profile_query",
     "hpx_tbq_encode",
     "hpx_tbq_decode",
     "hpx_terngrad_encode",
@@ -50,6 +53,8 @@ def load():
     L.hpx_version.restype = C.c_int
     L.hpx_last_error.restype = C.c_char_p
     L.hpx_release_workspaces.restype = C.c_int
+    L.hpx_profile_enable.argtypes = [C.c_int]
+    L.hpx_profile_query.argtypes = [C.c_char_p, C.POINTER(C.c_double), C.POINTER(C.c_int64)]
     L.hpx_tbq_encode.argtypes = [i32, pp, p, pp, pp, p, p]
     L.hpx_tbq_decode.argtypes = [i32, pp, p, pp, p, p, p]
     L.hpx_terngrad_encode.argtypes = [i32, pp, p, pp, p, p, p, p, p]
@@ -97,3 +102,12 @@ def f32_array(vals):
 
 def f64_array(vals):
     return (C.c_double * len(vals))(*[float(v) for v in vals])
+
+
+def profile_query(kernel):
+    """(total milliseconds, launches) recorded for `kernel` since the last reset."""
+    ms, n = C.c_double(), C.c_int64()
+    rc = load().hpx_profile_query(kernel.encode(), C.byref(ms), C.byref(n))
+    if rc:
+        raise HpxError(rc, last_error())
+    return ms.value, n.value

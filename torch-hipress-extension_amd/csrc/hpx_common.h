@@ -32,6 +32,20 @@ void clear_error();
     }                             \
   } while (0)
 
+// ---- per-kernel timing (measurement aid, off by default) ---------------------
+extern bool g_prof_on;
+void prof_begin(const char* name, hipStream_t st);
+void prof_end(hipStream_t st);
+
+// Every kernel goes out through this macro so that hpx_profile_* can bracket it
+// with HIP events on the stream it is launched on.
+#define HPX_LAUNCH(NAME, KERNEL, GRID, BLOCK, STREAM, ...)            \
+  do {                                                                \
+    if (hpx::g_prof_on) hpx::prof_begin(NAME, STREAM);                \
+    hipLaunchKernelGGL(KERNEL, GRID, BLOCK, 0, STREAM, __VA_ARGS__);  \
+    if (hpx::g_prof_on) hpx::prof_end(STREAM);                        \
+  } while (0)
+
 // ---- per-(device, stream) workspace ----------------------------------------
 // `dev` is grow-only scratch whose contents are meaningless between calls.
 // `state` is a small block that is zero when the library creates it and that

@@ -424,8 +424,8 @@ int sort_pairs_desc(uint32_t* keys_a, int32_t* idx_a, uint32_t* keys_b, int32_t*
   const uint32_t nblk = cdiv(n, kSortTile);
   for (int pass = 0; pass < 4; pass++) {
     const int shift = pass * 8;
-    hipLaunchKernelGGL(gd_sort_count_kernel, dim3(nblk), dim3(kThreads), 0, st, keys_a, n, shift, counts, nblk);
-    hipLaunchKernelGGL(gd_sort_scatter_kernel, dim3(nblk), dim3(kThreads), 0, st, keys_a, idx_a, n, shift, counts, nblk,
+    HPX_LAUNCH("gd_sort_count_kernel", gd_sort_count_kernel, dim3(nblk), dim3(kThreads), st, keys_a, n, shift, counts, nblk);
+    HPX_LAUNCH("gd_sort_scatter_kernel", gd_sort_scatter_kernel, dim3(nblk), dim3(kThreads), st, keys_a, idx_a, n, shift, counts, nblk,
                        keys_b, idx_b);
     HPX_HIP(hipGetLastError());
     std::swap(keys_a, keys_b);
@@ -478,19 +478,19 @@ int gd_encode_one(const float* g, int32_t N, float* r, uint8_t* out, double samp
              samples, hist, state};
   uint32_t sel_blocks = cdiv(sample_cnt, kSelThreads * 8);
   if (sel_blocks > kSelBlocksMax) sel_blocks = kSelBlocksMax;
-  hipLaunchKernelGGL(gd_select_kernel<1>, dim3(sel_blocks), dim3(kSelThreads), 0, st, sa);
-  hipLaunchKernelGGL(gd_select_kernel<2>, dim3(sel_blocks), dim3(kSelThreads), 0, st, sa);
-  hipLaunchKernelGGL(gd_select_kernel<3>, dim3(sel_blocks), dim3(kSelThreads), 0, st, sa);
-  hipLaunchKernelGGL(gd_threshold_kernel, dim3(1), dim3(kSelThreads), 0, st, sa);
-  hipLaunchKernelGGL(gd_stream_kernel, dim3(ntiles), dim3(kThreads), 0, st, g, r, n, state, masks, blk_cnt);
-  hipLaunchKernelGGL(gd_scan_kernel, dim3(1), dim3(kSelThreads), 0, st, blk_cnt, blk_off, ntiles, &state->total);
+  HPX_LAUNCH("gd_select_kernel", gd_select_kernel<1>, dim3(sel_blocks), dim3(kSelThreads), st, sa);
+  HPX_LAUNCH("gd_select_kernel", gd_select_kernel<2>, dim3(sel_blocks), dim3(kSelThreads), st, sa);
+  HPX_LAUNCH("gd_select_kernel", gd_select_kernel<3>, dim3(sel_blocks), dim3(kSelThreads), st, sa);
+  HPX_LAUNCH("gd_threshold_kernel", gd_threshold_kernel, dim3(1), dim3(kSelThreads), st, sa);
+  HPX_LAUNCH("gd_stream_kernel", gd_stream_kernel, dim3(ntiles), dim3(kThreads), st, g, r, n, state, masks, blk_cnt);
+  HPX_LAUNCH("gd_scan_kernel", gd_scan_kernel, dim3(1), dim3(kSelThreads), st, blk_cnt, blk_off, ntiles, &state->total);
   HPX_HIP(hipGetLastError());
   // Common case (nothing to cut) queued before the host knows the count.
   int32_t* out_idx = reinterpret_cast<int32_t*>(out + 4);
   const uint32_t lim = static_cast<uint32_t>(expected);
-  hipLaunchKernelGGL(gd_expand_kernel, dim3(cdiv(ntiles, kThreads / kWave)), dim3(kThreads), 0, st, masks, blk_off, ntiles,
+  HPX_LAUNCH("gd_expand_kernel", gd_expand_kernel, dim3(cdiv(ntiles, kThreads / kWave)), dim3(kThreads), st, masks, blk_off, ntiles,
                      state, out_idx, lim, 1);
-  hipLaunchKernelGGL(gd_gather_kernel, dim3(cdiv(lim > 0 ? lim : 1, kThreads)), dim3(kThreads), 0, st, out, r, state, lim,
+  HPX_LAUNCH("gd_gather_kernel", gd_gather_kernel, dim3(cdiv(lim > 0 ? lim : 1, kThreads)), dim3(kThreads), st, out, r, state, lim,
                      -1);
   HPX_HIP(hipGetLastError());
   uint32_t* h_total = reinterpret_cast<uint32_t*>(ws->pinned);
@@ -529,14 +529,14 @@ int gd_encode_one(const float* g, int32_t N, float* r, uint8_t* out, double samp
   int32_t* ia = reinterpret_cast<int32_t*>(base + o_ia);
   int32_t* ib = reinterpret_cast<int32_t*>(base + o_ib);
   uint32_t* sc = reinterpret_cast<uint32_t*>(base + o_sc);
-  hipLaunchKernelGGL(gd_expand_kernel, dim3(cdiv(ntiles, kThreads / kWave)), dim3(kThreads), 0, st, masks, blk_off, ntiles,
+  HPX_LAUNCH("gd_expand_kernel", gd_expand_kernel, dim3(cdiv(ntiles, kThreads / kWave)), dim3(kThreads), st, masks, blk_off, ntiles,
                      state, ia, total, 0);
-  hipLaunchKernelGGL(gd_keys_kernel, dim3(cdiv(total, kThreads)), dim3(kThreads), 0, st, ia, r, total, ka);
+  HPX_LAUNCH("gd_keys_kernel", gd_keys_kernel, dim3(cdiv(total, kThreads)), dim3(kThreads), st, ia, r, total, ka);
   HPX_HIP(hipGetLastError());
   rc = sort_pairs_desc(ka, ia, kb, ib, sc, total, st);
   if (rc != HPX_OK) return rc;
-  if (lim > 0) hipLaunchKernelGGL(gd_copy_idx_kernel, dim3(cdiv(lim, kThreads)), dim3(kThreads), 0, st, ia, out_idx, lim);
-  hipLaunchKernelGGL(gd_gather_kernel, dim3(cdiv(lim > 0 ? lim : 1, kThreads)), dim3(kThreads), 0, st, out, r, state, lim,
+  if (lim > 0) HPX_LAUNCH("gd_copy_idx_kernel", gd_copy_idx_kernel, dim3(cdiv(lim, kThreads)), dim3(kThreads), st, ia, out_idx, lim);
+  HPX_LAUNCH("gd_gather_kernel", gd_gather_kernel, dim3(cdiv(lim > 0 ? lim : 1, kThreads)), dim3(kThreads), st, out, r, state, lim,
                      int32_t(lim));
   HPX_HIP(hipGetLastError());
   return HPX_OK;
@@ -607,11 +607,11 @@ HPX_API int hpx_gd_decode(int count, const uint8_t* const* ins, const int32_t* i
       const uint32_t n = static_cast<uint32_t>(out_sizes[i]);
       if (n) {
         uint32_t blocks = cdiv(n, kThreads * 4);
-        hipLaunchKernelGGL(gd_zero_kernel, dim3(blocks), dim3(kThreads), 0, st, outs[i], n);
+        HPX_LAUNCH("gd_zero_kernel", gd_zero_kernel, dim3(blocks), dim3(kThreads), st, outs[i], n);
       }
-      if (k) hipLaunchKernelGGL(gd_scatter_kernel<false>, dim3(cdiv(k, kThreads)), dim3(kThreads), 0, st, idx, val, k, outs[i]);
+      if (k) HPX_LAUNCH("gd_scatter_kernel", gd_scatter_kernel<false>, dim3(cdiv(k, kThreads)), dim3(kThreads), st, idx, val, k, outs[i]);
     } else if (k) {
-      hipLaunchKernelGGL(gd_scatter_kernel<true>, dim3(cdiv(k, kThreads)), dim3(kThreads), 0, st, idx, val, k, outs[i]);
+      HPX_LAUNCH("gd_scatter_kernel", gd_scatter_kernel<true>, dim3(cdiv(k, kThreads)), dim3(kThreads), st, idx, val, k, outs[i]);
     }
     HPX_HIP(hipGetLastError());
   }

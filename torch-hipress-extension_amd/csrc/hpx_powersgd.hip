@@ -374,10 +374,10 @@ int check_dims(const char* who, const Batch& b, int* max_cg) {
 
 #define PSGD_LAUNCH_CG(KERNEL, cg, grid, st, args)                                              \
   switch (cg) {                                                                                 \
-    case 1: hipLaunchKernelGGL(KERNEL<1>, dim3(grid), dim3(kThreads), 0, st, args); break;      \
-    case 2: hipLaunchKernelGGL(KERNEL<2>, dim3(grid), dim3(kThreads), 0, st, args); break;      \
-    case 3: hipLaunchKernelGGL(KERNEL<3>, dim3(grid), dim3(kThreads), 0, st, args); break;      \
-    default: hipLaunchKernelGGL(KERNEL<4>, dim3(grid), dim3(kThreads), 0, st, args); break;     \
+    case 1: HPX_LAUNCH(#KERNEL, KERNEL<1>, dim3(grid), dim3(kThreads), st, args); break;      \
+    case 2: HPX_LAUNCH(#KERNEL, KERNEL<2>, dim3(grid), dim3(kThreads), st, args); break;      \
+    case 3: HPX_LAUNCH(#KERNEL, KERNEL<3>, dim3(grid), dim3(kThreads), st, args); break;      \
+    default: HPX_LAUNCH(#KERNEL, KERNEL<4>, dim3(grid), dim3(kThreads), st, args); break;     \
   }
 
 }  // namespace
@@ -463,11 +463,11 @@ HPX_API int hpx_powersgd_encode2(int count, float* const* Ps, const float* const
       i++;
     }
     (void)first;
-    hipLaunchKernelGGL(psgd_orth_kernel, dim3(a.nseg), dim3(kOrthThreads), 0, st, a);
+    HPX_LAUNCH("psgd_orth_kernel", psgd_orth_kernel, dim3(a.nseg), dim3(kOrthThreads), st, a);
     PSGD_LAUNCH_CG(psgd_mtp_kernel, cg, a.tile_start[a.nseg], st, a);
     HPX_HIP(hipGetLastError());
     for (int k = 0; k <= a.nseg; k++) a.tile_start[k] = red_start[k];
-    hipLaunchKernelGGL(psgd_qreduce_kernel, dim3(a.tile_start[a.nseg]), dim3(kThreads), 0, st, a);
+    HPX_LAUNCH("psgd_qreduce_kernel", psgd_qreduce_kernel, dim3(a.tile_start[a.nseg]), dim3(kThreads), st, a);
     HPX_HIP(hipGetLastError());
   }
   return HPX_OK;

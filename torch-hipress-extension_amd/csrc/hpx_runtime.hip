@@ -4,7 +4,9 @@
 #include <cstdio>
 #include <map>
 #include <memory>
+#include <cstring>
 #include <utility>
+#include <vector>
 
 #include "hpx_common.h"
 
@@ -59,6 +61,39 @@ int ensure_workspace(Workspace* ws, size_t dev_bytes) {
   return HPX_OK;
 }
 
+// ---- per-kernel timing --------------------------------------------------------
+bool g_prof_on = false;
+namespace {
+struct ProfRec {
+  const char* name;
+  hipEvent_t start, stop;
+};
+std::mutex g_prof_mu;
+std::vector<ProfRec> g_prof_recs;
+std::vector<hipEvent_t> g_prof_pool;
+hipEvent_t prof_event() {
+  if (!g_prof_pool.empty()) {
+    hipEvent_t e = g_prof_pool.back();
+    g_prof_pool.pop_back();
+    return e;
+  }
+  hipEvent_t e = nullptr;
+  (void)hipEventCreate(&e);
+  return e;
+}
+}  // namespace
+
+void prof_begin(const char* name, hipStream_t st) {
+  std::lock_guard<std::mutex> g(g_prof_mu);
+  ProfRec r{name, prof_event(), prof_event()};
+  (void)hipEventRecord(r.start, st);
+  g_prof_recs.push_back(r);
+}
+void prof_end(hipStream_t st) {
+  std::lock_guard<std::mutex> g(g_prof_mu);
+  if (!g_prof_recs.empty()) (void)hipEventRecord(g_prof_recs.back().stop, st);
+}
+
 uint64_t clock_seed() {
   return static_cast<uint64_t>(
       std::chrono::high_resolution_clock::now().time_since_epoch().count());
@@ -86,4 +121,40 @@ HPX_API int hpx_release_workspaces(void) {
   hpx::g_ws.clear();
   if (cur >= 0) (void)hipSetDevice(cur);
   return rc;
+}
+
+HPX_API int hpx_profile_enable(int on) {
+  std::lock_guard<std::mutex> g(hpx::g_prof_mu);
+  hpx::g_prof_on = on != 0;
+  return HPX_OK;
+}
+
+HPX_API int hpx_profile_reset(void) {
+  std::lock_guard<std::mutex> g(hpx::g_prof_mu);
+  for (auto& r : hpx::g_prof_recs) {
+    (void)hipEventSynchronize(r.stop);
+    hpx::g_prof_pool.push_back(r.start);
+    hpx::g_prof_pool.push_back(r.stop);
+  }
+  hpx::g_prof_recs.clear();
+  return HPX_OK;
+}
+
+HPX_API int hpx_profile_query(const char* kernel, double* total_ms, int64_t* launches) {
+  hpx::clear_error();
+  HPX_ARG(kernel && total_ms && launches, "hpx_profile_query: null argument");
+  std::lock_guard<std::mutex> g(hpx::g_prof_mu);
+  double sum = 0;
+  int64_t n = 0;
+  for (auto& r : hpx::g_prof_recs) {
+    if (std::strcmp(r.name, kernel) != 0) continue;
+    HPX_HIP(hipEventSynchronize(r.stop));
+    float ms = 0;
+    HPX_HIP(hipEventElapsedTime(&ms, r.start, r.stop));
+    sum += ms;
+    n++;
+  }
+  *total_ms = sum;
+  *launches = n;
+  return HPX_OK;
 }

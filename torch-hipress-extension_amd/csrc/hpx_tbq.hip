@@ -217,7 +217,7 @@ HPX_API int hpx_tbq_encode(int count, const float* const* grads, const int32_t* 
       i++;
     }
     if (a.nseg == 0) continue;
-    hipLaunchKernelGGL(tbq_encode_kernel, dim3(a.tile_start[a.nseg]), dim3(kThreads), 0, st, a);
+    HPX_LAUNCH("tbq_encode_kernel", tbq_encode_kernel, dim3(a.tile_start[a.nseg]), dim3(kThreads), st, a);
     HPX_HIP(hipGetLastError());
   }
   return HPX_OK;
@@ -250,7 +250,7 @@ HPX_API int hpx_tbq_decode(int count, float* const* outs, const int32_t* sizes,
       i++;
     }
     if (a.nseg == 0) continue;
-    hipLaunchKernelGGL(tbq_decode_kernel, dim3(a.tile_start[a.nseg]), dim3(kThreads), 0, st, a);
+    HPX_LAUNCH("tbq_decode_kernel", tbq_decode_kernel, dim3(a.tile_start[a.nseg]), dim3(kThreads), st, a);
     HPX_HIP(hipGetLastError());
   }
   return HPX_OK;

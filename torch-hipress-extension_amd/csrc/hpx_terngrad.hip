@@ -459,13 +459,13 @@ HPX_API int hpx_terngrad_encode(int count, const float* const* ins, const int32_
       a.nseg++;
       i++;
     }
-    hipLaunchKernelGGL(terngrad_minmax_kernel, dim3(a.tile_start[a.nseg]), dim3(kThreads), 0, st, a);
+    HPX_LAUNCH("terngrad_minmax_kernel", terngrad_minmax_kernel, dim3(a.tile_start[a.nseg]), dim3(kThreads), st, a);
     HPX_HIP(hipGetLastError());
-    hipLaunchKernelGGL(terngrad_finalize_kernel, dim3(a.nseg), dim3(kThreads), 0, st, a);
+    HPX_LAUNCH("terngrad_finalize_kernel", terngrad_finalize_kernel, dim3(a.nseg), dim3(kThreads), st, a);
     HPX_HIP(hipGetLastError());
     part_off += size_t(a.tile_start[a.nseg]);
     for (int k = 0; k <= a.nseg; k++) a.tile_start[k] = qstart[k];
-    hipLaunchKernelGGL(terngrad_quant_kernel, dim3(a.tile_start[a.nseg]), dim3(kThreads), 0, st, a);
+    HPX_LAUNCH("terngrad_quant_kernel", terngrad_quant_kernel, dim3(a.tile_start[a.nseg]), dim3(kThreads), st, a);
     HPX_HIP(hipGetLastError());
   }
   return HPX_OK;
@@ -504,7 +504,7 @@ HPX_API int hpx_terngrad_decode(int count, float* const* outs, const int32_t* ou
       i++;
     }
     if (a.nseg == 0) continue;
-    hipLaunchKernelGGL(terngrad_decode_kernel, dim3(a.tile_start[a.nseg]), dim3(kThreads), 0, st, a);
+    HPX_LAUNCH("terngrad_decode_kernel", terngrad_decode_kernel, dim3(a.tile_start[a.nseg]), dim3(kThreads), st, a);
     HPX_HIP(hipGetLastError());
   }
   return HPX_OK;
