@@ -100,7 +100,7 @@ def test_bucket_of_many_tensors(tbq, oracle_cpu):
     # More tensors than one launch table holds, ragged sizes, per-tensor thresholds,
     # an empty tensor in the middle; two consecutive steps exercise residual feedback.
     rng = np.random.default_rng(1)
-    sizes = [int(s) for s in np.exp(rng.uniform(np.log(3), np.log(60000), 230))]
+    sizes = [int(s) for s in np.exp(rng.uniform(np.log(3), np.log(30000), 600))]
     sizes[17] = 0
     gs = [rng.normal(0, 5e-3, n).astype(np.float32) for n in sizes]
     rs = [np.zeros(n, np.float32) for n in sizes]

@@ -55,7 +55,7 @@ def test_sizes_and_tails(tg, oracle_cpu, b, rnd):
 
 def test_more_tensors_than_one_table(tg, oracle_cpu):
     rng = np.random.default_rng(21)
-    sizes = [int(s) for s in np.exp(rng.uniform(np.log(2), np.log(40000), 150))]
+    sizes = [int(s) for s in np.exp(rng.uniform(np.log(2), np.log(20000), 450))]
     xs = [rng.normal(0, 1e-2, n).astype(np.float32) for n in sizes]
     bws = [int(b) for b in rng.choice([1, 2, 4, 8], len(sizes))]
     rnds = [int(r) for r in rng.integers(0, 2, len(sizes))]

@@ -12,9 +12,9 @@
 //   stream      ONE pass over the tensor: r = g + r, store r, compare with the
 //               threshold, wave64 ballot -> one 64-bit word per 64 elements
 //               (bit i = element i) and a popcount per workgroup
-//   scan        exclusive prefix of the per-workgroup counts
-//   expand      bit words -> ascending indices at the scanned offsets
-//   gather      values out, residual zeroed, header written
+//   scan        two-level exclusive prefix of the per-workgroup counts
+//   expand      bit words -> ascending indices at the scanned offsets, values
+//               out, residual entries zeroed, header written
 //
 // The stream pass moves 12 bytes per element (g, r in; r out) plus 1/8 byte of
 // mask; everything else touches O(sample + selected) data.  The host waits for
@@ -39,8 +39,11 @@ constexpr int kBins1 = 2048, kBins2 = 2048, kBins3 = 1024;  // key = d1:11 | d2:
 struct GdState {
   uint32_t total;     // candidates found by the stream pass
   uint32_t thr_bits;  // threshold as fp32 bits
-  uint32_t pad[62];
+  uint32_t arrive;    // arrival counter of the scan kernel's workgroups
+  uint32_t pad[61];
 };
+constexpr int kScanChunk = 4096;   // per-tile counts scanned by one workgroup
+constexpr int kMaxChunks = 128;    // 2^31 elements / kTile / kScanChunk
 
 struct SelArgs {
   const float* g;
@@ -103,25 +106,34 @@ __device__ __forceinline__ uint32_t sample_index(uint32_t seed, uint32_t x, uint
   return (lcg_mul(2) * (seed + x) + lcg_add(2)) % n;
 }
 
+// One sample per lane: all the random gathers of the sample are in flight at
+// once.  The same launch clears the histograms and the counters of this call.
+__global__ __launch_bounds__(kThreads) void gd_sample_kernel(const SelArgs a) {
+  const uint32_t x = blockIdx.x * kThreads + threadIdx.x;
+  if (x < uint32_t(kBins1 + kBins2 + kBins3)) a.hist[x] = 0;
+  if (x == 0) {
+    a.st->total = 0;
+    a.st->arrive = 0;
+  }
+  if (x < a.sample_cnt) {
+    const uint32_t i = sample_index(a.seed, x, a.n);
+    a.samples[x] = __float_as_uint(__builtin_fabsf(a.g[i] + a.r[i]));
+  }
+}
+
 template <int PASS>
 __device__ __forceinline__ void hist_accumulate(const SelArgs& a, uint32_t* s_hist, uint32_t prefix) {
   // PASS 1: all keys, digit = key >> 21.  PASS 2: keys with key>>21 == prefix,
   // digit = (key >> 10) & 2047.  PASS 3: keys with key>>10 == prefix, digit = key & 1023.
   const uint32_t stride = gridDim.x * kSelThreads;
   for (uint32_t x = blockIdx.x * kSelThreads + threadIdx.x; x < a.sample_cnt; x += stride) {
-    uint32_t key;
+    const uint32_t key = a.samples[x];
     if (PASS == 1) {
-      const uint32_t i = sample_index(a.seed, x, a.n);
-      key = __float_as_uint(__builtin_fabsf(a.g[i] + a.r[i]));
-      a.samples[x] = key;
       atomicAdd(&s_hist[key >> 21], 1u);
+    } else if (PASS == 2) {
+      if ((key >> 21) == prefix) atomicAdd(&s_hist[(key >> 10) & 2047u], 1u);
     } else {
-      key = a.samples[x];
-      if (PASS == 2) {
-        if ((key >> 21) == prefix) atomicAdd(&s_hist[(key >> 10) & 2047u], 1u);
-      } else {
-        if ((key >> 10) == prefix) atomicAdd(&s_hist[key & 1023u], 1u);
-      }
+      if ((key >> 10) == prefix) atomicAdd(&s_hist[key & 1023u], 1u);
     }
   }
 }
@@ -213,41 +225,85 @@ __global__ __launch_bounds__(kThreads) void gd_stream_kernel(const float* __rest
   if (threadIdx.x == 0) blk_counts[blockIdx.x] = s_cnt[0] + s_cnt[1] + s_cnt[2] + s_cnt[3];
 }
 
-// Exclusive prefix of `cnt[0..n)` into `off`, grand total into *total.
+// Exclusive prefix of the per-tile counts, two levels.  Workgroup c scans counts
+// [c*4096, (c+1)*4096) into `off` (relative to its chunk) and publishes the chunk
+// total; the last workgroup to arrive (at most 128 of them, so the shared
+// counter costs microseconds at worst) turns the totals into chunk offsets and
+// the grand total.
 __global__ __launch_bounds__(kSelThreads) void gd_scan_kernel(const uint32_t* __restrict__ cnt, uint32_t* __restrict__ off,
-                                                              uint32_t n, uint32_t* __restrict__ total) {
-  __shared__ uint32_t s_scan[kSelThreads];
-  const uint32_t t = threadIdx.x;
-  const uint32_t per = (n + kSelThreads - 1) / kSelThreads;
-  const uint32_t b = t * per, e = (b + per < n) ? b + per : n;
-  uint32_t sum = 0;
-  for (uint32_t i = b; i < e; i++) sum += cnt[i];
-  s_scan[t] = sum;
+                                                              uint32_t n, uint32_t* __restrict__ chunk_tot,
+                                                              uint32_t* __restrict__ chunk_off, GdState* __restrict__ st) {
+  __shared__ uint32_t s_wave[kSelThreads / kWave];
+  __shared__ uint32_t s_last;
+  const uint32_t t = threadIdx.x, lane = t & (kWave - 1), wave = t / kWave;
+  const uint32_t i0 = blockIdx.x * uint32_t(kScanChunk) + t * 4;
+  uint32_t c[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) c[j] = (i0 + j < n) ? cnt[i0 + j] : 0u;
+  const uint32_t sum = c[0] + c[1] + c[2] + c[3];
+  uint32_t incl = sum;
+#pragma unroll
+  for (int o = 1; o < kWave; o <<= 1) {
+    const uint32_t v = __shfl_up(incl, o, kWave);
+    if (lane >= uint32_t(o)) incl += v;
+  }
+  if (lane == kWave - 1) s_wave[wave] = incl;
   __syncthreads();
-  for (int o = 1; o < kSelThreads; o <<= 1) {
-    const uint32_t v = t >= uint32_t(o) ? s_scan[t - o] : 0u;
-    __syncthreads();
-    s_scan[t] += v;
-    __syncthreads();
+  uint32_t before = 0, all = 0;
+#pragma unroll
+  for (uint32_t w = 0; w < kSelThreads / kWave; w++) {
+    const uint32_t v = s_wave[w];
+    if (w < wave) before += v;
+    all += v;
   }
-  uint32_t run = s_scan[t] - sum;
-  for (uint32_t i = b; i < e; i++) {
-    const uint32_t c = cnt[i];
-    off[i] = run;
-    run += c;
+  uint32_t run = before + incl - sum;
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    if (i0 + j < n) off[i0 + j] = run;
+    run += c[j];
   }
-  if (t == kSelThreads - 1) *total = s_scan[t];
+  if (t == 0) {
+    chunk_tot[blockIdx.x] = all;
+    __threadfence();
+    s_last = (atomicAdd(&st->arrive, 1u) == gridDim.x - 1);
+  }
+  __syncthreads();
+  if (!s_last) return;
+  __threadfence();
+  if (t < kWave) {
+    // up to 128 chunk totals: two per lane
+    const uint32_t a0 = (2 * t < gridDim.x) ? __hip_atomic_load(&chunk_tot[2 * t], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+    const uint32_t a1 = (2 * t + 1 < gridDim.x) ? __hip_atomic_load(&chunk_tot[2 * t + 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+    uint32_t inc2 = a0 + a1;
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+      const uint32_t v = __shfl_up(inc2, o, kWave);
+      if (t >= uint32_t(o)) inc2 += v;
+    }
+    const uint32_t ex = inc2 - a0 - a1;
+    if (2 * t < gridDim.x) chunk_off[2 * t] = ex;
+    if (2 * t + 1 < gridDim.x) chunk_off[2 * t + 1] = ex + a0;
+    if (t == kWave - 1) st->total = inc2;
+  }
 }
 
-// One wave per stream tile: 64 mask words -> ascending indices.
-// only_if_fits != 0: do nothing when the stream pass found more than `limit`.
+// One wave per stream tile: 64 mask words -> ascending indices at the scanned
+// offsets.  With `out` set this is the common-case finish (gd_body.h:193-229):
+// nothing happens if the stream pass found more than `limit` candidates,
+// otherwise indices, values and header are written and the residual entries are
+// cleared.  With `out` null the indices go to `dst` (the candidate list of the
+// cut path) and nothing else is touched.
 __global__ __launch_bounds__(kThreads) void gd_expand_kernel(const uint64_t* __restrict__ masks,
-                                                             const uint32_t* __restrict__ blk_off, uint32_t ntiles,
+                                                             const uint32_t* __restrict__ tile_off,
+                                                             const uint32_t* __restrict__ chunk_off, uint32_t ntiles,
                                                              const GdState* __restrict__ st, int32_t* __restrict__ dst,
-                                                             uint32_t limit, int only_if_fits) {
-  if (only_if_fits && st->total > limit) return;
+                                                             uint32_t limit, uint8_t* __restrict__ out,
+                                                             float* __restrict__ r) {
+  const uint32_t total = st->total;
+  if (out && total > limit) return;
   const uint32_t lane = threadIdx.x & (kWave - 1);
   const uint32_t tile = blockIdx.x * (kThreads / kWave) + threadIdx.x / kWave;
+  if (out && tile == 0 && lane == 0) *reinterpret_cast<int32_t*>(out) = int32_t(4 + total * 8);
   if (tile >= ntiles) return;
   uint64_t m = masks[size_t(tile) * kWave + lane];
   const uint32_t c = __popcll(m);
@@ -257,28 +313,27 @@ __global__ __launch_bounds__(kThreads) void gd_expand_kernel(const uint64_t* __r
     const uint32_t v = __shfl_up(incl, o, kWave);
     if (lane >= uint32_t(o)) incl += v;
   }
-  uint32_t pos = blk_off[tile] + incl - c;
+  uint32_t pos = chunk_off[tile / kScanChunk] + tile_off[tile] + incl - c;
   const uint32_t e0 = tile * uint32_t(kTile) + lane * kWave;
+  int32_t* idx = out ? reinterpret_cast<int32_t*>(out + 4) : dst;
+  float* val = out ? reinterpret_cast<float*>(out + 4 + size_t(total) * 4) : nullptr;
   while (m) {
-    const uint32_t b = __builtin_ctzll(m);
+    const uint32_t e = e0 + uint32_t(__builtin_ctzll(m));
     m &= m - 1;
-    if (pos < limit) dst[pos] = int32_t(e0 + b);
+    if (pos < limit) {
+      idx[pos] = int32_t(e);
+      if (out) {
+        val[pos] = r[e];
+        r[e] = 0.0f;
+      }
+    }
     pos++;
   }
 }
 
-// generate_S_value, gd_body.h:80-99, plus the header (gd_body.h:193-201).
-// k_host < 0: k is the stream pass's total, and nothing happens if it exceeds `limit`.
-__global__ __launch_bounds__(kThreads) void gd_gather_kernel(uint8_t* __restrict__ out, float* __restrict__ r,
-                                                             const GdState* __restrict__ st, uint32_t limit,
-                                                             int32_t k_host) {
-  uint32_t k;
-  if (k_host < 0) {
-    k = st->total;
-    if (k > limit) return;
-  } else {
-    k = uint32_t(k_host);
-  }
+// generate_S_value, gd_body.h:80-99, plus the header (gd_body.h:193-201), for a
+// list of k indices already in place (the cut path).
+__global__ __launch_bounds__(kThreads) void gd_gather_kernel(uint8_t* __restrict__ out, float* __restrict__ r, uint32_t k) {
   const int32_t* idx = reinterpret_cast<const int32_t*>(out + 4);
   float* val = reinterpret_cast<float*>(out + 4 + size_t(k) * 4);
   const uint32_t x = blockIdx.x * kThreads + threadIdx.x;
@@ -451,11 +506,12 @@ int gd_encode_one(const float* g, int32_t N, float* r, uint8_t* out, double samp
   size_t off = 0;
   const size_t o_state = off; off += align256(sizeof(GdState));
   const size_t o_hist = off;  off += align256(sizeof(uint32_t) * (kBins1 + kBins2 + kBins3));
-  const size_t zero_bytes = off;  // state + histograms start at zero
   const size_t o_samples = off; off += align256(sizeof(uint32_t) * size_t(sample_cnt));
   const size_t o_masks = off; off += align256(sizeof(uint64_t) * size_t(ntiles) * kWave);
   const size_t o_cnt = off; off += align256(sizeof(uint32_t) * size_t(ntiles));
   const size_t o_off = off; off += align256(sizeof(uint32_t) * size_t(ntiles));
+  const size_t o_ctot = off; off += align256(sizeof(uint32_t) * kMaxChunks);
+  const size_t o_coff = off; off += align256(sizeof(uint32_t) * kMaxChunks);
   // Room for the cut path (sorted copies of the candidates) is reserved for a
   // typical overshoot so that path normally needs no reallocation.
   uint64_t cap = uint64_t(expected) * 2 > uint64_t(expected) + 65536 ? uint64_t(expected) * 2 : uint64_t(expected) + 65536;
@@ -472,26 +528,30 @@ int gd_encode_one(const float* g, int32_t N, float* r, uint8_t* out, double samp
   uint64_t* masks = reinterpret_cast<uint64_t*>(base + o_masks);
   uint32_t* blk_cnt = reinterpret_cast<uint32_t*>(base + o_cnt);
   uint32_t* blk_off = reinterpret_cast<uint32_t*>(base + o_off);
+  uint32_t* chunk_tot = reinterpret_cast<uint32_t*>(base + o_ctot);
+  uint32_t* chunk_off = reinterpret_cast<uint32_t*>(base + o_coff);
+  const uint32_t nchunks = cdiv(ntiles, kScanChunk);
 
-  HPX_HIP(hipMemsetAsync(base, 0, zero_bytes, st));
   SelArgs sa{g, r, n, static_cast<uint32_t>(sample_cnt), static_cast<uint32_t>(seed), static_cast<uint32_t>(thr_index),
              samples, hist, state};
   uint32_t sel_blocks = cdiv(sample_cnt, kSelThreads * 8);
   if (sel_blocks > kSelBlocksMax) sel_blocks = kSelBlocksMax;
+  const uint32_t zero_words = kBins1 + kBins2 + kBins3;
+  HPX_LAUNCH("gd_sample_kernel", gd_sample_kernel,
+             dim3(cdiv(uint32_t(sample_cnt) > zero_words ? uint32_t(sample_cnt) : zero_words, kThreads)), dim3(kThreads), st, sa);
   HPX_LAUNCH("gd_select_kernel", gd_select_kernel<1>, dim3(sel_blocks), dim3(kSelThreads), st, sa);
   HPX_LAUNCH("gd_select_kernel", gd_select_kernel<2>, dim3(sel_blocks), dim3(kSelThreads), st, sa);
   HPX_LAUNCH("gd_select_kernel", gd_select_kernel<3>, dim3(sel_blocks), dim3(kSelThreads), st, sa);
   HPX_LAUNCH("gd_threshold_kernel", gd_threshold_kernel, dim3(1), dim3(kSelThreads), st, sa);
   HPX_LAUNCH("gd_stream_kernel", gd_stream_kernel, dim3(ntiles), dim3(kThreads), st, g, r, n, state, masks, blk_cnt);
-  HPX_LAUNCH("gd_scan_kernel", gd_scan_kernel, dim3(1), dim3(kSelThreads), st, blk_cnt, blk_off, ntiles, &state->total);
+  HPX_LAUNCH("gd_scan_kernel", gd_scan_kernel, dim3(nchunks), dim3(kSelThreads), st, blk_cnt, blk_off, ntiles, chunk_tot,
+             chunk_off, state);
   HPX_HIP(hipGetLastError());
   // Common case (nothing to cut) queued before the host knows the count.
   int32_t* out_idx = reinterpret_cast<int32_t*>(out + 4);
   const uint32_t lim = static_cast<uint32_t>(expected);
-  HPX_LAUNCH("gd_expand_kernel", gd_expand_kernel, dim3(cdiv(ntiles, kThreads / kWave)), dim3(kThreads), st, masks, blk_off, ntiles,
-                     state, out_idx, lim, 1);
-  HPX_LAUNCH("gd_gather_kernel", gd_gather_kernel, dim3(cdiv(lim > 0 ? lim : 1, kThreads)), dim3(kThreads), st, out, r, state, lim,
-                     -1);
+  HPX_LAUNCH("gd_expand_kernel", gd_expand_kernel, dim3(cdiv(ntiles, kThreads / kWave)), dim3(kThreads), st, masks, blk_off,
+             chunk_off, ntiles, state, out_idx, lim, out, r);
   HPX_HIP(hipGetLastError());
   uint32_t* h_total = reinterpret_cast<uint32_t*>(ws->pinned);
   HPX_HIP(hipMemcpyAsync(h_total, &state->total, sizeof(uint32_t), hipMemcpyDeviceToHost, st));
@@ -523,21 +583,21 @@ int gd_encode_one(const float* g, int32_t N, float* r, uint8_t* out, double samp
     state = reinterpret_cast<GdState*>(base + o_state);
     masks = reinterpret_cast<uint64_t*>(base + o_masks);
     blk_off = reinterpret_cast<uint32_t*>(base + o_off);
+    chunk_off = reinterpret_cast<uint32_t*>(base + o_coff);
   }
   uint32_t* ka = reinterpret_cast<uint32_t*>(base + o_ka);
   uint32_t* kb = reinterpret_cast<uint32_t*>(base + o_kb);
   int32_t* ia = reinterpret_cast<int32_t*>(base + o_ia);
   int32_t* ib = reinterpret_cast<int32_t*>(base + o_ib);
   uint32_t* sc = reinterpret_cast<uint32_t*>(base + o_sc);
-  HPX_LAUNCH("gd_expand_kernel", gd_expand_kernel, dim3(cdiv(ntiles, kThreads / kWave)), dim3(kThreads), st, masks, blk_off, ntiles,
-                     state, ia, total, 0);
+  HPX_LAUNCH("gd_expand_kernel", gd_expand_kernel, dim3(cdiv(ntiles, kThreads / kWave)), dim3(kThreads), st, masks, blk_off,
+             chunk_off, ntiles, state, ia, total, static_cast<uint8_t*>(nullptr), static_cast<float*>(nullptr));
   HPX_LAUNCH("gd_keys_kernel", gd_keys_kernel, dim3(cdiv(total, kThreads)), dim3(kThreads), st, ia, r, total, ka);
   HPX_HIP(hipGetLastError());
   rc = sort_pairs_desc(ka, ia, kb, ib, sc, total, st);
   if (rc != HPX_OK) return rc;
   if (lim > 0) HPX_LAUNCH("gd_copy_idx_kernel", gd_copy_idx_kernel, dim3(cdiv(lim, kThreads)), dim3(kThreads), st, ia, out_idx, lim);
-  HPX_LAUNCH("gd_gather_kernel", gd_gather_kernel, dim3(cdiv(lim > 0 ? lim : 1, kThreads)), dim3(kThreads), st, out, r, state, lim,
-                     int32_t(lim));
+  HPX_LAUNCH("gd_gather_kernel", gd_gather_kernel, dim3(cdiv(lim > 0 ? lim : 1, kThreads)), dim3(kThreads), st, out, r, lim);
   HPX_HIP(hipGetLastError());
   return HPX_OK;
 }

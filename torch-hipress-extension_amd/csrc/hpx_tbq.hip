@@ -16,7 +16,7 @@ using namespace hpx;
 constexpr int kThreads = 256;
 constexpr int kIters = 4;                           // groups per lane
 constexpr int kTileGroups = kThreads * kIters;      // 1024 bytes of codes
-constexpr int kMaxSeg = 96;                         // table must fit 4 KiB of kernargs
+constexpr int kMaxSeg = 256;                        // 9 KiB of kernel arguments: a 200-tensor bucket is one launch
 
 struct EncSeg {
   const float* g;
@@ -43,7 +43,7 @@ struct DecArgs {
   int32_t tile_start[kMaxSeg + 1];
   DecSeg seg[kMaxSeg];
 };
-static_assert(sizeof(EncArgs) <= 4096 && sizeof(DecArgs) <= 4096, "kernarg limit");
+static_assert(sizeof(EncArgs) <= 9600 && sizeof(DecArgs) <= 9600, "kernel-argument budget");
 
 // One element of the reference rule; returns the 2-bit code.
 __device__ __forceinline__ uint32_t tbq_code(float g, float& r, float thr) {

@@ -27,7 +27,7 @@ namespace {
 using namespace hpx;
 
 constexpr int kThreads = 256;
-constexpr int kMaxSeg = 64;
+constexpr int kMaxSeg = 192;
 constexpr int kRedIters = 8;                                 // float4 loads per lane
 constexpr int kRedTile = kThreads * kRedIters * 4;           // 8192 elements
 constexpr int kQIters = 4;                                   // units per lane
@@ -72,7 +72,7 @@ struct DecArgs {
   DecSeg seg[kMaxSeg];
   uint32_t* status;
 };
-static_assert(sizeof(EncArgs) <= 4096 && sizeof(DecArgs) <= 4096, "kernarg limit");
+static_assert(sizeof(EncArgs) <= 9600 && sizeof(DecArgs) <= 9600, "kernel-argument budget");
 
 __device__ __forceinline__ float wave_min(float v) {
 #pragma unroll
@@ -156,6 +156,7 @@ __global__ __launch_bounds__(kThreads) void terngrad_finalize_kernel(const EncAr
   const Partial* pp = a.partials + a.tile_start[s];
   mn = __builtin_inff(); mx = -__builtin_inff();
   uint32_t first_zero_tile = 0xFFFFFFFFu;
+#pragma unroll 4
   for (int i = threadIdx.x; i < ntiles; i += kThreads) {
     const float pmn = pp[i].mn, pmx = pp[i].mx;
     const uint32_t hz = pp[i].has_zero;
