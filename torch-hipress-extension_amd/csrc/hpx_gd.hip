@@ -190,13 +190,13 @@ __global__ __launch_bounds__(kThreads) void gd_stream_kernel(const float* __rest
     float gv[kPerLane], rv[kPerLane];
 #pragma unroll
     for (int c = 0; c < kPerLane; c++) {
-      gv[c] = g[size_t(wbase) + c * kWave + lane];
-      rv[c] = r[size_t(wbase) + c * kWave + lane];
+      gv[c] = __builtin_nontemporal_load(g + size_t(wbase) + c * kWave + lane);
+      rv[c] = __builtin_nontemporal_load(r + size_t(wbase) + c * kWave + lane);
     }
 #pragma unroll
     for (int c = 0; c < kPerLane; c++) {
       const float x = gv[c] + rv[c];  // thrust::plus<float>()(G, R), gd_body.h:121-128
-      r[size_t(wbase) + c * kWave + lane] = x;
+      __builtin_nontemporal_store(x, r + size_t(wbase) + c * kWave + lane);
       const uint64_t m = __ballot((x > thr) || (x < nthr));  // gd_body.h:59-67
       cnt += __popcll(m);
       lo = lane == uint32_t(c) ? uint32_t(m) : lo;  // lane c keeps mask word c

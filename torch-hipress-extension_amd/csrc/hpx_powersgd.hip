@@ -89,7 +89,7 @@ __global__ __launch_bounds__(kThreads) void psgd_encode1_kernel(const Args a) {
     float v[4];
     if (rows_full && k0 + 64 <= m) {
       const int64_t f = int64_t(row) * m + kk;
-      const float4 g4 = ld4(G + f), r4 = ld4(R + f);
+      const float4 g4 = ld4_stream(G + f), r4 = ld4_stream(R + f);
       const float4 m4 = make_float4(g4.x + r4.x, g4.y + r4.y, g4.z + r4.z, g4.w + r4.w);
       st4(M + f, m4);
       v[0] = m4.x; v[1] = m4.y; v[2] = m4.z; v[3] = m4.w;
@@ -227,7 +227,7 @@ __global__ __launch_bounds__(kThreads) void psgd_mtp_kernel(const Args a) {
   for (int row = rbeg; row < rend; row++) {
     float v[4];
     if (cols_full) {
-      const float4 m4 = ld4(M + int64_t(row) * m + kk);
+      const float4 m4 = ld4_stream(M + int64_t(row) * m + kk);
       v[0] = m4.x; v[1] = m4.y; v[2] = m4.z; v[3] = m4.w;
     } else {
 #pragma unroll
@@ -331,9 +331,9 @@ __global__ __launch_bounds__(kThreads) void psgd_decode_kernel(const Args a) {
       const int64_t f = int64_t(row) * m + kk;
       const float4 m4 = make_float4(acc[0][ii], acc[1][ii], acc[2][ii], acc[3][ii]);
       if (cols_full && f + 4 <= N) {
-        const float4 g4 = ld4(G + f);
-        st4(R + f, make_float4(g4.x - m4.x, g4.y - m4.y, g4.z - m4.z, g4.w - m4.w));
-        st4(G + f, m4);
+        const float4 g4 = ld4_stream(G + f);
+        st4_stream(R + f, make_float4(g4.x - m4.x, g4.y - m4.y, g4.z - m4.z, g4.w - m4.w));
+        st4_stream(G + f, m4);
         st4(M + f, m4);
       } else {
         const float mv[4] = {m4.x, m4.y, m4.z, m4.w};

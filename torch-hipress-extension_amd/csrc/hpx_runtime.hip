@@ -4,6 +4,7 @@
 #include <cstdio>
 #include <map>
 #include <memory>
+#include <cstdlib>
 #include <cstring>
 #include <utility>
 #include <vector>
@@ -92,6 +93,14 @@ void prof_begin(const char* name, hipStream_t st) {
 void prof_end(hipStream_t st) {
   std::lock_guard<std::mutex> g(g_prof_mu);
   if (!g_prof_recs.empty()) (void)hipEventRecord(g_prof_recs.back().stop, st);
+}
+
+size_t stream_store_max_bytes() {
+  static const size_t v = [] {
+    const char* e = std::getenv("HPX_STREAM_STORE_MAX_MB");
+    return e ? size_t(std::strtoull(e, nullptr, 10)) << 20 : kStreamStoreMaxBytes;
+  }();
+  return v;
 }
 
 uint64_t clock_seed() {

@@ -16,7 +16,8 @@ using namespace hpx;
 constexpr int kThreads = 256;
 constexpr int kIters = 4;                           // groups per lane
 constexpr int kTileGroups = kThreads * kIters;      // 1024 bytes of codes
-constexpr int kMaxSeg = 256;                        // 9 KiB of kernel arguments: a 200-tensor bucket is one launch
+constexpr int kCapLarge = 256;  // 9 KiB of kernel arguments: a 200-tensor bucket is one launch
+constexpr int kCapSmall = 8;    // calls with a few tensors pass a table of a few hundred bytes
 
 struct EncSeg {
   const float* g;
@@ -25,10 +26,11 @@ struct EncSeg {
   int32_t n;
   float thr;
 };
+template <int CAP>
 struct EncArgs {
   int32_t nseg;
-  int32_t tile_start[kMaxSeg + 1];
-  EncSeg seg[kMaxSeg];
+  int32_t tile_start[CAP + 1];
+  EncSeg seg[CAP];
 };
 struct DecSeg {
   float* out;
@@ -38,12 +40,14 @@ struct DecSeg {
   int32_t add;
   int32_t pad;
 };
+template <int CAP>
 struct DecArgs {
   int32_t nseg;
-  int32_t tile_start[kMaxSeg + 1];
-  DecSeg seg[kMaxSeg];
+  int32_t stream_store;  // see kStreamStoreMaxBytes
+  int32_t tile_start[CAP + 1];
+  DecSeg seg[CAP];
 };
-static_assert(sizeof(EncArgs) <= 9600 && sizeof(DecArgs) <= 9600, "kernel-argument budget");
+static_assert(sizeof(EncArgs<kCapLarge>) <= 9600 && sizeof(DecArgs<kCapLarge>) <= 9600, "kernel-argument budget");
 
 // One element of the reference rule; returns the 2-bit code.
 __device__ __forceinline__ uint32_t tbq_code(float g, float& r, float thr) {
@@ -67,9 +71,10 @@ __device__ __forceinline__ uint32_t tbq_code4(const float4& g, float4& r, float 
   return q;
 }
 
-__global__ __launch_bounds__(kThreads) void tbq_encode_kernel(const EncArgs a) {
+template <int CAP>
+__global__ __launch_bounds__(kThreads) void tbq_encode_kernel(const EncArgs<CAP> a) {
   const int tile = blockIdx.x;
-  const int s = find_segment<kMaxSeg>(a.tile_start, a.nseg, tile);
+  const int s = find_segment<CAP>(a.tile_start, a.nseg, tile);
   const float* __restrict__ gp = a.seg[s].g;
   float* __restrict__ rp = a.seg[s].r;
   uint8_t* __restrict__ op = a.seg[s].out;
@@ -83,14 +88,14 @@ __global__ __launch_bounds__(kThreads) void tbq_encode_kernel(const EncArgs a) {
 #pragma unroll
     for (int k = 0; k < kIters; k++) {
       const size_t e = size_t(g0 + k * kThreads) * 4;
-      gv[k] = ld4(gp + e);
-      rv[k] = ld4(rp + e);
+      gv[k] = ld4_stream(gp + e);
+      rv[k] = ld4_stream(rp + e);
     }
 #pragma unroll
     for (int k = 0; k < kIters; k++) {
       const uint32_t grp = g0 + k * kThreads;
       const uint32_t q = tbq_code4(gv[k], rv[k], thr);
-      st4(rp + size_t(grp) * 4, rv[k]);
+      st4_stream(rp + size_t(grp) * 4, rv[k]);
       op[grp] = static_cast<uint8_t>(q);
     }
     return;
@@ -126,7 +131,7 @@ __device__ __forceinline__ float4 tbq_values(uint32_t q, float thr) {
 }
 
 template <bool ADD>
-__device__ __forceinline__ void tbq_decode_tile(const DecSeg& sg, uint32_t g0) {
+__device__ __forceinline__ void tbq_decode_tile(const DecSeg& sg, uint32_t g0, bool stream_store) {
   float* __restrict__ op = sg.out;
   const uint8_t* __restrict__ ip = sg.in;
   const uint32_t n = static_cast<uint32_t>(sg.n);
@@ -139,7 +144,7 @@ __device__ __forceinline__ void tbq_decode_tile(const DecSeg& sg, uint32_t g0) {
     for (int k = 0; k < kIters; k++) {
       const uint32_t grp = g0 + k * kThreads;
       q[k] = ip[grp];
-      if (ADD) acc[k] = ld4(op + size_t(grp) * 4);
+      if (ADD) acc[k] = ld4_stream(op + size_t(grp) * 4);
     }
 #pragma unroll
     for (int k = 0; k < kIters; k++) {
@@ -147,8 +152,12 @@ __device__ __forceinline__ void tbq_decode_tile(const DecSeg& sg, uint32_t g0) {
       float4 v = tbq_values(q[k], thr);
       if (ADD) {
         v.x += acc[k].x; v.y += acc[k].y; v.z += acc[k].z; v.w += acc[k].w;
+        st4_stream(op + size_t(grp) * 4, v);  // in-place update: streaming store
+      } else if (stream_store) {
+        st4_stream(op + size_t(grp) * 4, v);
+      } else {
+        st4(op + size_t(grp) * 4, v);
       }
-      st4(op + size_t(grp) * 4, v);
     }
     return;
   }
@@ -173,14 +182,15 @@ __device__ __forceinline__ void tbq_decode_tile(const DecSeg& sg, uint32_t g0) {
   }
 }
 
-__global__ __launch_bounds__(kThreads) void tbq_decode_kernel(const DecArgs a) {
+template <int CAP>
+__global__ __launch_bounds__(kThreads) void tbq_decode_kernel(const DecArgs<CAP> a) {
   const int tile = blockIdx.x;
-  const int s = find_segment<kMaxSeg>(a.tile_start, a.nseg, tile);
+  const int s = find_segment<CAP>(a.tile_start, a.nseg, tile);
   const uint32_t g0 = static_cast<uint32_t>(tile - a.tile_start[s]) * kTileGroups + threadIdx.x;
   if (a.seg[s].add)
-    tbq_decode_tile<true>(a.seg[s], g0);
+    tbq_decode_tile<true>(a.seg[s], g0, true);
   else
-    tbq_decode_tile<false>(a.seg[s], g0);
+    tbq_decode_tile<false>(a.seg[s], g0, a.stream_store != 0);
 }
 
 inline int32_t tiles_for(int32_t n) {
@@ -188,22 +198,15 @@ inline int32_t tiles_for(int32_t n) {
   return static_cast<int32_t>((groups + kTileGroups - 1) / kTileGroups);
 }
 
-}  // namespace
-
-HPX_API int hpx_tbq_encode(int count, const float* const* grads, const int32_t* sizes,
-                           float* const* residuals, uint8_t* const* outs, const float* thresholds,
-                           hpx_stream_t stream) {
-  hpx::clear_error();
-  HPX_ARG(count >= 0, "hpx_tbq_encode: negative count");
-  if (count == 0) return HPX_OK;
-  HPX_ARG(grads && sizes && residuals && outs && thresholds, "hpx_tbq_encode: null argument array");
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  EncArgs a;
+template <int CAP>
+int launch_encode(int count, const float* const* grads, const int32_t* sizes, float* const* residuals,
+                  uint8_t* const* outs, const float* thresholds, hipStream_t st) {
+  EncArgs<CAP> a;
   int i = 0;
   while (i < count) {
     a.nseg = 0;
     a.tile_start[0] = 0;
-    while (i < count && a.nseg < kMaxSeg) {
+    while (i < count && a.nseg < CAP) {
       const int32_t n = sizes[i];
       HPX_ARG(n >= 0, "hpx_tbq_encode: tensor %d has negative size %d", i, n);
       if (n > 0) {
@@ -217,26 +220,24 @@ HPX_API int hpx_tbq_encode(int count, const float* const* grads, const int32_t* 
       i++;
     }
     if (a.nseg == 0) continue;
-    HPX_LAUNCH("tbq_encode_kernel", tbq_encode_kernel, dim3(a.tile_start[a.nseg]), dim3(kThreads), st, a);
+    HPX_LAUNCH("tbq_encode_kernel", tbq_encode_kernel<CAP>, dim3(a.tile_start[a.nseg]), dim3(kThreads), st, a);
     HPX_HIP(hipGetLastError());
   }
   return HPX_OK;
 }
 
-HPX_API int hpx_tbq_decode(int count, float* const* outs, const int32_t* sizes,
-                           const uint8_t* const* ins, const float* thresholds,
-                           const int32_t* is_add_tos, hpx_stream_t stream) {
-  hpx::clear_error();
-  HPX_ARG(count >= 0, "hpx_tbq_decode: negative count");
-  if (count == 0) return HPX_OK;
-  HPX_ARG(outs && sizes && ins && thresholds && is_add_tos, "hpx_tbq_decode: null argument array");
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  DecArgs a;
+template <int CAP>
+int launch_decode(int count, float* const* outs, const int32_t* sizes, const uint8_t* const* ins,
+                  const float* thresholds, const int32_t* is_add_tos, hipStream_t st) {
+  DecArgs<CAP> a;
+  size_t out_bytes = 0;
+  for (int k = 0; k < count; k++) out_bytes += sizes[k] > 0 ? size_t(sizes[k]) * 4 : 0;
+  a.stream_store = out_bytes <= hpx::stream_store_max_bytes();
   int i = 0;
   while (i < count) {
     a.nseg = 0;
     a.tile_start[0] = 0;
-    while (i < count && a.nseg < kMaxSeg) {
+    while (i < count && a.nseg < CAP) {
       const int32_t n = sizes[i];
       HPX_ARG(n >= 0, "hpx_tbq_decode: tensor %d has negative size %d", i, n);
       if (n > 0) {
@@ -250,8 +251,34 @@ HPX_API int hpx_tbq_decode(int count, float* const* outs, const int32_t* sizes,
       i++;
     }
     if (a.nseg == 0) continue;
-    HPX_LAUNCH("tbq_decode_kernel", tbq_decode_kernel, dim3(a.tile_start[a.nseg]), dim3(kThreads), st, a);
+    HPX_LAUNCH("tbq_decode_kernel", tbq_decode_kernel<CAP>, dim3(a.tile_start[a.nseg]), dim3(kThreads), st, a);
     HPX_HIP(hipGetLastError());
   }
   return HPX_OK;
+}
+
+}  // namespace
+
+HPX_API int hpx_tbq_encode(int count, const float* const* grads, const int32_t* sizes,
+                           float* const* residuals, uint8_t* const* outs, const float* thresholds,
+                           hpx_stream_t stream) {
+  hpx::clear_error();
+  HPX_ARG(count >= 0, "hpx_tbq_encode: negative count");
+  if (count == 0) return HPX_OK;
+  HPX_ARG(grads && sizes && residuals && outs && thresholds, "hpx_tbq_encode: null argument array");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (count <= kCapSmall) return launch_encode<kCapSmall>(count, grads, sizes, residuals, outs, thresholds, st);
+  return launch_encode<kCapLarge>(count, grads, sizes, residuals, outs, thresholds, st);
+}
+
+HPX_API int hpx_tbq_decode(int count, float* const* outs, const int32_t* sizes,
+                           const uint8_t* const* ins, const float* thresholds,
+                           const int32_t* is_add_tos, hpx_stream_t stream) {
+  hpx::clear_error();
+  HPX_ARG(count >= 0, "hpx_tbq_decode: negative count");
+  if (count == 0) return HPX_OK;
+  HPX_ARG(outs && sizes && ins && thresholds && is_add_tos, "hpx_tbq_decode: null argument array");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (count <= kCapSmall) return launch_decode<kCapSmall>(count, outs, sizes, ins, thresholds, is_add_tos, st);
+  return launch_decode<kCapLarge>(count, outs, sizes, ins, thresholds, is_add_tos, st);
 }

@@ -27,11 +27,13 @@ namespace {
 using namespace hpx;
 
 constexpr int kThreads = 256;
-constexpr int kMaxSeg = 192;
+constexpr int kCapLarge = 192;  // tensors per launch table (about 7 KiB of kernel arguments)
+constexpr int kCapSmall = 8;    // calls with a few tensors pass a table of a few hundred bytes
 constexpr int kRedIters = 8;                                 // float4 loads per lane
 constexpr int kRedTile = kThreads * kRedIters * 4;           // 8192 elements
 constexpr int kQIters = 4;                                   // units per lane
-constexpr int kDecTile = kThreads * kQIters * 4;             // 4096 elements
+constexpr int kDIters = 4;                                   // 4-element groups per lane in decode
+constexpr int kDecTile = kThreads * kDIters * 4;
 
 struct Partial {
   float mn, mx;
@@ -51,10 +53,11 @@ struct EncSeg {
   uint8_t random;
   uint16_t pad;
 };
+template <int CAP>
 struct EncArgs {
   int32_t nseg;
-  int32_t tile_start[kMaxSeg + 1];
-  EncSeg seg[kMaxSeg];
+  int32_t tile_start[CAP + 1];
+  EncSeg seg[CAP];
   Partial* partials;    // one per reduction tile of this launch
   Scalars* scalars;     // one per segment
 };
@@ -66,13 +69,15 @@ struct DecSeg {
   int32_t add;
   int32_t pad;
 };
+template <int CAP>
 struct DecArgs {
   int32_t nseg;
-  int32_t tile_start[kMaxSeg + 1];
-  DecSeg seg[kMaxSeg];
+  int32_t stream_store;  // see kStreamStoreMaxBytes
+  int32_t tile_start[CAP + 1];
+  DecSeg seg[CAP];
   uint32_t* status;
 };
-static_assert(sizeof(EncArgs) <= 9600 && sizeof(DecArgs) <= 9600, "kernel-argument budget");
+static_assert(sizeof(EncArgs<kCapLarge>) <= 9600 && sizeof(DecArgs<kCapLarge>) <= 9600, "kernel-argument budget");
 
 __device__ __forceinline__ float wave_min(float v) {
 #pragma unroll
@@ -117,9 +122,10 @@ __device__ __forceinline__ void acc3(float v, float& mn, float& mx, float& am) {
   am = a < am ? a : am;
 }
 
-__global__ __launch_bounds__(kThreads) void terngrad_minmax_kernel(const EncArgs a) {
+template <int CAP>
+__global__ __launch_bounds__(kThreads) void terngrad_minmax_kernel(const EncArgs<CAP> a) {
   const int tile = blockIdx.x;
-  const int s = find_segment<kMaxSeg>(a.tile_start, a.nseg, tile);
+  const int s = find_segment<CAP>(a.tile_start, a.nseg, tile);
   const float* __restrict__ xp = a.seg[s].x;
   const uint32_t n = static_cast<uint32_t>(a.seg[s].n);
   const uint32_t t = static_cast<uint32_t>(tile - a.tile_start[s]);
@@ -147,7 +153,8 @@ __global__ __launch_bounds__(kThreads) void terngrad_minmax_kernel(const EncArgs
 // and writes the header.  (A last-arriving-workgroup scheme inside the
 // reduction kernel would save this launch, but thousands of workgroups bumping
 // one arrival counter serialise at ~40 ns each across the XCDs.)
-__global__ __launch_bounds__(kThreads) void terngrad_finalize_kernel(const EncArgs a) {
+template <int CAP>
+__global__ __launch_bounds__(kThreads) void terngrad_finalize_kernel(const EncArgs<CAP> a) {
   const int s = blockIdx.x;
   const float* __restrict__ xp = a.seg[s].x;
   const uint32_t n = static_cast<uint32_t>(a.seg[s].n);
@@ -252,7 +259,7 @@ __device__ __forceinline__ void quant_tile(const EncSeg& sg, const Scalars sc, u
     for (int k = 0; k < kQIters; k++)
 #pragma unroll
       for (int h = 0; h < UNIT / 4; h++)
-        v[k][h] = ld4(xp + size_t(u0 + k * kThreads) * UNIT + h * 4);
+        v[k][h] = ld4_stream(xp + size_t(u0 + k * kThreads) * UNIT + h * 4);
 #pragma unroll
     for (int k = 0; k < kQIters; k++) {
       const uint32_t u = u0 + k * kThreads;
@@ -309,9 +316,10 @@ __device__ __forceinline__ void quant_dispatch(const EncSeg& sg, const Scalars s
 }
 
 // tile_start here counts quantise tiles (kThreads*kQIters units each).
-__global__ __launch_bounds__(kThreads) void terngrad_quant_kernel(const EncArgs a) {
+template <int CAP>
+__global__ __launch_bounds__(kThreads) void terngrad_quant_kernel(const EncArgs<CAP> a) {
   const int tile = blockIdx.x;
-  const int s = find_segment<kMaxSeg>(a.tile_start, a.nseg, tile);
+  const int s = find_segment<CAP>(a.tile_start, a.nseg, tile);
   const Scalars sc = a.scalars[s];
   const uint32_t t = static_cast<uint32_t>(tile - a.tile_start[s]);
   switch (a.seg[s].bits) {
@@ -322,29 +330,53 @@ __global__ __launch_bounds__(kThreads) void terngrad_quant_kernel(const EncArgs 
   }
 }
 
-template <int B, bool ADD>
+// The 4*B bits holding the codes of the 4-element group that starts at element e.
+template <int B>
+__device__ __forceinline__ uint32_t group_bits(const uint8_t* __restrict__ pay, size_t e) {
+  if (B == 1) return (uint32_t(pay[e >> 3]) >> (e & 4)) & 0xFu;
+  if (B == 2) return pay[e >> 2];
+  if (B == 4) return uint32_t(pay[e >> 1]) | (uint32_t(pay[(e >> 1) + 1]) << 8);
+  return uint32_t(pay[e]) | (uint32_t(pay[e + 1]) << 8) | (uint32_t(pay[e + 2]) << 16) | (uint32_t(pay[e + 3]) << 24);
+}
+
+template <int B>
+__device__ __forceinline__ float4 group_values(uint32_t bits, float gap, float mn) {
+  constexpr uint32_t MASK = (1u << B) - 1u;
+  // static_cast<float>(qval*gap + min_f), terngrad_body.h:127
+  return make_float4(float(int((bits >> (0 * B)) & MASK)) * gap + mn, float(int((bits >> (1 * B)) & MASK)) * gap + mn,
+                     float(int((bits >> (2 * B)) & MASK)) * gap + mn, float(int((bits >> (3 * B)) & MASK)) * gap + mn);
+}
+
+// STREAM selects the streaming store for the write-only case (the in-place add
+// always streams).
+template <int B, bool ADD, bool STREAM>
 __device__ __forceinline__ void decode_tile(const DecSeg& sg, float mn, float gap, uint32_t cnt, uint32_t tile_in_seg) {
   constexpr int DPB = 8 / B;
   constexpr uint32_t MASK = (1u << B) - 1u;
   float* __restrict__ op = sg.out;
   const uint8_t* __restrict__ pay = sg.in + 10;
-  const uint32_t g0 = tile_in_seg * uint32_t(kThreads * kQIters) + threadIdx.x;  // groups of 4 elements
+  const uint32_t g0 = tile_in_seg * uint32_t(kThreads * kDIters) + threadIdx.x;  // groups of 4 elements
+  if (uint64_t(g0 - threadIdx.x + kThreads * kDIters) * 4 <= cnt) {
+    // Whole tile inside the tensor.  Each step's store is kept behind its own
+    // load (the barrier stops the compiler from batching the four stores):
+    // streaming stores issued back to back run about 35 % slower here.
 #pragma unroll
-  for (int k = 0; k < kQIters; k++) {
-    const uint32_t grp = g0 + k * kThreads;
-    const size_t e = size_t(grp) * 4;
+    for (int k = 0; k < kDIters; k++) {
+      const size_t e = size_t(g0 + k * kThreads) * 4;
+      float4 v = group_values<B>(group_bits<B>(pay, e), gap, mn);
+      if (ADD) {
+        const float4 o = ld4_stream(op + e);
+        v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w;
+      }
+      if (ADD || STREAM) st4_stream(op + e, v); else st4(op + e, v);
+      __asm__ volatile("" ::: "memory");
+    }
+    return;
+  }
+  for (int k = 0; k < kDIters; k++) {
+    const size_t e = size_t(g0 + k * kThreads) * 4;
     if (e + 4 <= cnt) {
-      uint32_t bits;  // the 4*B bits holding this group's codes
-      if (B == 1) bits = (pay[e >> 3] >> (e & 4)) & 0xFu;
-      else if (B == 2) bits = pay[e >> 2];
-      else if (B == 4) bits = uint32_t(pay[e >> 1]) | (uint32_t(pay[(e >> 1) + 1]) << 8);
-      else bits = uint32_t(pay[e]) | (uint32_t(pay[e + 1]) << 8) | (uint32_t(pay[e + 2]) << 16) | (uint32_t(pay[e + 3]) << 24);
-      float4 v;
-      // static_cast<float>(qval*gap + min_f), terngrad_body.h:127
-      v.x = float(int((bits >> (0 * B)) & MASK)) * gap + mn;
-      v.y = float(int((bits >> (1 * B)) & MASK)) * gap + mn;
-      v.z = float(int((bits >> (2 * B)) & MASK)) * gap + mn;
-      v.w = float(int((bits >> (3 * B)) & MASK)) * gap + mn;
+      float4 v = group_values<B>(group_bits<B>(pay, e), gap, mn);
       if (ADD) {
         const float4 o = ld4(op + e);
         v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w;
@@ -361,13 +393,16 @@ __device__ __forceinline__ void decode_tile(const DecSeg& sg, float mn, float ga
 }
 
 template <int B>
-__device__ __forceinline__ void decode_dispatch(const DecSeg& sg, float mn, float gap, uint32_t cnt, uint32_t t) {
-  if (sg.add) decode_tile<B, true>(sg, mn, gap, cnt, t); else decode_tile<B, false>(sg, mn, gap, cnt, t);
+__device__ __forceinline__ void decode_dispatch(const DecSeg& sg, float mn, float gap, uint32_t cnt, uint32_t t, bool ss) {
+  if (sg.add) decode_tile<B, true, true>(sg, mn, gap, cnt, t);
+  else if (ss) decode_tile<B, false, true>(sg, mn, gap, cnt, t);
+  else decode_tile<B, false, false>(sg, mn, gap, cnt, t);
 }
 
-__global__ __launch_bounds__(kThreads) void terngrad_decode_kernel(const DecArgs a) {
+template <int CAP>
+__global__ __launch_bounds__(kThreads) void terngrad_decode_kernel(const DecArgs<CAP> a) {
   const int tile = blockIdx.x;
-  const int s = find_segment<kMaxSeg>(a.tile_start, a.nseg, tile);
+  const int s = find_segment<CAP>(a.tile_start, a.nseg, tile);
   const uint8_t* __restrict__ in = a.seg[s].in;
   const uint32_t bits = in[0];
   const uint32_t tail = in[1];
@@ -390,14 +425,88 @@ __global__ __launch_bounds__(kThreads) void terngrad_decode_kernel(const DecArgs
   const uint32_t cnt = static_cast<uint32_t>(c);
   const uint32_t t = static_cast<uint32_t>(tile - a.tile_start[s]);
   switch (bits) {
-    case 1: decode_dispatch<1>(a.seg[s], mn, gap, cnt, t); break;
-    case 2: decode_dispatch<2>(a.seg[s], mn, gap, cnt, t); break;
-    case 4: decode_dispatch<4>(a.seg[s], mn, gap, cnt, t); break;
-    default: decode_dispatch<8>(a.seg[s], mn, gap, cnt, t); break;
+    case 1: decode_dispatch<1>(a.seg[s], mn, gap, cnt, t, a.stream_store != 0); break;
+    case 2: decode_dispatch<2>(a.seg[s], mn, gap, cnt, t, a.stream_store != 0); break;
+    case 4: decode_dispatch<4>(a.seg[s], mn, gap, cnt, t, a.stream_store != 0); break;
+    default: decode_dispatch<8>(a.seg[s], mn, gap, cnt, t, a.stream_store != 0); break;
   }
 }
 
 inline int32_t ceil_div(int64_t a, int64_t b) { return static_cast<int32_t>((a + b - 1) / b); }
+
+template <int CAP>
+int launch_encode(int count, const float* const* ins, const int32_t* in_sizes, uint8_t* const* outs,
+                  const int32_t* out_sizes, const uint8_t* bitwidths, const int32_t* enable_randoms,
+                  const uint64_t* seeds, Scalars* scal_base, Partial* part_base, hipStream_t st) {
+  EncArgs<CAP> a;
+  int i = 0;
+  size_t part_off = 0;
+  while (i < count) {
+    const int first = i;
+    a.nseg = 0;
+    a.tile_start[0] = 0;
+    a.partials = part_base + part_off;
+    a.scalars = scal_base + first;
+    int32_t qstart[CAP + 1];
+    qstart[0] = 0;
+    while (i < count && a.nseg < CAP) {
+      const int32_t n = in_sizes[i];
+      const int b = bitwidths[i];
+      const int unit = (8 / b) > 4 ? (8 / b) : 4;
+      const int32_t rt = ceil_div(n, kRedTile);
+      const int32_t qt = ceil_div(ceil_div(n, unit), kThreads * kQIters);
+      if (int64_t(a.tile_start[a.nseg]) + rt > INT32_MAX || int64_t(qstart[a.nseg]) + qt > INT32_MAX) break;
+      const uint64_t seed = seeds ? seeds[i] : hpx::clock_seed();
+      a.seg[a.nseg] = EncSeg{ins[i], outs[i], n, out_sizes[i], static_cast<uint32_t>(seed),
+                             static_cast<uint8_t>(b), static_cast<uint8_t>(enable_randoms[i] != 0), 0};
+      a.tile_start[a.nseg + 1] = a.tile_start[a.nseg] + rt;
+      qstart[a.nseg + 1] = qstart[a.nseg] + qt;
+      a.nseg++;
+      i++;
+    }
+    HPX_LAUNCH("terngrad_minmax_kernel", terngrad_minmax_kernel<CAP>, dim3(a.tile_start[a.nseg]), dim3(kThreads), st, a);
+    HPX_HIP(hipGetLastError());
+    HPX_LAUNCH("terngrad_finalize_kernel", terngrad_finalize_kernel<CAP>, dim3(a.nseg), dim3(kThreads), st, a);
+    HPX_HIP(hipGetLastError());
+    part_off += size_t(a.tile_start[a.nseg]);
+    for (int k = 0; k <= a.nseg; k++) a.tile_start[k] = qstart[k];
+    HPX_LAUNCH("terngrad_quant_kernel", terngrad_quant_kernel<CAP>, dim3(a.tile_start[a.nseg]), dim3(kThreads), st, a);
+    HPX_HIP(hipGetLastError());
+  }
+  return HPX_OK;
+}
+
+template <int CAP>
+int launch_decode(int count, float* const* outs, const int32_t* out_sizes, const uint8_t* const* ins,
+                  const int32_t* in_sizes, const int32_t* is_add_tos, uint32_t* status, hipStream_t st) {
+  DecArgs<CAP> a;
+  a.status = status;
+  size_t out_bytes = 0;
+  for (int k = 0; k < count; k++) out_bytes += out_sizes[k] > 0 ? size_t(out_sizes[k]) * 4 : 0;
+  a.stream_store = out_bytes <= hpx::stream_store_max_bytes();
+  int i = 0;
+  while (i < count) {
+    a.nseg = 0;
+    a.tile_start[0] = 0;
+    while (i < count && a.nseg < CAP) {
+      HPX_ARG(out_sizes[i] >= 0 && in_sizes[i] >= 10, "hpx_terngrad_decode: message %d: out_size %d, in_size %d", i,
+              out_sizes[i], in_sizes[i]);
+      if (out_sizes[i] > 0) {
+        HPX_ARG(outs[i] && ins[i], "hpx_terngrad_decode: message %d has a null pointer", i);
+        const int32_t t = ceil_div(out_sizes[i], kDecTile);
+        if (int64_t(a.tile_start[a.nseg]) + t > INT32_MAX) break;
+        a.seg[a.nseg] = DecSeg{outs[i], ins[i], out_sizes[i], in_sizes[i], is_add_tos[i] != 0, 0};
+        a.tile_start[a.nseg + 1] = a.tile_start[a.nseg] + t;
+        a.nseg++;
+      }
+      i++;
+    }
+    if (a.nseg == 0) continue;
+    HPX_LAUNCH("terngrad_decode_kernel", terngrad_decode_kernel<CAP>, dim3(a.tile_start[a.nseg]), dim3(kThreads), st, a);
+    HPX_HIP(hipGetLastError());
+  }
+  return HPX_OK;
+}
 
 }  // namespace
 
@@ -434,42 +543,11 @@ HPX_API int hpx_terngrad_encode(int count, const float* const* ins, const int32_
   Scalars* scal_base = reinterpret_cast<Scalars*>(ws->dev);
   Partial* part_base = reinterpret_cast<Partial*>(ws->dev + scal_bytes);
 
-  EncArgs a;
-  int i = 0;
-  size_t part_off = 0;
-  while (i < count) {
-    const int first = i;
-    a.nseg = 0;
-    a.tile_start[0] = 0;
-    a.partials = part_base + part_off;
-    a.scalars = scal_base + first;
-    int32_t qstart[kMaxSeg + 1];
-    qstart[0] = 0;
-    while (i < count && a.nseg < kMaxSeg) {
-      const int32_t n = in_sizes[i];
-      const int b = bitwidths[i];
-      const int unit = (8 / b) > 4 ? (8 / b) : 4;
-      const int32_t rt = ceil_div(n, kRedTile);
-      const int32_t qt = ceil_div(ceil_div(n, unit), kThreads * kQIters);
-      if (int64_t(a.tile_start[a.nseg]) + rt > INT32_MAX || int64_t(qstart[a.nseg]) + qt > INT32_MAX) break;
-      const uint64_t seed = seeds ? seeds[i] : hpx::clock_seed();
-      a.seg[a.nseg] = EncSeg{ins[i], outs[i], n, out_sizes[i], static_cast<uint32_t>(seed),
-                             static_cast<uint8_t>(b), static_cast<uint8_t>(enable_randoms[i] != 0), 0};
-      a.tile_start[a.nseg + 1] = a.tile_start[a.nseg] + rt;
-      qstart[a.nseg + 1] = qstart[a.nseg] + qt;
-      a.nseg++;
-      i++;
-    }
-    HPX_LAUNCH("terngrad_minmax_kernel", terngrad_minmax_kernel, dim3(a.tile_start[a.nseg]), dim3(kThreads), st, a);
-    HPX_HIP(hipGetLastError());
-    HPX_LAUNCH("terngrad_finalize_kernel", terngrad_finalize_kernel, dim3(a.nseg), dim3(kThreads), st, a);
-    HPX_HIP(hipGetLastError());
-    part_off += size_t(a.tile_start[a.nseg]);
-    for (int k = 0; k <= a.nseg; k++) a.tile_start[k] = qstart[k];
-    HPX_LAUNCH("terngrad_quant_kernel", terngrad_quant_kernel, dim3(a.tile_start[a.nseg]), dim3(kThreads), st, a);
-    HPX_HIP(hipGetLastError());
-  }
-  return HPX_OK;
+  if (count <= kCapSmall)
+    return launch_encode<kCapSmall>(count, ins, in_sizes, outs, out_sizes, bitwidths, enable_randoms, seeds, scal_base,
+                                    part_base, st);
+  return launch_encode<kCapLarge>(count, ins, in_sizes, outs, out_sizes, bitwidths, enable_randoms, seeds, scal_base,
+                                  part_base, st);
 }
 
 HPX_API int hpx_terngrad_decode(int count, float* const* outs, const int32_t* out_sizes,
@@ -485,30 +563,9 @@ HPX_API int hpx_terngrad_decode(int count, float* const* outs, const int32_t* ou
   std::lock_guard<std::mutex> lock(ws->mu);
   int rc = hpx::ensure_workspace(ws, 0);
   if (rc != HPX_OK) return rc;
-  DecArgs a;
-  a.status = ws->state + hpx::kStatusWord;
-  int i = 0;
-  while (i < count) {
-    a.nseg = 0;
-    a.tile_start[0] = 0;
-    while (i < count && a.nseg < kMaxSeg) {
-      HPX_ARG(out_sizes[i] >= 0 && in_sizes[i] >= 10, "hpx_terngrad_decode: message %d: out_size %d, in_size %d", i,
-              out_sizes[i], in_sizes[i]);
-      if (out_sizes[i] > 0) {
-        HPX_ARG(outs[i] && ins[i], "hpx_terngrad_decode: message %d has a null pointer", i);
-        const int32_t t = ceil_div(out_sizes[i], kDecTile);
-        if (int64_t(a.tile_start[a.nseg]) + t > INT32_MAX) break;
-        a.seg[a.nseg] = DecSeg{outs[i], ins[i], out_sizes[i], in_sizes[i], is_add_tos[i] != 0, 0};
-        a.tile_start[a.nseg + 1] = a.tile_start[a.nseg] + t;
-        a.nseg++;
-      }
-      i++;
-    }
-    if (a.nseg == 0) continue;
-    HPX_LAUNCH("terngrad_decode_kernel", terngrad_decode_kernel, dim3(a.tile_start[a.nseg]), dim3(kThreads), st, a);
-    HPX_HIP(hipGetLastError());
-  }
-  return HPX_OK;
+  uint32_t* status = ws->state + hpx::kStatusWord;
+  if (count <= kCapSmall) return launch_decode<kCapSmall>(count, outs, out_sizes, ins, in_sizes, is_add_tos, status, st);
+  return launch_decode<kCapLarge>(count, outs, out_sizes, ins, in_sizes, is_add_tos, status, st);
 }
 
 HPX_API int hpx_terngrad_decode_status(hpx_stream_t stream) {
