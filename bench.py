@@ -34,9 +34,13 @@ FP32_MFMA_PEAK_TF = 157.3   # MI355X dense fp32 matrix, published
 N_TERNGRAD = 25_557_032
 N_DGC = 138_357_544
 
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
-# (scaled by a copy kernel of known size); None until such a run has been summarised under profiles/.
-MEASURED_TRAFFIC_BYTES = {}
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, each scaled by what the same
+# counter reads for a plain copy of known size.
+MEASURED_TRAFFIC_BYTES = {  # profiles/terngrad_25M_pmc_fetch_write.txt (FETCH x1.99949 + WRITE x1.0, KiB -> bytes)
+    "terngrad_minmax_kernel": int((49946.2 * 1.99949 + 122.1) * 1024),
+    "terngrad_quant_kernel": int((49957.5 * 1.99949 + 6434.6) * 1024),
+    "terngrad_decode_kernel": int((3573.3 * 1.99949 + 99909.5) * 1024),
+}
 
 
 def parse():
@@ -48,6 +52,9 @@ def parse():
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="time budget of the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the TBQ / DGC / PowerSGD side measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-calibration", type=int, default=0,
+                    help="also run this many plain 4*N-byte device copies (a kernel of known traffic for scaling "
+                         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings)")
     return ap.parse_args()
 
 
@@ -139,6 +146,8 @@ def main():
         enc()
         dcd()
 
+    for _ in range(args.copy_calibration):
+        sets[0][2].copy_(sets[0][0])  # reads 4*N bytes, writes 4*N bytes
     sec = timed(torch, step, args.steps, args.warmup)
     value = 4.0 * n / sec / 1e9
 
