@@ -84,7 +84,42 @@ __global__ __launch_bounds__(kThreads) void psgd_encode1_kernel(const Args a) {
   for (int c = 0; c < CG; c++) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   const bool rows_full = (row0 + 3 < n) && (int64_t(row0 + 4) * m <= N);
-  for (int k0 = kbeg; k0 < kend; k0 += 64) {
+  int k0 = kbeg;
+  if (rows_full) {
+    // Main loop: kUnroll 64-column steps at a time, every load issued before the first use.
+    constexpr int kUnroll = 4;
+    for (; k0 + 64 * kUnroll <= kend; k0 += 64 * kUnroll) {
+      float4 g4[kUnroll], r4[kUnroll];
+      float q[kUnroll][4][CG];
+#pragma unroll
+      for (int u = 0; u < kUnroll; u++) {
+        const int64_t f = int64_t(row) * m + k0 + 64 * u + 4 * b;
+        g4[u] = ld4_stream(G + f);
+        r4[u] = ld4_stream(R + f);
+      }
+#pragma unroll
+      for (int u = 0; u < kUnroll; u++)
+#pragma unroll
+        for (int t = 0; t < 4; t++)
+#pragma unroll
+          for (int c = 0; c < CG; c++) {
+            const int col = c * 4 + i;  // B operand: lane 4b+j holds Q[k][j]
+            q[u][t][c] = col < r ? Q[int64_t(k0 + 64 * u + 4 * b + t) * r + col] : 0.f;
+          }
+#pragma unroll
+      for (int u = 0; u < kUnroll; u++) {
+        const int64_t f = int64_t(row) * m + k0 + 64 * u + 4 * b;
+        const float4 m4 = make_float4(g4[u].x + r4[u].x, g4[u].y + r4[u].y, g4[u].z + r4[u].z, g4[u].w + r4[u].w);
+        st4(M + f, m4);
+        const float v[4] = {m4.x, m4.y, m4.z, m4.w};
+#pragma unroll
+        for (int t = 0; t < 4; t++)
+#pragma unroll
+          for (int c = 0; c < CG; c++) acc[c] = mfma4(v[t], q[u][t][c], acc[c]);
+      }
+    }
+  }
+  for (; k0 < kend; k0 += 64) {
     const int kk = k0 + 4 * b;
     float v[4];
     if (rows_full && k0 + 64 <= m) {
@@ -163,32 +198,61 @@ __device__ __forceinline__ double block_sum(double v, double* s_red) {
   return t;
 }
 
-__global__ __launch_bounds__(kOrthThreads) void psgd_orth_kernel(const Args a) {
-  __shared__ double s_red[kOrthThreads / kWave];
-  const Seg& sg = a.seg[blockIdx.x];
-  float* __restrict__ P = sg.P;
-  const int n = sg.n, r = sg.r;
+// P[row][c] of the matrix being orthonormalised: either the caller's row-major
+// array in global memory or a column-major copy in LDS (conflict-free for the
+// row-strided sweeps below).
+template <bool LDS>
+struct PView {
+  float* p;
+  int n, r;
+  __device__ __forceinline__ float& at(int row, int c) const { return LDS ? p[c * n + row] : p[int64_t(row) * r + c]; }
+};
+
+template <bool LDS>
+__device__ __forceinline__ void gram_schmidt(const PView<LDS> P, double* s_red) {
+  const int n = P.n, r = P.r;
   for (int sweep = 0; sweep < 2; sweep++) {
     for (int c = 0; c < r; c++) {
       double ss = 0;
       for (int row = threadIdx.x; row < n; row += kOrthThreads) {
-        const double x = P[int64_t(row) * r + c];
+        const double x = P.at(row, c);
         ss += x * x;
       }
       ss = block_sum(ss, s_red);
       const float inv = ss > 0 ? static_cast<float>(1.0 / sqrt(ss)) : 0.f;
-      for (int row = threadIdx.x; row < n; row += kOrthThreads) P[int64_t(row) * r + c] *= inv;
+      for (int row = threadIdx.x; row < n; row += kOrthThreads) P.at(row, c) *= inv;
       for (int c2 = c + 1; c2 < r; c2++) {
         double d = 0;
-        for (int row = threadIdx.x; row < n; row += kOrthThreads)
-          d += double(P[int64_t(row) * r + c]) * double(P[int64_t(row) * r + c2]);
+        for (int row = threadIdx.x; row < n; row += kOrthThreads) d += double(P.at(row, c)) * double(P.at(row, c2));
         d = block_sum(d, s_red);
         const float df = static_cast<float>(d);
-        for (int row = threadIdx.x; row < n; row += kOrthThreads)
-          P[int64_t(row) * r + c2] -= df * P[int64_t(row) * r + c];
+        for (int row = threadIdx.x; row < n; row += kOrthThreads) P.at(row, c2) -= df * P.at(row, c);
       }
     }
   }
+}
+
+// Global-memory variant: any n x r.
+__global__ __launch_bounds__(kOrthThreads) void psgd_orth_kernel(const Args a) {
+  __shared__ double s_red[kOrthThreads / kWave];
+  const Seg& sg = a.seg[blockIdx.x];
+  gram_schmidt(PView<false>{sg.P, sg.n, sg.r}, s_red);
+}
+
+// LDS variant: the whole n x r factor (at most kOrthLdsFloats values) is staged in
+// dynamic shared memory, orthonormalised there and written back.
+constexpr int kOrthLdsFloats = 36 * 1024;  // 144 KiB of the 160 KiB LDS
+__global__ __launch_bounds__(kOrthThreads) void psgd_orth_lds_kernel(const Args a) {
+  __shared__ double s_red[kOrthThreads / kWave];
+  extern __shared__ float s_p[];
+  const Seg& sg = a.seg[blockIdx.x];
+  float* __restrict__ Pg = sg.P;
+  const int n = sg.n, r = sg.r;
+  for (int e = threadIdx.x; e < n * r; e += kOrthThreads) s_p[(e % r) * n + e / r] = Pg[e];
+  __syncthreads();
+  gram_schmidt(PView<true>{s_p, n, r}, s_red);
+  __syncthreads();
+  for (int e = threadIdx.x; e < n * r; e += kOrthThreads) Pg[e] = s_p[(e % r) * n + e / r];
 }
 
 // ---- encode2, step 2: Q = M^T P ------------------------------------------------
@@ -315,6 +379,12 @@ __global__ __launch_bounds__(kThreads) void psgd_decode_kernel(const Args a) {
 
   const bool cols_full = k0 + kStrip <= m;
   for (int row0 = rbeg; row0 < rend; row0 += 4) {
+    const bool full4 = cols_full && row0 + 4 <= rend && int64_t(row0 + 3) * m + kk + 4 <= N;
+    float4 g4[4];
+    if (full4) {
+#pragma unroll
+      for (int ii = 0; ii < 4; ii++) g4[ii] = ld4_stream(G + int64_t(row0 + ii) * m + kk);
+    }
     f32x4 acc[4];
 #pragma unroll
     for (int t = 0; t < 4; t++) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -324,28 +394,32 @@ __global__ __launch_bounds__(kThreads) void psgd_decode_kernel(const Args a) {
 #pragma unroll
       for (int t = 0; t < 4; t++) acc[t] = mfma4(p, q[t][col], acc[t]);
     }
+    if (full4) {
+#pragma unroll
+      for (int ii = 0; ii < 4; ii++) {
+        const int64_t f = int64_t(row0 + ii) * m + kk;
+        const float4 m4 = make_float4(acc[0][ii], acc[1][ii], acc[2][ii], acc[3][ii]);
+        const float4 r4 = make_float4(g4[ii].x - m4.x, g4[ii].y - m4.y, g4[ii].z - m4.z, g4[ii].w - m4.w);
+        st4_stream(R + f, r4);
+        st4_stream(G + f, m4);  // in place over the line just read
+        st4(M + f, m4);
+      }
+      continue;
+    }
 #pragma unroll
     for (int ii = 0; ii < 4; ii++) {
       const int row = row0 + ii;
       if (row >= rend) break;
       const int64_t f = int64_t(row) * m + kk;
-      const float4 m4 = make_float4(acc[0][ii], acc[1][ii], acc[2][ii], acc[3][ii]);
-      if (cols_full && f + 4 <= N) {
-        const float4 g4 = ld4_stream(G + f);
-        st4_stream(R + f, make_float4(g4.x - m4.x, g4.y - m4.y, g4.z - m4.z, g4.w - m4.w));
-        st4_stream(G + f, m4);
-        st4(M + f, m4);
-      } else {
-        const float mv[4] = {m4.x, m4.y, m4.z, m4.w};
+      const float mv[4] = {acc[0][ii], acc[1][ii], acc[2][ii], acc[3][ii]};
 #pragma unroll
-        for (int t = 0; t < 4; t++) {
-          if (kk + t < m) {
-            if (f + t < N) {
-              R[f + t] = G[f + t] - mv[t];
-              G[f + t] = mv[t];
-            }
-            M[f + t] = mv[t];
+      for (int t = 0; t < 4; t++) {
+        if (kk + t < m) {
+          if (f + t < N) {
+            R[f + t] = G[f + t] - mv[t];
+            G[f + t] = mv[t];
           }
+          M[f + t] = mv[t];
         }
       }
     }
@@ -463,7 +537,18 @@ HPX_API int hpx_powersgd_encode2(int count, float* const* Ps, const float* const
       i++;
     }
     (void)first;
-    HPX_LAUNCH("psgd_orth_kernel", psgd_orth_kernel, dim3(a.nseg), dim3(kOrthThreads), st, a);
+    int64_t max_nr = 0;
+    for (int k = 0; k < a.nseg; k++) max_nr = int64_t(a.seg[k].n) * a.seg[k].r > max_nr ? int64_t(a.seg[k].n) * a.seg[k].r : max_nr;
+    if (max_nr <= kOrthLdsFloats) {
+      const size_t lds = size_t(max_nr) * sizeof(float);
+      HPX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(psgd_orth_lds_kernel),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, int(lds)));
+      if (hpx::g_prof_on) hpx::prof_begin("psgd_orth_kernel", st);
+      hipLaunchKernelGGL(psgd_orth_lds_kernel, dim3(a.nseg), dim3(kOrthThreads), lds, st, a);
+      if (hpx::g_prof_on) hpx::prof_end(st);
+    } else {
+      HPX_LAUNCH("psgd_orth_kernel", psgd_orth_kernel, dim3(a.nseg), dim3(kOrthThreads), st, a);
+    }
     PSGD_LAUNCH_CG(psgd_mtp_kernel, cg, a.tile_start[a.nseg], st, a);
     HPX_HIP(hipGetLastError());
     for (int k = 0; k <= a.nseg; k++) a.tile_start[k] = red_start[k];
