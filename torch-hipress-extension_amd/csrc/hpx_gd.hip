@@ -232,7 +232,8 @@ __global__ __launch_bounds__(kThreads) void gd_stream_kernel(const float* __rest
 // the grand total.
 __global__ __launch_bounds__(kSelThreads) void gd_scan_kernel(const uint32_t* __restrict__ cnt, uint32_t* __restrict__ off,
                                                               uint32_t n, uint32_t* __restrict__ chunk_tot,
-                                                              uint32_t* __restrict__ chunk_off, GdState* __restrict__ st) {
+                                                              uint32_t* __restrict__ chunk_off, GdState* __restrict__ st,
+                                                              uint32_t* __restrict__ host_total) {
   __shared__ uint32_t s_wave[kSelThreads / kWave];
   __shared__ uint32_t s_last;
   const uint32_t t = threadIdx.x, lane = t & (kWave - 1), wave = t / kWave;
@@ -283,7 +284,11 @@ __global__ __launch_bounds__(kSelThreads) void gd_scan_kernel(const uint32_t* __
     const uint32_t ex = inc2 - a0 - a1;
     if (2 * t < gridDim.x) chunk_off[2 * t] = ex;
     if (2 * t + 1 < gridDim.x) chunk_off[2 * t + 1] = ex + a0;
-    if (t == kWave - 1) st->total = inc2;
+    if (t == kWave - 1) {
+      st->total = inc2;
+      // pinned host word: the host reads it after its one wait on the stream, no copy command needed
+      __hip_atomic_store(host_total, inc2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
   }
 }
 
@@ -544,8 +549,9 @@ int gd_encode_one(const float* g, int32_t N, float* r, uint8_t* out, double samp
   HPX_LAUNCH("gd_select_kernel", gd_select_kernel<3>, dim3(sel_blocks), dim3(kSelThreads), st, sa);
   HPX_LAUNCH("gd_threshold_kernel", gd_threshold_kernel, dim3(1), dim3(kSelThreads), st, sa);
   HPX_LAUNCH("gd_stream_kernel", gd_stream_kernel, dim3(ntiles), dim3(kThreads), st, g, r, n, state, masks, blk_cnt);
+  uint32_t* h_total = reinterpret_cast<uint32_t*>(ws->pinned);
   HPX_LAUNCH("gd_scan_kernel", gd_scan_kernel, dim3(nchunks), dim3(kSelThreads), st, blk_cnt, blk_off, ntiles, chunk_tot,
-             chunk_off, state);
+             chunk_off, state, h_total);
   HPX_HIP(hipGetLastError());
   // Common case (nothing to cut) queued before the host knows the count.
   int32_t* out_idx = reinterpret_cast<int32_t*>(out + 4);
@@ -553,10 +559,8 @@ int gd_encode_one(const float* g, int32_t N, float* r, uint8_t* out, double samp
   HPX_LAUNCH("gd_expand_kernel", gd_expand_kernel, dim3(cdiv(ntiles, kThreads / kWave)), dim3(kThreads), st, masks, blk_off,
              chunk_off, ntiles, state, out_idx, lim, out, r);
   HPX_HIP(hipGetLastError());
-  uint32_t* h_total = reinterpret_cast<uint32_t*>(ws->pinned);
-  HPX_HIP(hipMemcpyAsync(h_total, &state->total, sizeof(uint32_t), hipMemcpyDeviceToHost, st));
   HPX_HIP(hipStreamSynchronize(st));
-  const uint32_t total = *h_total;
+  const uint32_t total = *reinterpret_cast<volatile uint32_t*>(h_total);
   if (total <= lim) return HPX_OK;
 
   // More candidates than `expected`: order them by |r| descending and keep the first `expected`.

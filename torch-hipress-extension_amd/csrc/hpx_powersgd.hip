@@ -288,7 +288,30 @@ __global__ __launch_bounds__(kThreads) void psgd_mtp_kernel(const Args a) {
 
   const bool cols_full = k0 + kStrip <= m;
   const int j = lane & 3;
-  for (int row = rbeg; row < rend; row++) {
+  int row = rbeg;
+  if (cols_full) {
+    // Main loop: 8 rows at a time, every load issued before the first use.
+    constexpr int kRows = 8;
+    for (; row + kRows <= rend; row += kRows) {
+      float4 m4[kRows];
+      float p[kRows][CG];
+#pragma unroll
+      for (int u = 0; u < kRows; u++) m4[u] = ld4_stream(M + int64_t(row + u) * m + kk);
+#pragma unroll
+      for (int u = 0; u < kRows; u++)
+#pragma unroll
+        for (int c = 0; c < CG; c++) p[u][c] = (c * 4 + j) < r ? P[int64_t(row + u) * r + c * 4 + j] : 0.f;
+#pragma unroll
+      for (int u = 0; u < kRows; u++) {
+        const float v[4] = {m4[u].x, m4[u].y, m4[u].z, m4[u].w};
+#pragma unroll
+        for (int c = 0; c < CG; c++)
+#pragma unroll
+          for (int t = 0; t < 4; t++) acc[c][t] = mfma4(v[t], p[u][c], acc[c][t]);
+      }
+    }
+  }
+  for (; row < rend; row++) {
     float v[4];
     if (cols_full) {
       const float4 m4 = ld4_stream(M + int64_t(row) * m + kk);
