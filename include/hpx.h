@@ -24,6 +24,9 @@
  *     Entry points may be called from several host threads; calls that share a
  *     stream are serialised while they enqueue.
  *   - Sizes are int32 element/byte counts exactly as in the reference.
+ *   - Tuning: the environment variable HPX_STREAM_STORE_MAX_MB (read once) sets the
+ *     output size up to which the write-only decoders use streaming stores
+ *     (default 128).
  */
 #ifndef HPX_H_
 #define HPX_H_
