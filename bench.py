@@ -261,7 +261,23 @@ def extra(torch, np, capi, L, stream, gen):
         "ms_per_step": round(sec * 1e3, 4), "GBps_of_gradient": round(4.0 * tot / sec / 1e9, 1),
         "algorithmic_bytes": 16.5 * tot, "frac_of_hbm_peak": round(16.5 * tot / sec / 1e9 / HBM_PEAK_GBS, 4),
         "kernel_us_per_launch": {k: round(v * 1e6, 1) for k, v in kt.items() if v}}
-    del gs, rs, ps, os_
+    # the root's gather-decode: 7 gathered messages per tensor accumulate into the tensor (hp_cuda.cpp:241-259)
+    slots = 7
+    msgs7 = [[torch.randint(0, 255, ((int(s) + 3) // 4,), dtype=torch.uint8, device="cuda", generator=gen) & 0xA5
+              for s in sizes] for _ in range(slots)]
+    outs7, ins7 = [], []
+    for k in range(slots):
+        outs7 += os_
+        ins7 += msgs7[k]
+    root = Call(L.hpx_tbq_decode, slots * len(sizes), capi.ptr_array([o.data_ptr() for o in outs7]),
+                capi.i32_array([int(s) for s in sizes] * slots), capi.ptr_array([m_.data_ptr() for m_ in ins7]),
+                capi.f32_array([1e-2] * (slots * len(sizes))), capi.i32_array([1] * (slots * len(sizes))), stream)
+    sec = timed(torch, root, 10, 2)
+    alg = (8.0 + 0.25 * slots) * tot
+    res["tbq_root_decode_add_7_messages_per_tensor"] = {
+        "ms": round(sec * 1e3, 4), "algorithmic_bytes": alg, "frac_of_hbm_peak": round(alg / sec / 1e9 / HBM_PEAK_GBS, 4),
+        "bytes_if_applied_one_message_at_a_time": 8.25 * slots * tot}
+    del gs, rs, ps, os_, msgs7, outs7, ins7
     torch.cuda.empty_cache()
 
     # ---- DGC / GradDrop top-0.1 %: 138,357,544 elements --------------------------------------

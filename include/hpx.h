@@ -80,7 +80,11 @@ int hpx_tbq_encode(int count, const float* const* grads, const int32_t* sizes,
 
 /* Replaces hp_cuda_tbqr (hp_cuda.cpp:41-50, hp_cuda_kernel.cu:161-198; body
  * tbq_body.h:160-200).  outs[t][i] = (code-1)*thr, added to the existing value
- * when is_add_tos[t] != 0. */
+ * when is_add_tos[t] != 0.  The same output may be named by several messages
+ * (the reference's root path decodes every gathered message into one tensor,
+ * hp_cuda.cpp:241-259): they are applied in call order, and when the outputs are
+ * exact duplicates all messages of a tensor are applied in a single pass over
+ * it with the same sequence of fp32 additions. */
 int hpx_tbq_decode(int count, float* const* outs, const int32_t* sizes,
                    const uint8_t* const* ins, const float* thresholds,
                    const int32_t* is_add_tos, hpx_stream_t stream);
@@ -110,7 +114,9 @@ int hpx_terngrad_encode(int count, const float* const* ins, const int32_t* in_si
  * reference, and is additionally clamped to out_sizes[t] so a malformed header
  * cannot write outside the output.  A message whose bitwidth byte is invalid
  * decodes to nothing and raises the sticky flag hpx_terngrad_decode_status
- * reports. */
+ * reports.  Several messages may name the same output (hp_cuda.cpp:421-439);
+ * they are applied in call order, in a single pass over the tensor when the
+ * outputs are exact duplicates. */
 int hpx_terngrad_decode(int count, float* const* outs, const int32_t* out_sizes,
                         const uint8_t* const* ins, const int32_t* in_sizes,
                         const int32_t* is_add_tos, hpx_stream_t stream);

@@ -157,3 +157,57 @@ def test_full_size_bucket_properties(tbq):
         assert_bits_equal(host(packed[i]), p_ref, f"bucket packed[{i}]")
         assert_bits_equal(host(rs[i]), rh, f"bucket residual[{i}]")
         assert_bits_equal(host(outs[i]), cpu.tbq_decode(p_ref, gh.size, thr), f"bucket decoded[{i}]")
+
+
+@pytest.mark.parametrize("n", [7, 4096, 10007, 300001])
+def test_several_messages_into_one_tensor(tbq, oracle_cpu, n):
+    # the root's gather-decode (hp_cuda.cpp:241-259): every gathered message names the same output tensor
+    rng = np.random.default_rng(n)
+    msgs, thrs = [], []
+    for k in range(7):
+        thr = float(np.float32(rng.uniform(1e-3, 5e-3)))
+        g = rng.normal(0, 2e-3, n).astype(np.float32)
+        msgs.append(oracle_cpu.tbq_encode(g, np.zeros(n, np.float32), thr))
+        thrs.append(thr)
+    dm = [dev(m) for m in msgs]
+    for adds in ([1] * 7, [0] + [1] * 6, [1, 1, 0, 1, 1, 1, 1], [0] * 7):
+        base = rng.normal(0, 1, n).astype(np.float32)
+        out = dev(base)
+        tbq.decode(dm, [out] * 7, thrs, adds)
+        torch.cuda.synchronize()
+        ref = base.copy()
+        for m, thr, add in zip(msgs, thrs, adds):      # one message after the other, as the reference applies them
+            ref = oracle_cpu.tbq_decode(m, n, thr, ref, add)
+        assert_bits_equal(host(out), ref, f"accumulated n={n} adds={adds}")
+
+
+def test_many_tensors_each_with_several_messages(tbq, oracle_cpu):
+    rng = np.random.default_rng(77)
+    sizes = [int(s) for s in np.exp(rng.uniform(np.log(5), np.log(20000), 70))]
+    slots = 35                                  # more than one segment of the slot table holds per tensor
+    bases = [rng.normal(0, 1, n).astype(np.float32) for n in sizes]
+    outs = [dev(b) for b in bases]
+    call_outs, call_msgs, call_thr, call_add, refs = [], [], [], [], [b.copy() for b in bases]
+    for k in range(slots):                      # interleaved: slot-major, as a gathered buffer is walked
+        for t, n in enumerate(sizes):
+            thr = float(np.float32(rng.uniform(1e-3, 5e-3)))
+            m = oracle_cpu.tbq_encode(rng.normal(0, 2e-3, n).astype(np.float32), np.zeros(n, np.float32), thr)
+            call_outs.append(outs[t]); call_msgs.append(dev(m)); call_thr.append(thr); call_add.append(1)
+            refs[t] = oracle_cpu.tbq_decode(m, n, thr, refs[t], 1)
+    tbq.decode(call_msgs, call_outs, call_thr, call_add)     # 2450 messages: several launches of the slot table
+    torch.cuda.synchronize()
+    for t in range(len(sizes)):
+        assert_bits_equal(host(outs[t]), refs[t], f"tensor {t}")
+
+
+def test_partially_overlapping_outputs_keep_call_order(tbq, oracle_cpu):
+    rng = np.random.default_rng(5)
+    n = 5000
+    buf = torch.zeros(n + 1000, device="cuda")
+    m1 = oracle_cpu.tbq_encode(rng.normal(0, 2e-3, n).astype(np.float32), np.zeros(n, np.float32), 2e-3)
+    m2 = oracle_cpu.tbq_encode(rng.normal(0, 2e-3, n).astype(np.float32), np.zeros(n, np.float32), 3e-3)
+    tbq.decode([dev(m1), dev(m2)], [buf[:n], buf[1000:1000 + n]], [2e-3, 3e-3], [1, 1])
+    ref = np.zeros(n + 1000, np.float32)
+    ref[:n] = oracle_cpu.tbq_decode(m1, n, 2e-3, ref[:n].copy(), 1)
+    ref[1000:1000 + n] = oracle_cpu.tbq_decode(m2, n, 3e-3, ref[1000:1000 + n].copy(), 1)
+    assert_bits_equal(host(buf), ref, "overlapping views")

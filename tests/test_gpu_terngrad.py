@@ -170,3 +170,44 @@ def test_full_size_config2_properties(tg):
     assert_bits_equal(host(out), ref, "full-size message")
     rc, dref = cpu.terngrad_decode(ref, n)
     assert_bits_equal(host(dec), dref, "full-size decode")
+
+
+@pytest.mark.parametrize("n", [7, 4096, 10007, 300001])
+def test_several_messages_into_one_tensor(tg, oracle_cpu, n):
+    # the root's gather-decode (hp_cuda.cpp:421-439): every gathered message names the same output tensor
+    rng = np.random.default_rng(n)
+    msgs = []
+    for k, b in enumerate([2, 2, 1, 4, 8, 2, 2]):
+        x = rng.normal(0, 1e-2 * (k + 1), n).astype(np.float32)
+        rc, m = oracle_cpu.terngrad_encode(x, b, 1, 1000 + k)
+        assert rc == 0
+        msgs.append(m)
+    dm = [dev(m) for m in msgs]
+    for adds in ([1] * 7, [0] + [1] * 6, [1, 1, 0, 1, 1, 1, 1], [0] * 7):
+        base = rng.normal(0, 1, n).astype(np.float32)
+        out = dev(base)
+        tg.decode(dm, [out] * 7, adds)
+        torch.cuda.synchronize()
+        ref = base.copy()
+        for m, add in zip(msgs, adds):
+            rc, ref = oracle_cpu.terngrad_decode(m, n, ref, add)
+        assert_bits_equal(host(out), ref, f"accumulated n={n} adds={adds}")
+    assert tg.status() == 0
+
+
+def test_many_tensors_each_with_several_messages(tg, oracle_cpu):
+    rng = np.random.default_rng(78)
+    sizes = [int(s) for s in np.exp(rng.uniform(np.log(5), np.log(20000), 70))]
+    slots = 40                                   # more than one segment of the slot table holds per tensor
+    bases = [rng.normal(0, 1, n).astype(np.float32) for n in sizes]
+    outs = [dev(b) for b in bases]
+    call_outs, call_msgs, call_add, refs = [], [], [], [b.copy() for b in bases]
+    for k in range(slots):
+        for t, n in enumerate(sizes):
+            rc, m = oracle_cpu.terngrad_encode(rng.normal(0, 1e-2, n).astype(np.float32), 2, 1, k * 1000 + t)
+            call_outs.append(outs[t]); call_msgs.append(dev(m)); call_add.append(1)
+            rc, refs[t] = oracle_cpu.terngrad_decode(m, n, refs[t], 1)
+    tg.decode(call_msgs, call_outs, call_add)
+    torch.cuda.synchronize()
+    for t in range(len(sizes)):
+        assert_bits_equal(host(outs[t]), refs[t], f"tensor {t}")

@@ -72,6 +72,11 @@ int ensure_workspace(Workspace* ws, size_t dev_bytes);
 
 uint64_t clock_seed();
 
+// How the outputs of a decode call relate: 0 = pairwise disjoint, 1 = some are
+// named more than once but every overlap is an exact duplicate (same pointer,
+// same size: several messages accumulate into one tensor), 2 = partial overlaps.
+int classify_outputs(int count, float* const* outs, const int32_t* sizes);
+
 // ---- device helpers --------------------------------------------------------
 constexpr int kWave = 64;
 

@@ -4,6 +4,7 @@
 #include <cstdio>
 #include <map>
 #include <memory>
+#include <algorithm>
 #include <cstdlib>
 #include <cstring>
 #include <utility>
@@ -101,6 +102,26 @@ size_t stream_store_max_bytes() {
     return e ? size_t(std::strtoull(e, nullptr, 10)) << 20 : kStreamStoreMaxBytes;
   }();
   return v;
+}
+
+int classify_outputs(int count, float* const* outs, const int32_t* sizes) {
+  struct Span { uintptr_t b, e; };
+  std::vector<Span> v;
+  v.reserve(count);
+  for (int i = 0; i < count; i++)
+    if (sizes[i] > 0 && outs[i]) v.push_back({reinterpret_cast<uintptr_t>(outs[i]), reinterpret_cast<uintptr_t>(outs[i]) + size_t(sizes[i]) * 4});
+  std::sort(v.begin(), v.end(), [](const Span& x, const Span& y) { return x.b < y.b || (x.b == y.b && x.e < y.e); });
+  int cls = 0;
+  uintptr_t cur_b = 0, cur_e = 0;
+  for (const Span& s : v) {
+    if (s.b < cur_e) {
+      if (s.b == cur_b && s.e == cur_e) { cls = cls < 1 ? 1 : cls; continue; }
+      return 2;
+    }
+    cur_b = s.b;
+    cur_e = s.e;
+  }
+  return cls;
 }
 
 uint64_t clock_seed() {

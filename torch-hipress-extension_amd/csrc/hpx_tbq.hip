@@ -8,6 +8,9 @@
 // call needs no device-side setup, no workspace and no host synchronisation;
 // the partial last group of a tensor is packed in the same kernel (the
 // reference round-trips it through the host, tbq_body.h:114-155).
+#include <unordered_map>
+#include <vector>
+
 #include "hpx_common.h"
 
 namespace {
@@ -193,6 +196,107 @@ __global__ __launch_bounds__(kThreads) void tbq_decode_kernel(const DecArgs<CAP>
     tbq_decode_tile<false>(a.seg[s], g0, a.stream_store != 0);
 }
 
+// ---- several messages into one tensor ---------------------------------------
+// The reference's root path hands tbq_r_body the same output tensor once per
+// gathered message (hp_cuda.cpp:241-259, is_add_to = 1) and the messages are
+// applied one after the other.  Here all messages of a tensor are applied in one
+// pass: the tensor is read once, every message contributes its byte per group in
+// call order (same sequence of fp32 additions, so the sums are bit-identical),
+// and the tensor is written once.
+constexpr int kMultiSegs = 64;
+constexpr int kMultiSlots = 448;
+constexpr int kMultiSlotsPerSeg = 32;  // a tensor's messages are staged in LDS; more of them go to a later launch
+struct MSeg {
+  float* out;
+  int32_t n;
+  int32_t first_slot;
+  int32_t nslots;
+  int32_t pad;
+};
+struct MSlot {
+  const uint8_t* in;
+  float thr;
+  int32_t add;
+};
+struct MArgs {
+  int32_t nseg;
+  int32_t tile_start[kMultiSegs + 1];
+  MSeg seg[kMultiSegs];
+  MSlot slot[kMultiSlots];
+};
+static_assert(sizeof(MArgs) <= 9600, "kernel-argument budget");
+
+__global__ __launch_bounds__(kThreads) void tbq_decode_multi_kernel(const MArgs a) {
+  __shared__ const uint8_t* s_in[kMultiSlotsPerSeg];
+  __shared__ float s_thr[kMultiSlotsPerSeg];
+  __shared__ int32_t s_add[kMultiSlotsPerSeg];
+  const int tile = blockIdx.x;
+  const int s = find_segment<kMultiSegs>(a.tile_start, a.nseg, tile);
+  float* __restrict__ op = a.seg[s].out;
+  const uint32_t n = static_cast<uint32_t>(a.seg[s].n);
+  const int s0 = a.seg[s].first_slot, ns = a.seg[s].nslots;
+  if (int(threadIdx.x) < ns) {
+    s_in[threadIdx.x] = a.slot[s0 + threadIdx.x].in;
+    s_thr[threadIdx.x] = a.slot[s0 + threadIdx.x].thr;
+    s_add[threadIdx.x] = a.slot[s0 + threadIdx.x].add;
+  }
+  __syncthreads();
+  const bool need_old = s_add[0] != 0;
+  const uint32_t full = n >> 2;
+  const uint32_t g0 = static_cast<uint32_t>(tile - a.tile_start[s]) * kTileGroups + threadIdx.x;
+  if (g0 - threadIdx.x + kTileGroups <= full) {
+    // whole tile inside the tensor: the old values and the bytes of up to 8 messages x 4 groups are requested
+    // together, then folded in message order
+    float4 acc[kIters];
+#pragma unroll
+    for (int k = 0; k < kIters; k++)
+      acc[k] = need_old ? ld4_stream(op + size_t(g0 + k * kThreads) * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int j0 = 0; j0 < ns; j0 += 8) {
+      uint32_t q[8][kIters];
+#pragma unroll
+      for (int jj = 0; jj < 8; jj++)
+#pragma unroll
+        for (int k = 0; k < kIters; k++) q[jj][k] = (j0 + jj < ns) ? s_in[j0 + jj][g0 + k * kThreads] : 0u;
+#pragma unroll
+      for (int jj = 0; jj < 8; jj++) {
+        if (j0 + jj < ns) {
+          const float thr = s_thr[j0 + jj];
+          const bool add = s_add[j0 + jj] != 0;
+#pragma unroll
+          for (int k = 0; k < kIters; k++) {
+            const float4 v = tbq_values(q[jj][k], thr);
+            if (add) {
+              acc[k].x = v.x + acc[k].x; acc[k].y = v.y + acc[k].y; acc[k].z = v.z + acc[k].z; acc[k].w = v.w + acc[k].w;
+            } else {
+              acc[k] = v;
+            }
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < kIters; k++) {
+      st4_stream(op + size_t(g0 + k * kThreads) * 4, acc[k]);
+      __asm__ volatile("" ::: "memory");
+    }
+    return;
+  }
+  for (int k = 0; k < kIters; k++) {
+    const uint32_t grp = g0 + k * kThreads;
+    const size_t e = size_t(grp) * 4;
+    const uint32_t lim = grp < full ? 4u : (grp == full ? (n & 3u) : 0u);
+    for (uint32_t i = 0; i < lim; i++) {
+      float acc = need_old ? op[e + i] : 0.f;
+      for (int j = 0; j < ns; j++) {
+        const uint32_t q = s_in[j][grp];
+        const float v = (static_cast<float>((q >> (2 * i)) & 3) - 1) * s_thr[j];
+        acc = s_add[j] ? v + acc : v;
+      }
+      op[e + i] = acc;
+    }
+  }
+}
+
 inline int32_t tiles_for(int32_t n) {
   const int64_t groups = (int64_t(n) + 3) >> 2;
   return static_cast<int32_t>((groups + kTileGroups - 1) / kTileGroups);
@@ -257,6 +361,76 @@ int launch_decode(int count, float* const* outs, const int32_t* sizes, const uin
   return HPX_OK;
 }
 
+// Plans the launches of a multi-message decode.  Messages are visited in call order; each launch takes up to
+// kMultiSegs tensors and up to kMultiSlotsPerSeg messages per tensor (kMultiSlots in all).  A message that does not
+// fit is left for a later launch together with every later message of the same tensor, so the messages of a tensor
+// are always applied in call order (launches are ordered by the stream); tensors do not overlap, so the order
+// between different tensors is immaterial.
+struct MultiGroup {
+  float* out;
+  int32_t n;
+  std::vector<int> msgs;
+};
+template <typename TilesFn>
+std::vector<MultiGroup> plan_multi_launch(int count, float* const* outs, const int32_t* sizes, std::vector<char>& done,
+                                          TilesFn tiles_of) {
+  std::vector<MultiGroup> groups;
+  std::unordered_map<float*, int> index;  // tensor -> group, or -1 once the tensor is closed for this launch
+  int used_slots = 0;
+  int64_t tiles = 0;
+  for (int j = 0; j < count; j++) {
+    if (done[j]) continue;
+    auto it = index.find(outs[j]);
+    if (it != index.end()) {
+      if (it->second < 0) continue;
+      MultiGroup& g = groups[it->second];
+      if (used_slots == kMultiSlots || int(g.msgs.size()) == kMultiSlotsPerSeg) { it->second = -1; continue; }
+      g.msgs.push_back(j);
+    } else {
+      if (used_slots == kMultiSlots || int(groups.size()) == kMultiSegs || tiles + tiles_of(sizes[j]) > INT32_MAX) {
+        index[outs[j]] = -1;
+        continue;
+      }
+      index[outs[j]] = int(groups.size());
+      groups.push_back(MultiGroup{outs[j], sizes[j], {j}});
+      tiles += tiles_of(sizes[j]);
+    }
+    used_slots++;
+    done[j] = 1;
+  }
+  return groups;
+}
+
+int launch_decode_multi(int count, float* const* outs, const int32_t* sizes, const uint8_t* const* ins,
+                        const float* thresholds, const int32_t* is_add_tos, hipStream_t st) {
+  std::vector<char> done(count, 0);
+  int left = 0;
+  for (int j = 0; j < count; j++) {
+    HPX_ARG(sizes[j] >= 0, "hpx_tbq_decode: tensor %d has negative size %d", j, sizes[j]);
+    if (sizes[j] == 0) { done[j] = 1; continue; }
+    HPX_ARG(outs[j] && ins[j], "hpx_tbq_decode: tensor %d has a null pointer", j);
+    left++;
+  }
+  MArgs a;
+  while (left > 0) {
+    const std::vector<MultiGroup> groups = plan_multi_launch(count, outs, sizes, done, tiles_for);
+    a.nseg = 0;
+    a.tile_start[0] = 0;
+    int nslots = 0;
+    for (const MultiGroup& g : groups) {
+      a.seg[a.nseg] = MSeg{g.out, g.n, nslots, static_cast<int32_t>(g.msgs.size()), 0};
+      for (int m : g.msgs) a.slot[nslots++] = MSlot{ins[m], thresholds[m], is_add_tos[m] != 0};
+      a.tile_start[a.nseg + 1] = a.tile_start[a.nseg] + tiles_for(g.n);
+      a.nseg++;
+    }
+    if (nslots == 0) { hpx::set_error("hpx_tbq_decode: could not place the remaining messages"); return HPX_ERR_ARG; }
+    left -= nslots;
+    HPX_LAUNCH("tbq_decode_multi_kernel", tbq_decode_multi_kernel, dim3(a.tile_start[a.nseg]), dim3(kThreads), st, a);
+    HPX_HIP(hipGetLastError());
+  }
+  return HPX_OK;
+}
+
 }  // namespace
 
 HPX_API int hpx_tbq_encode(int count, const float* const* grads, const int32_t* sizes,
@@ -279,6 +453,18 @@ HPX_API int hpx_tbq_decode(int count, float* const* outs, const int32_t* sizes,
   if (count == 0) return HPX_OK;
   HPX_ARG(outs && sizes && ins && thresholds && is_add_tos, "hpx_tbq_decode: null argument array");
   hipStream_t st = static_cast<hipStream_t>(stream);
+  switch (hpx::classify_outputs(count, outs, sizes)) {
+    case 0: break;
+    case 1:  // several messages accumulate into the same tensor(s): one pass per tensor
+      return launch_decode_multi(count, outs, sizes, ins, thresholds, is_add_tos, st);
+    default: {  // partially overlapping outputs: keep the reference's one-message-at-a-time order
+      for (int i = 0; i < count; i++) {
+        const int rc = launch_decode<kCapSmall>(1, outs + i, sizes + i, ins + i, thresholds + i, is_add_tos + i, st);
+        if (rc != HPX_OK) return rc;
+      }
+      return HPX_OK;
+    }
+  }
   if (count <= kCapSmall) return launch_decode<kCapSmall>(count, outs, sizes, ins, thresholds, is_add_tos, st);
   return launch_decode<kCapLarge>(count, outs, sizes, ins, thresholds, is_add_tos, st);
 }

@@ -21,6 +21,9 @@
 //   * min and max are the FIRST smallest / largest element as
 //     thrust::minmax_element returns them, which only matters for the sign of
 //     a zero extreme; it is recovered from the first zero of the tensor.
+#include <unordered_map>
+#include <vector>
+
 #include "hpx_common.h"
 
 namespace {
@@ -432,6 +435,153 @@ __global__ __launch_bounds__(kThreads) void terngrad_decode_kernel(const DecArgs
   }
 }
 
+// ---- several messages into one tensor ---------------------------------------
+// The reference's root path hands terngrad_r_body the same output tensor once per
+// gathered message (hp_cuda.cpp:421-439) and applies them one after the other.
+// Here a tensor's messages are applied in one pass in call order: same sequence
+// of fp32 operations per element, one read and one write of the tensor.
+constexpr int kMultiSegs = 64;
+constexpr int kMultiSlots = 448;
+constexpr int kMultiSlotsPerSeg = 32;  // header fields of one tensor's messages are staged in LDS
+struct MSeg {
+  float* out;
+  int32_t out_size;
+  int32_t first_slot;
+  int32_t nslots;
+  int32_t pad;
+};
+struct MSlot {
+  const uint8_t* in;
+  int32_t in_size;
+  int32_t add;
+};
+struct MArgs {
+  int32_t nseg;
+  int32_t tile_start[kMultiSegs + 1];
+  MSeg seg[kMultiSegs];
+  MSlot slot[kMultiSlots];
+  uint32_t* status;
+};
+static_assert(sizeof(MArgs) <= 9600, "kernel-argument budget");
+
+__device__ __forceinline__ uint32_t code_at(const uint8_t* __restrict__ pay, size_t i, uint32_t bits) {
+  const uint32_t dpb = 8u / bits;
+  return (uint32_t(pay[i / dpb]) >> ((i % dpb) * bits)) & ((1u << bits) - 1u);
+}
+
+__global__ __launch_bounds__(kThreads) void terngrad_decode_multi_kernel(const MArgs a) {
+  __shared__ float s_mn[kMultiSlotsPerSeg], s_gap[kMultiSlotsPerSeg];
+  __shared__ uint32_t s_cnt[kMultiSlotsPerSeg], s_bits[kMultiSlotsPerSeg];
+  __shared__ int32_t s_add[kMultiSlotsPerSeg];
+  __shared__ const uint8_t* s_pay[kMultiSlotsPerSeg];
+  const int tile = blockIdx.x;
+  const int s = find_segment<kMultiSegs>(a.tile_start, a.nseg, tile);
+  float* __restrict__ op = a.seg[s].out;
+  const int s0 = a.seg[s].first_slot, ns = a.seg[s].nslots;
+  if (int(threadIdx.x) < ns) {
+    const int j = threadIdx.x;
+    const uint8_t* in = a.slot[s0 + j].in;
+    const uint32_t bits = in[0], tail = in[1];
+    uint32_t mb = 0, xb = 0;
+    for (int i = 0; i < 4; i++) {
+      mb |= uint32_t(in[2 + i]) << (8 * i);
+      xb |= uint32_t(in[6 + i]) << (8 * i);
+    }
+    uint32_t cnt = 0;
+    float gap = 0.f;
+    if (bits == 1 || bits == 2 || bits == 4 || bits == 8) {
+      gap = (__uint_as_float(xb) - __uint_as_float(mb)) / (float(1 << bits) - 1.0f);
+      int64_t c = int64_t(a.slot[s0 + j].in_size - 10) * int64_t(8 / bits) - int64_t(tail);
+      if (c > a.seg[s].out_size) c = a.seg[s].out_size;
+      cnt = c > 0 ? uint32_t(c) : 0u;
+    } else if (tile == a.tile_start[s]) {
+      atomicOr(a.status, 1u);
+    }
+    s_mn[j] = __uint_as_float(mb);
+    s_gap[j] = gap;
+    s_cnt[j] = cnt;
+    s_bits[j] = cnt ? bits : 8u;
+    s_add[j] = a.slot[s0 + j].add;
+    s_pay[j] = in + 10;
+  }
+  __syncthreads();
+  const uint32_t n = static_cast<uint32_t>(a.seg[s].out_size);
+  const bool need_old = s_add[0] != 0;
+  const uint32_t g0 = static_cast<uint32_t>(tile - a.tile_start[s]) * uint32_t(kThreads * kDIters) + threadIdx.x;
+  bool all_cover = true;  // every message covers the whole tensor (the normal case)
+  for (int j = 0; j < ns; j++) all_cover = all_cover && s_cnt[j] == n;
+  if (all_cover && uint64_t(g0 - threadIdx.x + kThreads * kDIters) * 4 <= n) {
+    // Whole tile, every message complete: old values and the code bytes of up to 8 messages x 4 groups are
+    // requested together, then folded in message order.
+    float4 acc[kDIters];
+#pragma unroll
+    for (int k = 0; k < kDIters; k++)
+      acc[k] = need_old ? ld4_stream(op + size_t(g0 + k * kThreads) * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int j0 = 0; j0 < ns; j0 += 8) {
+      uint32_t raw[8][kDIters];
+#pragma unroll
+      for (int jj = 0; jj < 8; jj++)
+#pragma unroll
+        for (int k = 0; k < kDIters; k++) {
+          raw[jj][k] = 0;
+          if (j0 + jj < ns) {
+            const size_t e = size_t(g0 + k * kThreads) * 4;
+            const uint32_t bits = s_bits[j0 + jj];
+            const uint8_t* __restrict__ pay = s_pay[j0 + jj];
+            if (bits == 1) raw[jj][k] = (uint32_t(pay[e >> 3]) >> (e & 4)) & 0xFu;
+            else if (bits == 2) raw[jj][k] = pay[e >> 2];
+            else if (bits == 4) raw[jj][k] = group_bits<4>(pay, e);
+            else raw[jj][k] = group_bits<8>(pay, e);
+          }
+        }
+#pragma unroll
+      for (int jj = 0; jj < 8; jj++) {
+        if (j0 + jj < ns) {
+          const uint32_t bits = s_bits[j0 + jj];
+          const float gap = s_gap[j0 + jj], mn = s_mn[j0 + jj];
+          const bool add = s_add[j0 + jj] != 0;
+#pragma unroll
+          for (int k = 0; k < kDIters; k++) {
+            float4 v;
+            if (bits == 1) v = group_values<1>(raw[jj][k], gap, mn);
+            else if (bits == 2) v = group_values<2>(raw[jj][k], gap, mn);
+            else if (bits == 4) v = group_values<4>(raw[jj][k], gap, mn);
+            else v = group_values<8>(raw[jj][k], gap, mn);
+            if (add) {
+              acc[k].x = v.x + acc[k].x; acc[k].y = v.y + acc[k].y; acc[k].z = v.z + acc[k].z; acc[k].w = v.w + acc[k].w;
+            } else {
+              acc[k] = v;
+            }
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < kDIters; k++) {
+      st4_stream(op + size_t(g0 + k * kThreads) * 4, acc[k]);
+      __asm__ volatile("" ::: "memory");
+    }
+    return;
+  }
+  for (int k = 0; k < kDIters; k++) {
+    const size_t e = size_t(g0 + k * kThreads) * 4;
+    if (e >= n) break;
+    const int lim = (n - e >= 4) ? 4 : int(n - e);
+    for (int i = 0; i < lim; i++) {
+      float acc = need_old ? op[e + i] : 0.f;
+      bool touched = need_old;
+      for (int j = 0; j < ns; j++) {
+        if (e + i < s_cnt[j]) {
+          const float v = float(int(code_at(s_pay[j], e + i, s_bits[j]))) * s_gap[j] + s_mn[j];  // terngrad_body.h:127, :158
+          acc = s_add[j] ? v + acc : v;
+          touched = true;
+        }
+      }
+      if (touched) op[e + i] = acc;
+    }
+  }
+}
+
 inline int32_t ceil_div(int64_t a, int64_t b) { return static_cast<int32_t>((a + b - 1) / b); }
 
 template <int CAP>
@@ -508,6 +658,79 @@ int launch_decode(int count, float* const* outs, const int32_t* out_sizes, const
   return HPX_OK;
 }
 
+// Plans the launches of a multi-message decode.  Messages are visited in call order; each launch takes up to
+// kMultiSegs tensors and up to kMultiSlotsPerSeg messages per tensor (kMultiSlots in all).  A message that does not
+// fit is left for a later launch together with every later message of the same tensor, so the messages of a tensor
+// are always applied in call order (launches are ordered by the stream); tensors do not overlap, so the order
+// between different tensors is immaterial.
+struct MultiGroup {
+  float* out;
+  int32_t n;
+  std::vector<int> msgs;
+};
+template <typename TilesFn>
+std::vector<MultiGroup> plan_multi_launch(int count, float* const* outs, const int32_t* sizes, std::vector<char>& done,
+                                          TilesFn tiles_of) {
+  std::vector<MultiGroup> groups;
+  std::unordered_map<float*, int> index;  // tensor -> group, or -1 once the tensor is closed for this launch
+  int used_slots = 0;
+  int64_t tiles = 0;
+  for (int j = 0; j < count; j++) {
+    if (done[j]) continue;
+    auto it = index.find(outs[j]);
+    if (it != index.end()) {
+      if (it->second < 0) continue;
+      MultiGroup& g = groups[it->second];
+      if (used_slots == kMultiSlots || int(g.msgs.size()) == kMultiSlotsPerSeg) { it->second = -1; continue; }
+      g.msgs.push_back(j);
+    } else {
+      if (used_slots == kMultiSlots || int(groups.size()) == kMultiSegs || tiles + tiles_of(sizes[j]) > INT32_MAX) {
+        index[outs[j]] = -1;
+        continue;
+      }
+      index[outs[j]] = int(groups.size());
+      groups.push_back(MultiGroup{outs[j], sizes[j], {j}});
+      tiles += tiles_of(sizes[j]);
+    }
+    used_slots++;
+    done[j] = 1;
+  }
+  return groups;
+}
+
+int launch_decode_multi(int count, float* const* outs, const int32_t* out_sizes, const uint8_t* const* ins,
+                        const int32_t* in_sizes, const int32_t* is_add_tos, uint32_t* status, hipStream_t st) {
+  std::vector<char> done(count, 0);
+  int left = 0;
+  for (int j = 0; j < count; j++) {
+    HPX_ARG(out_sizes[j] >= 0 && in_sizes[j] >= 10, "hpx_terngrad_decode: message %d: out_size %d, in_size %d", j,
+            out_sizes[j], in_sizes[j]);
+    if (out_sizes[j] == 0) { done[j] = 1; continue; }
+    HPX_ARG(outs[j] && ins[j], "hpx_terngrad_decode: message %d has a null pointer", j);
+    left++;
+  }
+  MArgs a;
+  a.status = status;
+  auto tiles_of = [](int32_t n) { return ceil_div(n, kDecTile); };
+  while (left > 0) {
+    const std::vector<MultiGroup> groups = plan_multi_launch(count, outs, out_sizes, done, tiles_of);
+    a.nseg = 0;
+    a.tile_start[0] = 0;
+    int nslots = 0;
+    for (const MultiGroup& g : groups) {
+      a.seg[a.nseg] = MSeg{g.out, g.n, nslots, static_cast<int32_t>(g.msgs.size()), 0};
+      for (int m : g.msgs) a.slot[nslots++] = MSlot{ins[m], in_sizes[m], is_add_tos[m] != 0};
+      a.tile_start[a.nseg + 1] = a.tile_start[a.nseg] + tiles_of(g.n);
+      a.nseg++;
+    }
+    if (nslots == 0) { hpx::set_error("hpx_terngrad_decode: could not place the remaining messages"); return HPX_ERR_ARG; }
+    left -= nslots;
+    HPX_LAUNCH("terngrad_decode_multi_kernel", terngrad_decode_multi_kernel, dim3(a.tile_start[a.nseg]), dim3(kThreads), st, a);
+    HPX_HIP(hipGetLastError());
+  }
+  return HPX_OK;
+}
+
 }  // namespace
 
 HPX_API int hpx_terngrad_encode(int count, const float* const* ins, const int32_t* in_sizes,
@@ -564,6 +787,18 @@ HPX_API int hpx_terngrad_decode(int count, float* const* outs, const int32_t* ou
   int rc = hpx::ensure_workspace(ws, 0);
   if (rc != HPX_OK) return rc;
   uint32_t* status = ws->state + hpx::kStatusWord;
+  switch (hpx::classify_outputs(count, outs, out_sizes)) {
+    case 0: break;
+    case 1:  // several messages accumulate into the same tensor(s): one pass per tensor
+      return launch_decode_multi(count, outs, out_sizes, ins, in_sizes, is_add_tos, status, st);
+    default: {  // partially overlapping outputs: keep the reference's one-message-at-a-time order
+      for (int i = 0; i < count; i++) {
+        const int rc1 = launch_decode<kCapSmall>(1, outs + i, out_sizes + i, ins + i, in_sizes + i, is_add_tos + i, status, st);
+        if (rc1 != HPX_OK) return rc1;
+      }
+      return HPX_OK;
+    }
+  }
   if (count <= kCapSmall) return launch_decode<kCapSmall>(count, outs, out_sizes, ins, in_sizes, is_add_tos, status, st);
   return launch_decode<kCapLarge>(count, outs, out_sizes, ins, in_sizes, is_add_tos, status, st);
 }
