@@ -166,7 +166,7 @@ def main():
     sec_dec = timed(torch, only(4), max(20, args.steps // 4), 5)
 
     kt = kernel_times(torch, capi, step,
-                      ["terngrad_minmax_kernel", "terngrad_finalize_kernel", "terngrad_quant_kernel", "terngrad_decode_kernel"])
+                      ["terngrad_minmax_kernel", "terngrad_quant_kernel", "terngrad_decode_kernel"])
     alg_bytes = {  # algorithmic bytes per launch: every distinct input byte once, every output byte once
         "terngrad_minmax_kernel": 4.0 * n,
         "terngrad_quant_kernel": 4.0 * n + msg_bytes,

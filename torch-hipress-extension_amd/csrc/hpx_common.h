@@ -59,6 +59,11 @@ struct Workspace {
   size_t dev_bytes = 0;
   uint32_t* state = nullptr;
   uint8_t* pinned = nullptr;
+  // Epoch-tagged 64-bit reduction slots (see ensure_slots): memory that only ever
+  // holds (epoch << 32 | key) words, so a call with a newer epoch needs no reset.
+  uint64_t* slots = nullptr;
+  size_t slot_words = 0;
+  uint32_t epoch = 0;
 };
 constexpr size_t kStateWords = 4096;       // 16 KiB
 constexpr size_t kStatusWord = kStateWords - 16;  // sticky flags live here
@@ -69,6 +74,8 @@ constexpr size_t kPinnedBytes = 1 << 16;
 // the call needs (may wait for the stream when the block has to grow).
 Workspace* workspace_record(hipStream_t stream);
 int ensure_workspace(Workspace* ws, size_t dev_bytes);
+// At least `words` zero-initialised-at-allocation 64-bit slots, never used for anything else.
+int ensure_slots(Workspace* ws, size_t words);
 
 uint64_t clock_seed();
 

@@ -96,6 +96,19 @@ void prof_end(hipStream_t st) {
   if (!g_prof_recs.empty()) (void)hipEventRecord(g_prof_recs.back().stop, st);
 }
 
+int ensure_slots(Workspace* ws, size_t words) {
+  if (words <= ws->slot_words) return HPX_OK;
+  HPX_HIP(hipStreamSynchronize(ws->stream));
+  if (ws->slots) HPX_HIP(hipFree(ws->slots));
+  ws->slots = nullptr;
+  ws->slot_words = 0;
+  const size_t want = words < 4096 ? 4096 : words * 2;
+  HPX_HIP(hipMalloc(reinterpret_cast<void**>(&ws->slots), want * sizeof(uint64_t)));
+  HPX_HIP(hipMemset(ws->slots, 0, want * sizeof(uint64_t)));  // epoch 0 is never used by a call
+  ws->slot_words = want;
+  return HPX_OK;
+}
+
 size_t stream_store_max_bytes() {
   static const size_t v = [] {
     const char* e = std::getenv("HPX_STREAM_STORE_MAX_MB");
@@ -146,6 +159,7 @@ HPX_API int hpx_release_workspaces(void) {
     if (hipSetDevice(ws->device) != hipSuccess) { rc = HPX_ERR_HIP; continue; }
     if (ws->dev && hipFree(ws->dev) != hipSuccess) rc = HPX_ERR_HIP;
     if (ws->state && hipFree(ws->state) != hipSuccess) rc = HPX_ERR_HIP;
+    if (ws->slots && hipFree(ws->slots) != hipSuccess) rc = HPX_ERR_HIP;
     if (ws->pinned && hipHostFree(ws->pinned) != hipSuccess) rc = HPX_ERR_HIP;
   }
   hpx::g_ws.clear();

@@ -38,13 +38,11 @@ constexpr int kQIters = 4;                                   // units per lane
 constexpr int kDIters = 4;                                   // 4-element groups per lane in decode
 constexpr int kDecTile = kThreads * kDIters * 4;
 
-struct Partial {
-  float mn, mx;
-  uint32_t has_zero;
-};
-struct Scalars {
-  float mn, gi;
-};
+// Per tensor, 3 x 64 epoch-tagged slots: [0,64) largest ordered key of x, [64,128)
+// largest complemented key (i.e. the minimum), [128,192) largest complemented
+// index of a tile that holds a zero (i.e. the first such tile).
+constexpr int kSlotWays = 64;
+constexpr int kSlotsPerTensor = 3 * kSlotWays;
 
 struct EncSeg {
   const float* x;
@@ -61,8 +59,8 @@ struct EncArgs {
   int32_t nseg;
   int32_t tile_start[CAP + 1];
   EncSeg seg[CAP];
-  Partial* partials;    // one per reduction tile of this launch
-  Scalars* scalars;     // one per segment
+  uint64_t* slots;      // kSlotsPerTensor words per segment of this launch
+  uint32_t epoch;       // tag of this call; slots carrying an older tag are stale
 };
 struct DecSeg {
   float* out;
@@ -125,6 +123,27 @@ __device__ __forceinline__ void acc3(float v, float& mn, float& mx, float& am) {
   am = a < am ? a : am;
 }
 
+// Order-preserving map of a float onto unsigned integers, and back.
+__device__ __forceinline__ uint32_t okey(float f) {
+  const uint32_t b = __float_as_uint(f);
+  return b ^ ((b >> 31) ? 0xFFFFFFFFu : 0x80000000u);
+}
+__device__ __forceinline__ float from_okey(uint32_t k) {
+  return __uint_as_float(k ^ ((k >> 31) ? 0x80000000u : 0xFFFFFFFFu));
+}
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) { uint32_t t = __shfl_xor(v, o, 64); v = t > v ? t : v; }
+  return v;
+}
+
+// Pass 1 of encode.  Each workgroup reduces one 8192-element tile and folds its
+// result into one of 64 slots of its tensor with a 64-bit atomic max on
+// (epoch << 32 | key).  Tiles spread over the slots, so about n_tiles/64 atomics
+// meet on one address over the whole run of the kernel (same-address atomics
+// from different workgroups cost ~37 ns each), and because a newer epoch beats
+// any older word the slots are never cleared.  The quantise kernel folds the 64
+// slots itself, so no separate reduction launch is needed.
 template <int CAP>
 __global__ __launch_bounds__(kThreads) void terngrad_minmax_kernel(const EncArgs<CAP> a) {
   const int tile = blockIdx.x;
@@ -149,35 +168,42 @@ __global__ __launch_bounds__(kThreads) void terngrad_minmax_kernel(const EncArgs
   }
   uint32_t z = (am == 0.0f) ? 0u : 1u;  // 0 when this tile holds a zero
   block_reduce(mn, mx, z);
-  if (threadIdx.x == 0) a.partials[tile] = Partial{mn, mx, z == 0u ? 1u : 0u};
+  if (threadIdx.x == 0) {
+    unsigned long long* sl = reinterpret_cast<unsigned long long*>(a.slots) + size_t(s) * kSlotsPerTensor + (t % kSlotWays);
+    const unsigned long long ep = static_cast<unsigned long long>(a.epoch) << 32;
+    atomicMax(sl, ep | okey(mx));
+    atomicMax(sl + kSlotWays, ep | (~okey(mn)));
+    if (z == 0u) atomicMax(sl + 2 * kSlotWays, ep | (0xFFFFFFFFu - t));
+  }
 }
 
-// One workgroup per tensor folds that tensor's partials, derives the scalars
-// and writes the header.  (A last-arriving-workgroup scheme inside the
-// reduction kernel would save this launch, but thousands of workgroups bumping
-// one arrival counter serialise at ~40 ns each across the XCDs.)
+// Prologue of the quantise kernel: folds the tensor's 64 slots into min and max
+// (thrust::minmax_element semantics: a zero extreme takes the sign of the first
+// zero element of the tensor), derives gap and 1/(gap + 1e-8) as the reference
+// does (terngrad_body.h:204-206) and, in the workgroup of the tensor's first tile,
+// writes the 10-byte header (terngrad_body.h:219-224).  Every workgroup repeats
+// this; it reads 1.5 KB from L2.
 template <int CAP>
-__global__ __launch_bounds__(kThreads) void terngrad_finalize_kernel(const EncArgs<CAP> a) {
-  const int s = blockIdx.x;
+__device__ __forceinline__ void load_scalars(const EncArgs<CAP>& a, int s, bool first_tile, float& mn_out, float& gi_out) {
+  __shared__ uint32_t s_k[3];
   const float* __restrict__ xp = a.seg[s].x;
   const uint32_t n = static_cast<uint32_t>(a.seg[s].n);
-  const int ntiles = a.tile_start[s + 1] - a.tile_start[s];
-  float mn, mx;
-  const Partial* pp = a.partials + a.tile_start[s];
-  mn = __builtin_inff(); mx = -__builtin_inff();
-  uint32_t first_zero_tile = 0xFFFFFFFFu;
-#pragma unroll 4
-  for (int i = threadIdx.x; i < ntiles; i += kThreads) {
-    const float pmn = pp[i].mn, pmx = pp[i].mx;
-    const uint32_t hz = pp[i].has_zero;
-    mn = pmn < mn ? pmn : mn;
-    mx = pmx > mx ? pmx : mx;
-    if (hz && uint32_t(i) < first_zero_tile) first_zero_tile = uint32_t(i);
+  if (threadIdx.x < kWave) {
+    const unsigned long long* sl = reinterpret_cast<const unsigned long long*>(a.slots) + size_t(s) * kSlotsPerTensor + threadIdx.x;
+    const unsigned long long vx = sl[0], vn = sl[kSlotWays], vz = sl[2 * kSlotWays];
+    uint32_t kx = (uint32_t(vx >> 32) == a.epoch) ? uint32_t(vx) : 0u;
+    uint32_t kn = (uint32_t(vn >> 32) == a.epoch) ? uint32_t(vn) : 0u;
+    uint32_t kz = (uint32_t(vz >> 32) == a.epoch) ? uint32_t(vz) : 0u;
+    kx = wave_max_u32(kx);
+    kn = wave_max_u32(kn);
+    kz = wave_max_u32(kz);
+    if (threadIdx.x == 0) { s_k[0] = kx; s_k[1] = kn; s_k[2] = kz; }
   }
-  block_reduce(mn, mx, first_zero_tile);
-  if ((mn == 0.0f || mx == 0.0f) && first_zero_tile != 0xFFFFFFFFu) {
-    // A zero extreme takes the sign of the first zero element of the tensor.
-    const uint32_t b0 = first_zero_tile * uint32_t(kRedTile);
+  __syncthreads();
+  float mx = from_okey(s_k[0]), mn = from_okey(~s_k[1]);
+  const uint32_t kz = s_k[2];
+  if ((mn == 0.0f || mx == 0.0f) && kz != 0u) {
+    const uint32_t b0 = (0xFFFFFFFFu - kz) * uint32_t(kRedTile);
     const uint32_t b1 = (n - b0 < uint32_t(kRedTile)) ? n : b0 + uint32_t(kRedTile);
     uint32_t first = 0xFFFFFFFFu;
     for (uint32_t e = b0 + threadIdx.x; e < b1; e += kThreads)
@@ -190,10 +216,11 @@ __global__ __launch_bounds__(kThreads) void terngrad_finalize_kernel(const EncAr
       if (mx == 0.0f) mx = zv;
     }
   }
-  if (threadIdx.x == 0) {
-    const uint32_t bits = a.seg[s].bits;
-    const float gap = (mx - mn) / (float(1 << bits) - 1.0f);
-    const float gi = static_cast<float>(1.0 / (static_cast<double>(gap) + 1e-8));
+  const uint32_t bits = a.seg[s].bits;
+  const float gap = (mx - mn) / (float(1 << bits) - 1.0f);
+  gi_out = static_cast<float>(1.0 / (static_cast<double>(gap) + 1e-8));
+  mn_out = mn;
+  if (first_tile && threadIdx.x == 0) {
     const uint32_t dpb = 8u / bits;
     uint32_t tail = n % dpb;
     tail = tail == 0 ? 0 : dpb - tail;
@@ -206,7 +233,6 @@ __global__ __launch_bounds__(kThreads) void terngrad_finalize_kernel(const EncAr
       o[2 + i] = uint8_t(mb >> (8 * i));
       o[6 + i] = uint8_t(xb >> (8 * i));
     }
-    a.scalars[s] = Scalars{mn, gi};
   }
 }
 
@@ -231,7 +257,7 @@ __device__ __forceinline__ uint32_t quant_one(float x, float mn, float gi, uint3
 // One tile of the quantise stream.  A unit is UNIT = max(4, 8/B) consecutive
 // elements owned by one lane per step; it packs into BPU = UNIT*B/8 bytes.
 template <int B, bool RANDOM>
-__device__ __forceinline__ void quant_tile(const EncSeg& sg, const Scalars sc, uint32_t tile_in_seg) {
+__device__ __forceinline__ void quant_tile(const EncSeg& sg, const float mn, const float gi, uint32_t tile_in_seg) {
   constexpr int DPB = 8 / B;
   constexpr int UNIT = DPB > 4 ? DPB : 4;
   constexpr int BPU = UNIT / DPB;
@@ -240,7 +266,6 @@ __device__ __forceinline__ void quant_tile(const EncSeg& sg, const Scalars sc, u
   uint8_t* __restrict__ pay = sg.out + 10;
   const uint32_t n = static_cast<uint32_t>(sg.n);
   const uint32_t nbytes = n / DPB;  // bytes the reference's transform covers
-  const float mn = sc.mn, gi = sc.gi;
   const uint32_t u0 = tile_in_seg * uint32_t(kThreads * kQIters) + threadIdx.x;
 
   // Draw for slot j of byte (u*BPU + jb): A_{j+2} * (seed + byte) + C_{j+2}.
@@ -314,8 +339,8 @@ __device__ __forceinline__ void quant_tile(const EncSeg& sg, const Scalars sc, u
 }
 
 template <int B>
-__device__ __forceinline__ void quant_dispatch(const EncSeg& sg, const Scalars sc, uint32_t t) {
-  if (sg.random) quant_tile<B, true>(sg, sc, t); else quant_tile<B, false>(sg, sc, t);
+__device__ __forceinline__ void quant_dispatch(const EncSeg& sg, float mn, float gi, uint32_t t) {
+  if (sg.random) quant_tile<B, true>(sg, mn, gi, t); else quant_tile<B, false>(sg, mn, gi, t);
 }
 
 // tile_start here counts quantise tiles (kThreads*kQIters units each).
@@ -323,13 +348,14 @@ template <int CAP>
 __global__ __launch_bounds__(kThreads) void terngrad_quant_kernel(const EncArgs<CAP> a) {
   const int tile = blockIdx.x;
   const int s = find_segment<CAP>(a.tile_start, a.nseg, tile);
-  const Scalars sc = a.scalars[s];
   const uint32_t t = static_cast<uint32_t>(tile - a.tile_start[s]);
+  float mn, gi;
+  load_scalars<CAP>(a, s, t == 0, mn, gi);
   switch (a.seg[s].bits) {
-    case 1: quant_dispatch<1>(a.seg[s], sc, t); break;
-    case 2: quant_dispatch<2>(a.seg[s], sc, t); break;
-    case 4: quant_dispatch<4>(a.seg[s], sc, t); break;
-    default: quant_dispatch<8>(a.seg[s], sc, t); break;
+    case 1: quant_dispatch<1>(a.seg[s], mn, gi, t); break;
+    case 2: quant_dispatch<2>(a.seg[s], mn, gi, t); break;
+    case 4: quant_dispatch<4>(a.seg[s], mn, gi, t); break;
+    default: quant_dispatch<8>(a.seg[s], mn, gi, t); break;
   }
 }
 
@@ -587,16 +613,15 @@ inline int32_t ceil_div(int64_t a, int64_t b) { return static_cast<int32_t>((a +
 template <int CAP>
 int launch_encode(int count, const float* const* ins, const int32_t* in_sizes, uint8_t* const* outs,
                   const int32_t* out_sizes, const uint8_t* bitwidths, const int32_t* enable_randoms,
-                  const uint64_t* seeds, Scalars* scal_base, Partial* part_base, hipStream_t st) {
+                  const uint64_t* seeds, uint64_t* slot_base, uint32_t epoch, hipStream_t st) {
   EncArgs<CAP> a;
   int i = 0;
-  size_t part_off = 0;
   while (i < count) {
     const int first = i;
     a.nseg = 0;
     a.tile_start[0] = 0;
-    a.partials = part_base + part_off;
-    a.scalars = scal_base + first;
+    a.slots = slot_base + size_t(first) * kSlotsPerTensor;
+    a.epoch = epoch;
     int32_t qstart[CAP + 1];
     qstart[0] = 0;
     while (i < count && a.nseg < CAP) {
@@ -616,9 +641,6 @@ int launch_encode(int count, const float* const* ins, const int32_t* in_sizes, u
     }
     HPX_LAUNCH("terngrad_minmax_kernel", terngrad_minmax_kernel<CAP>, dim3(a.tile_start[a.nseg]), dim3(kThreads), st, a);
     HPX_HIP(hipGetLastError());
-    HPX_LAUNCH("terngrad_finalize_kernel", terngrad_finalize_kernel<CAP>, dim3(a.nseg), dim3(kThreads), st, a);
-    HPX_HIP(hipGetLastError());
-    part_off += size_t(a.tile_start[a.nseg]);
     for (int k = 0; k <= a.nseg; k++) a.tile_start[k] = qstart[k];
     HPX_LAUNCH("terngrad_quant_kernel", terngrad_quant_kernel<CAP>, dim3(a.tile_start[a.nseg]), dim3(kThreads), st, a);
     HPX_HIP(hipGetLastError());
@@ -742,7 +764,6 @@ HPX_API int hpx_terngrad_encode(int count, const float* const* ins, const int32_
   if (count == 0) return HPX_OK;
   HPX_ARG(ins && in_sizes && outs && out_sizes && bitwidths && enable_randoms,
           "hpx_terngrad_encode: null argument array");
-  int64_t red_tiles_total = 0;
   for (int i = 0; i < count; i++) {
     const uint8_t b = bitwidths[i];
     if (!(b == 1 || b == 2 || b == 4 || b == 8)) {
@@ -754,23 +775,27 @@ HPX_API int hpx_terngrad_encode(int count, const float* const* ins, const int32_
     const int64_t need = 10 + (int64_t(in_sizes[i]) + 8 / b - 1) / (8 / b);
     HPX_ARG(out_sizes[i] >= need, "hpx_terngrad_encode: tensor %d needs %lld output bytes, got %d", i,
             static_cast<long long>(need), out_sizes[i]);
-    red_tiles_total += ceil_div(in_sizes[i], kRedTile);
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
   hpx::Workspace* ws = hpx::workspace_record(st);
   if (!ws) return HPX_ERR_HIP;
   std::lock_guard<std::mutex> lock(ws->mu);
-  const size_t scal_bytes = (size_t(count) * sizeof(Scalars) + 255) & ~size_t(255);
-  int rc = hpx::ensure_workspace(ws, scal_bytes + size_t(red_tiles_total) * sizeof(Partial));
+  int rc = hpx::ensure_workspace(ws, 0);
   if (rc != HPX_OK) return rc;
-  Scalars* scal_base = reinterpret_cast<Scalars*>(ws->dev);
-  Partial* part_base = reinterpret_cast<Partial*>(ws->dev + scal_bytes);
+  rc = hpx::ensure_slots(ws, size_t(count) * kSlotsPerTensor);
+  if (rc != HPX_OK) return rc;
+  if (++ws->epoch == 0) {
+    // The 32-bit tag wrapped: start over from cleared slots.
+    HPX_HIP(hipStreamSynchronize(st));
+    HPX_HIP(hipMemset(ws->slots, 0, ws->slot_words * sizeof(uint64_t)));
+    ws->epoch = 1;
+  }
 
   if (count <= kCapSmall)
-    return launch_encode<kCapSmall>(count, ins, in_sizes, outs, out_sizes, bitwidths, enable_randoms, seeds, scal_base,
-                                    part_base, st);
-  return launch_encode<kCapLarge>(count, ins, in_sizes, outs, out_sizes, bitwidths, enable_randoms, seeds, scal_base,
-                                  part_base, st);
+    return launch_encode<kCapSmall>(count, ins, in_sizes, outs, out_sizes, bitwidths, enable_randoms, seeds, ws->slots,
+                                    ws->epoch, st);
+  return launch_encode<kCapLarge>(count, ins, in_sizes, outs, out_sizes, bitwidths, enable_randoms, seeds, ws->slots,
+                                  ws->epoch, st);
 }
 
 HPX_API int hpx_terngrad_decode(int count, float* const* outs, const int32_t* out_sizes,
