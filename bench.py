@@ -166,8 +166,9 @@ def main():
     sec_dec = timed(torch, only(4), max(20, args.steps // 4), 5)
 
     kt = kernel_times(torch, capi, step,
-                      ["terngrad_minmax_kernel", "terngrad_quant_kernel", "terngrad_decode_kernel"])
+                      ["terngrad_resident_kernel", "terngrad_minmax_kernel", "terngrad_quant_kernel", "terngrad_decode_kernel"])
     alg_bytes = {  # algorithmic bytes per launch: every distinct input byte once, every output byte once
+        "terngrad_resident_kernel": 4.0 * n + msg_bytes,   # x once in, message out
         "terngrad_minmax_kernel": 4.0 * n,
         "terngrad_quant_kernel": 4.0 * n + msg_bytes,
         "terngrad_decode_kernel": msg_bytes + 4.0 * n,
@@ -305,7 +306,7 @@ def extra(torch, np, capi, L, stream, gen):
     r.copy_(r0)
     scrub.sum()
     kt = kernel_times(torch, capi, gd, ["gd_sample_kernel", "gd_select_kernel", "gd_threshold_kernel", "gd_stream_kernel", "gd_scan_kernel",
-                                        "gd_expand_kernel", "gd_gather_kernel", "gd_sort_scatter_kernel"], reps=1)
+                                        "gd_expand_kernel", "gd_sort_pass_kernel"], reps=1)
     dout = torch.zeros(n, device="cuda")
     gdr = Call(L.hpx_gd_decode, 1, capi.ptr_array([out.data_ptr()]), capi.i32_array([out.numel()]),
                capi.ptr_array([dout.data_ptr()]), capi.i32_array([n]), capi.i32_array([1]), stream)

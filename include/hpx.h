@@ -24,9 +24,7 @@
  *     Entry points may be called from several host threads; calls that share a
  *     stream are serialised while they enqueue.
  *   - Sizes are int32 element/byte counts exactly as in the reference.
- *   - Tuning: the environment variable HPX_STREAM_STORE_MAX_MB (read once) sets the
- *     output size up to which the write-only decoders use streaming stores
- *     (default 128).
+ *   - Tuning options: see hpx_set_option.
  */
 #ifndef HPX_H_
 #define HPX_H_
@@ -52,6 +50,22 @@ const char* hpx_last_error(void);
  * No call may be in flight.  No counterpart in the reference (its scratch is
  * the caller's output buffer). */
 int hpx_release_workspaces(void);
+
+/* ---- tuning options -------------------------------------------------------
+ * No counterpart in the reference.  An option starts from the environment
+ * variable HPX_<NAME IN CAPITALS> when that is set, else from its default, and
+ * can be changed at any time (it applies to calls made afterwards):
+ *   "stream_store_max_bytes"  total output size up to which the write-only
+ *                             decoders use streaming stores (default 128 MiB)
+ *   "terngrad_resident_min"   smallest tensor, in elements, that
+ *                             hpx_terngrad_encode sends through its
+ *                             single-launch resident kernel (default 2^21;
+ *                             negative: never)
+ *   "terngrad_barrier_ms"     bound on that kernel's grid-barrier wait
+ *                             (default 2000)
+ * Unknown names return HPX_ERR_ARG. */
+int hpx_set_option(const char* name, int64_t value);
+int hpx_get_option(const char* name, int64_t* value);
 
 /* ---- measurement aid ------------------------------------------------------
  * No counterpart in the reference.  While enabled, every kernel the library
@@ -101,7 +115,14 @@ int hpx_tbq_decode(int count, float* const* outs, const int32_t* sizes,
  * seed from the wall clock inside the body (terngrad_body.h:247-251); pass
  * seeds == NULL for that behaviour, or an array of `count` values to fix it.
  * Returns -1 without launching if any bitwidth is not 1, 2, 4 or 8
- * (terngrad_body.h:207-212). */
+ * (terngrad_body.h:207-212).
+ * A tensor between "terngrad_resident_min" and about 33M elements (16M at
+ * 1 bit) is encoded by one launch that keeps it in registers and LDS between the
+ * min/max pass and the quantise pass, with a grid-wide barrier in between.  That
+ * barrier needs every CU of the device to be reachable from `stream` (no CU
+ * mask); its wait is bounded, and if it ever expires the call's output is
+ * invalid, the NEXT hpx_terngrad_encode on the stream returns -2 once and the
+ * stream falls back to the two-launch path for good. */
 int hpx_terngrad_encode(int count, const float* const* ins, const int32_t* in_sizes,
                         uint8_t* const* outs, const int32_t* out_sizes,
                         const uint8_t* bitwidths, const int32_t* enable_randoms,

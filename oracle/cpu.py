@@ -34,6 +34,8 @@ def lib():
         L.orc_u01_from_u32.argtypes = [C.c_uint32]
         L.orc_u01_shortcut_mismatches.restype = C.c_uint64
         L.orc_u01_shortcut_mismatches.argtypes = [C.c_uint32, C.c_uint32]
+        L.orc_u01_fp32_mismatches.restype = C.c_uint64
+        L.orc_u01_fp32_mismatches.argtypes = [C.c_uint32, C.c_uint32]
         L.orc_tbq_encode.argtypes = [f32p, C.c_int32, f32p, u8p, C.c_float]
         L.orc_tbq_decode.argtypes = [f32p, C.c_int32, u8p, C.c_float, C.c_int]
         L.orc_terngrad_encode.argtypes = [f32p, C.c_int32, u8p, C.c_int32, C.c_uint8, C.c_int32, C.c_uint64]
@@ -80,6 +82,10 @@ def u01_from_u32(x):
 
 def u01_shortcut_mismatches(lo, hi):
     return int(lib().orc_u01_shortcut_mismatches(lo, hi))
+
+
+def u01_fp32_mismatches(lo, hi):
+    return int(lib().orc_u01_fp32_mismatches(lo, hi))
 
 
 # ---- TBQ -------------------------------------------------------------------

@@ -85,6 +85,33 @@ ORC_API uint64_t orc_u01_shortcut_mismatches(uint32_t lo, uint32_t hi) {
     return bad;
 }
 
+/* Second proof obligation of the GPU kernel, which avoids fp64 altogether: with
+ *   A  = float(x & 0xFFFFFF00)   (24 significant bits: exact)
+ *   lo = float(x & 0xFF)
+ *   s  = A + fmaf(A, 0x1.ffff88p-33f, lo)
+ * s * 2^-32 equals float(double(x) / 4294967295.0) for every 32-bit x.  The
+ * fused term stands for the x * 2^-32 excess of the exact quotient over
+ * x * 2^-32: it only has to break ties upwards, except for x = 0xFFFFFD7F and
+ * 0xFFFFFF7F, where the fp64 quotient itself rounds onto a tie; the constant is
+ * the one float for which the fused term reaches 128 exactly there and nowhere
+ * it should not.  Returns the number of x in [lo, hi] where the two differ. */
+ORC_API uint64_t orc_u01_fp32_mismatches(uint32_t lo, uint32_t hi) {
+    uint64_t bad = 0;
+    int64_t a = lo, b = hi;
+#pragma omp parallel for reduction(+ : bad) schedule(static)
+    for (int64_t v = a; v <= b; v++) {
+        uint32_t x = (uint32_t)v;
+        float ref = (float)((double)x / 4294967295.0);
+        volatile float A = (float)(x & 0xFFFFFF00u);
+        volatile float l = (float)(x & 0xFFu);
+        volatile float t = fmaf(A, 0x1.ffff88p-33f, l);
+        volatile float s = A + t;
+        float alt = s * 0x1p-32f;
+        if (memcmp(&ref, &alt, 4) != 0) bad++;
+    }
+    return bad;
+}
+
 /* ------------------------------------------------------------------ TBQ -- */
 /* One element of the `compress` functor, tbq_body.h:70-84. */
 static inline uint8_t tbq_step(float g, float *r, float thr, int k, uint8_t q) {

@@ -211,3 +211,95 @@ def test_many_tensors_each_with_several_messages(tg, oracle_cpu):
     torch.cuda.synchronize()
     for t in range(len(sizes)):
         assert_bits_equal(host(outs[t]), refs[t], f"tensor {t}")
+
+
+# ---- the single-launch resident encode (tensor kept on chip between the two passes) ----
+@pytest.fixture
+def resident_forced(capi):
+    old = capi.set_option("terngrad_resident_min", 1)
+    yield
+    capi.set_option("terngrad_resident_min", old)
+
+
+@pytest.mark.parametrize("b", [1, 2, 4, 8])
+@pytest.mark.parametrize("rnd", [0, 1])
+def test_resident_sizes_and_tails(tg, oracle_cpu, resident_forced, b, rnd):
+    rng = np.random.default_rng(900 + 10 * b + rnd)
+    unit = max(4, 8 // b)
+    row = unit * 1024 * 256   # elements that one register row of a 256-CU grid covers
+    sizes = [1, 2, 3, 5, 7, 8, 9, 17, 4097, 300007, row - 1, row, row + unit - 1, row + unit + 1, 2 * row + 13, 3 * row - 5]
+    xs = [rng.normal(0, 1e-2, n).astype(np.float32) for n in sizes]
+    seeds = [int(s) for s in rng.integers(0, 2**63, len(sizes))]
+    _check(tg, oracle_cpu, xs, [b] * len(sizes), [rnd] * len(sizes), seeds, [i & 1 for i in range(len(sizes))], rng)
+
+
+def test_resident_constant_and_zero_tensors(tg, oracle_cpu, resident_forced):
+    rng = np.random.default_rng(3)
+    far = np.full(1_300_000, 0.5, np.float32); far[1_200_001] = -0.0; far[1_250_000] = 0.0   # first zero far from workgroup 0
+    neg = np.full(2_100_001, -0.25, np.float32); neg[5] = 0.0; neg[2_000_000] = -0.0
+    xs = [np.zeros(1000, np.float32), np.full(1003, -0.0, np.float32), np.full(4097, 0.125, np.float32),
+          np.array([0.5, -0.0, 0.0, 0.25, 0.0], np.float32), np.array([-0.5, 0.0, -0.0, -0.25], np.float32),
+          np.array([1e-45, 0, 3e-45, 2e-45] * 50, np.float32), far, neg]
+    for b in (1, 2, 8):
+        for rnd in (0, 1):
+            _check(tg, oracle_cpu, xs, [b] * len(xs), [rnd] * len(xs), [77] * len(xs), [0] * len(xs), rng)
+
+
+def test_resident_seed_edges_and_scalars(tg, oracle_cpu, resident_forced):
+    rng = np.random.default_rng(41)
+    x = rng.normal(0, 1e-2, 70001).astype(np.float32)
+    seeds = [0, 2**32 - 1, 2**32 - 70001 // 4 + 5, 2**64 - 1]
+    _check(tg, oracle_cpu, [x] * len(seeds), [2] * len(seeds), [1] * len(seeds), seeds, [0] * len(seeds), rng)
+    xs, bws = [], []
+    for k in range(60):
+        lo = np.float32(rng.normal() * 10.0 ** rng.uniform(-30, 20))
+        hi = np.float32(lo + abs(np.float32(rng.normal() * 10.0 ** rng.uniform(-38, 20))))
+        v = rng.uniform(lo, hi, int(rng.integers(2, 40))).astype(np.float32)
+        v[0], v[-1] = lo, hi
+        xs.append(v)
+        bws.append(int(rng.choice([1, 2, 4, 8])))
+    _check(tg, oracle_cpu, xs, bws, [1] * len(xs), [int(s) for s in rng.integers(0, 2**63, len(xs))], [0] * len(xs), rng)
+
+
+@pytest.mark.parametrize("b,n", [(2, 33_554_432), (1, 23_068_671), (1, 33_554_431), (4, 33_554_432 + 4096), (8, 29_000_003)])
+def test_resident_capacity_edge(tg, oracle_cpu, b, n):
+    # the largest tensors the chip holds (24 register rows + 8 LDS rows per lane; 14 + 8 at 1 bit with
+    # stochastic rounding), and some just past it
+    rng = np.random.default_rng(n % 1000 + b)
+    x = rng.normal(0, 1e-2, n).astype(np.float32)
+    x[rng.integers(0, n, 1000)] = 0.0
+    dx = dev(x)
+    out = tg.encode([dx], [b], [1], [123456789])[0]
+    rc, ref = oracle_cpu.terngrad_encode(x, b, 1, 123456789)
+    assert rc == 0
+    assert_bits_equal(host(out), ref, f"message n={n} b={b}")
+
+
+def test_resident_and_tiled_tensors_in_one_call(tg, oracle_cpu):
+    rng = np.random.default_rng(77)
+    sizes = [3_000_001, 1000, 2_500_000, 70001, 2_097_152, 2_097_151]
+    xs = [rng.normal(0, 1e-2, n).astype(np.float32) for n in sizes]
+    _check(tg, oracle_cpu, xs, [2, 4, 1, 8, 2, 2], [1, 0, 1, 1, 0, 1], [5, 6, 7, 8, 9, 10], [0] * len(sizes), rng)
+
+
+def test_resident_barrier_expiry_is_reported(tg, oracle_cpu, capi):
+    # A zero bound makes the barrier wait give up at once: every workgroup still leaves normally, the
+    # next encode on that stream reports it, and the stream then uses the two-launch path.
+    rng = np.random.default_rng(5)
+    x = rng.normal(0, 1e-2, 3_000_000).astype(np.float32)
+    side = torch.cuda.Stream()
+    old_ms = capi.set_option("terngrad_barrier_ms", 0)
+    try:
+        with torch.cuda.stream(side):
+            dx = dev(x)
+            tg.encode([dx], [2], [1], [9])
+            side.synchronize()
+            capi.set_option("terngrad_barrier_ms", old_ms)
+            tg.encode([dx], [2], [1], [9], expect_rc=-2)
+            assert "barrier" in capi.last_error()
+            out = tg.encode([dx], [2], [1], [9])[0]
+            side.synchronize()
+            rc, ref = oracle_cpu.terngrad_encode(x, 2, 1, 9)
+            assert_bits_equal(host(out), ref, "message after fallback")
+    finally:
+        capi.set_option("terngrad_barrier_ms", old_ms)

@@ -43,6 +43,14 @@ def test_u01_multiply_shortcut_is_exact_for_all_inputs(oracle_cpu):
     assert oracle_cpu.u01_shortcut_mismatches(0, 0xFFFFFFFF) == 0
 
 
+def test_u01_fp32_form_is_exact_for_all_inputs(oracle_cpu):
+    # The GPU evaluates it without fp64: (A + fma(A, c, lo)) * 2^-32 with A = x & ~0xFF, lo = x & 0xFF.
+    assert oracle_cpu.u01_fp32_mismatches(0, 0xFFFFFFFF) == 0
+    # the two inputs where the fp64 quotient rounds onto a tie of the fp32 grid
+    for x, want in ((0xFFFFFD7F, float.fromhex("0x1.fffffcp-1")), (0xFFFFFF7F, 1.0)):
+        assert float(oracle_cpu.u01_from_u32(x)) == want
+
+
 # ---- TBQ (tbq_body.h) ------------------------------------------------------
 def test_tbq_known_answer(oracle_cpu):
     g = np.array([.003, -.003, .001, -.001, .002, -.002, 0, .0041, .5, -.5], np.float32)

@@ -14,6 +14,8 @@ SYMBOLS = (
     "hpx_version",
     "hpx_last_error",
     "hpx_release_workspaces",
+    "hpx_set_option",
+    "hpx_get_option",
     "hpx_profile_enable",
     "hpx_profile_reset",
     "hpx_profile_query",
@@ -55,6 +57,8 @@ def load():
     L.hpx_release_workspaces.restype = C.c_int
     L.hpx_profile_enable.argtypes = [C.c_int]
     L.hpx_profile_query.argtypes = [C.c_char_p, C.POINTER(C.c_double), C.POINTER(C.c_int64)]
+    L.hpx_set_option.argtypes = [C.c_char_p, C.c_int64]
+    L.hpx_get_option.argtypes = [C.c_char_p, C.POINTER(C.c_int64)]
     L.hpx_tbq_encode.argtypes = [i32, pp, p, pp, pp, p, p]
     L.hpx_tbq_decode.argtypes = [i32, pp, p, pp, p, p, p]
     L.hpx_terngrad_encode.argtypes = [i32, pp, p, pp, p, p, p, p, p]
@@ -102,6 +106,17 @@ def f32_array(vals):
 
 def f64_array(vals):
     return (C.c_double * len(vals))(*[float(v) for v in vals])
+
+
+def set_option(name, value):
+    """Sets a tuning option of the library (see include/hpx.h); returns the previous value."""
+    old = C.c_int64()
+    rc = load().hpx_get_option(name.encode(), C.byref(old))
+    if rc == 0:
+        rc = load().hpx_set_option(name.encode(), int(value))
+    if rc:
+        raise HpxError(rc, last_error())
+    return old.value
 
 
 def profile_query(kernel):

@@ -64,10 +64,18 @@ struct Workspace {
   uint64_t* slots = nullptr;
   size_t slot_words = 0;
   uint32_t epoch = 0;
+  // Exchange memory of the grid-wide barrier (see ensure_barrier): it only ever
+  // holds generation-tagged words; bar_gen is the generation of the last launch.
+  uint32_t* bar = nullptr;
+  uint32_t bar_gen = 0;
+  int num_cus = 0;
+  bool barrier_broken = false;  // a barrier wait expired on this stream: barrier kernels stay off
 };
 constexpr size_t kStateWords = 4096;       // 16 KiB
 constexpr size_t kStatusWord = kStateWords - 16;  // sticky flags live here
 constexpr size_t kPinnedBytes = 1 << 16;
+constexpr size_t kBarWords = 40960;                       // 160 KiB of exchange memory for grid-wide barriers
+constexpr size_t kPinnedFlagOffset = kPinnedBytes - 64;   // host word raised by a kernel whose barrier wait expired
 
 // The record for the calling thread's current device and `stream` (created on
 // first use).  Lock its `mu`, then call ensure_workspace for the scratch size
@@ -76,6 +84,8 @@ Workspace* workspace_record(hipStream_t stream);
 int ensure_workspace(Workspace* ws, size_t dev_bytes);
 // At least `words` zero-initialised-at-allocation 64-bit slots, never used for anything else.
 int ensure_slots(Workspace* ws, size_t words);
+// Zeroed barrier exchange memory and the CU count of the device (both created once).
+int ensure_barrier(Workspace* ws);
 
 uint64_t clock_seed();
 
@@ -128,9 +138,19 @@ __device__ __forceinline__ void st4_stream(float* p, float4 v) {
 // size the write-back happens inside the kernel anyway and the plain store is
 // measurably faster.
 constexpr size_t kStreamStoreMaxBytes = size_t(128) << 20;
-// The limit in force: kStreamStoreMaxBytes unless the environment variable
-// HPX_STREAM_STORE_MAX_MB overrides it (read once; a tuning aid).
+// The limit in force: option "stream_store_max_bytes".
 size_t stream_store_max_bytes();
+
+// Tuning options (hpx_set_option / hpx_get_option).  Each starts from the
+// environment variable HPX_<NAME IN CAPITALS> when that is set, else from its default.
+enum Option {
+  kOptStreamStoreMaxBytes = 0,  // "stream_store_max_bytes", default kStreamStoreMaxBytes
+  kOptTerngradResidentMin,      // "terngrad_resident_min": smallest tensor (elements) that takes the
+                                // single-launch resident encode; negative = never.  Default 2^21.
+  kOptTerngradBarrierMs,        // "terngrad_barrier_ms": bound on the resident kernel's barrier wait.  Default 2000.
+  kOptCount
+};
+int64_t option(Option o);
 
 // Index of the segment owning `tile`: the largest s < nseg with start[s] <= tile,
 // where start[] is the strictly increasing exclusive prefix of tiles per

@@ -19,8 +19,10 @@
 // The stream pass moves 12 bytes per element (g, r in; r out) plus 1/8 byte of
 // mask; everything else touches O(sample + selected) data.  The host waits for
 // the stream once, after the common case (no cut) has been queued in full, to
-// learn whether the cut to `expected` entries is needed; that path orders the
-// candidates by |r| with a stable LSD radix sort (ties keep ascending index).
+// learn whether the cut to `expected` entries is needed.  The expand launch has
+// by then left the candidates, their keys and the first digit's counts where
+// the cut path wants them, so that path is four more launches: a stable LSD radix
+// sort by |r| (ties keep ascending index) whose last pass writes the message.
 #include <cmath>
 
 #include "hpx_common.h"
@@ -292,23 +294,33 @@ __global__ __launch_bounds__(kSelThreads) void gd_scan_kernel(const uint32_t* __
   }
 }
 
-// One wave per stream tile: 64 mask words -> ascending indices at the scanned
-// offsets.  With `out` set this is the common-case finish (gd_body.h:193-229):
-// nothing happens if the stream pass found more than `limit` candidates,
-// otherwise indices, values and header are written and the residual entries are
-// cleared.  With `out` null the indices go to `dst` (the candidate list of the
-// cut path) and nothing else is touched.
+// Shape of the cut path's radix sort (further down): tiles of 8192 pairs.
+constexpr int kSortThreads = 1024;
+constexpr int kSortPer = 8;
+constexpr int kSortTile = kSortThreads * kSortPer;
+constexpr int kSortWaves = kSortThreads / kWave;
+
+// Turns the per-tile bit masks into the ascending index list, one wave per tile,
+// at the offsets the scan produced.  If the stream pass found at most `limit`
+// candidates this is the finish (gd_body.h:193-229): indices, values and header
+// are written and the residual entries cleared.  If it found more, the candidates
+// and their keys (bits of |r|) go to `cand` / `keys` for the cut path instead and
+// nothing else is touched; more than `cap` candidates do not fit those buffers
+// and the kernel does nothing (the host then calls it again with larger ones and
+// limit = 0).
 __global__ __launch_bounds__(kThreads) void gd_expand_kernel(const uint64_t* __restrict__ masks,
                                                              const uint32_t* __restrict__ tile_off,
                                                              const uint32_t* __restrict__ chunk_off, uint32_t ntiles,
-                                                             const GdState* __restrict__ st, int32_t* __restrict__ dst,
-                                                             uint32_t limit, uint8_t* __restrict__ out,
-                                                             float* __restrict__ r) {
+                                                             const GdState* __restrict__ st, uint32_t limit,
+                                                             uint8_t* __restrict__ out, float* __restrict__ r,
+                                                             int32_t* __restrict__ cand, uint32_t* __restrict__ keys,
+                                                             uint32_t cap) {
   const uint32_t total = st->total;
-  if (out && total > limit) return;
+  const bool cut = total > limit;
+  if (cut && total > cap) return;
   const uint32_t lane = threadIdx.x & (kWave - 1);
   const uint32_t tile = blockIdx.x * (kThreads / kWave) + threadIdx.x / kWave;
-  if (out && tile == 0 && lane == 0) *reinterpret_cast<int32_t*>(out) = int32_t(4 + total * 8);
+  if (!cut && tile == 0 && lane == 0) *reinterpret_cast<int32_t*>(out) = int32_t(4 + total * 8);
   if (tile >= ntiles) return;
   uint64_t m = masks[size_t(tile) * kWave + lane];
   const uint32_t c = __popcll(m);
@@ -320,136 +332,199 @@ __global__ __launch_bounds__(kThreads) void gd_expand_kernel(const uint64_t* __r
   }
   uint32_t pos = chunk_off[tile / kScanChunk] + tile_off[tile] + incl - c;
   const uint32_t e0 = tile * uint32_t(kTile) + lane * kWave;
-  int32_t* idx = out ? reinterpret_cast<int32_t*>(out + 4) : dst;
-  float* val = out ? reinterpret_cast<float*>(out + 4 + size_t(total) * 4) : nullptr;
+  if (cut) {
+    while (m) {
+      const uint32_t e = e0 + uint32_t(__builtin_ctzll(m));
+      m &= m - 1;
+      cand[pos] = int32_t(e);
+      keys[pos] = __float_as_uint(__builtin_fabsf(r[e]));
+      pos++;
+    }
+    return;
+  }
+  int32_t* idx = reinterpret_cast<int32_t*>(out + 4);
+  float* val = reinterpret_cast<float*>(out + 4 + size_t(total) * 4);
   while (m) {
     const uint32_t e = e0 + uint32_t(__builtin_ctzll(m));
     m &= m - 1;
-    if (pos < limit) {
-      idx[pos] = int32_t(e);
-      if (out) {
-        val[pos] = r[e];
-        r[e] = 0.0f;
-      }
-    }
+    idx[pos] = int32_t(e);
+    val[pos] = r[e];
+    r[e] = 0.0f;
     pos++;
   }
 }
 
-// generate_S_value, gd_body.h:80-99, plus the header (gd_body.h:193-201), for a
-// list of k indices already in place (the cut path).
-__global__ __launch_bounds__(kThreads) void gd_gather_kernel(uint8_t* __restrict__ out, float* __restrict__ r, uint32_t k) {
-  const int32_t* idx = reinterpret_cast<const int32_t*>(out + 4);
-  float* val = reinterpret_cast<float*>(out + 4 + size_t(k) * 4);
-  const uint32_t x = blockIdx.x * kThreads + threadIdx.x;
-  if (x == 0) *reinterpret_cast<int32_t*>(out) = int32_t(4 + k * 8);
-  if (x < k) {
-    const int32_t i = idx[x];
-    val[x] = r[i];
-    r[i] = 0.0f;
-  }
-}
-
 // ---- cut to the `expected` largest |r| (gd_body.h:176-187) ------------------
-constexpr int kSortPer = 8;
-constexpr int kSortTile = kThreads * kSortPer;  // 2048 pairs per workgroup
+// Stable LSD radix sort of (key, index) pairs, 8 bits per pass, descending
+// (bin = 255 - digit).  A pass is a count launch and a scatter launch over tiles
+// of 8192 pairs (1024 lanes x 8), counts[tile * 256 + bin]; the last pass writes
+// the message instead of a sorted list.  (Counting a pass's digits where its
+// input is written, with global atomics, saves the count launches but was five
+// times slower: some 10^5 scattered atomics cost more than the launches.)
+struct SortArgs {
+  const uint32_t* keys_in;
+  const int32_t* idx_in;
+  uint32_t n;
+  int shift;
+  const uint32_t* counts;   // this pass, complete
+  uint32_t nblk;
+  uint32_t* keys_out;       // not used by the last pass
+  int32_t* idx_out;
+  uint8_t* msg;             // last pass only: the message, of which the first `keep` pairs are written
+  float* r;
+  uint32_t keep;
+};
 
-__global__ __launch_bounds__(kThreads) void gd_keys_kernel(const int32_t* __restrict__ cand, const float* __restrict__ r,
-                                                           uint32_t n, uint32_t* __restrict__ keys) {
-  const uint32_t x = blockIdx.x * kThreads + threadIdx.x;
-  if (x < n) keys[x] = __float_as_uint(__builtin_fabsf(r[cand[x]]));
-}
-
-// Descending order: bin = 255 - byte.  counts is bin-major: counts[bin * nblk + blk].
-__global__ __launch_bounds__(kThreads) void gd_sort_count_kernel(const uint32_t* __restrict__ keys, uint32_t n, int shift,
-                                                                 uint32_t* __restrict__ counts, uint32_t nblk) {
+__global__ __launch_bounds__(kSortThreads) void gd_sort_count_kernel(const uint32_t* __restrict__ keys, uint32_t n,
+                                                                     int shift, uint32_t* __restrict__ counts) {
   __shared__ uint32_t s_hist[256];
-  s_hist[threadIdx.x] = 0;
-  __syncthreads();
+  const uint32_t t = threadIdx.x;
+  if (t < 256) s_hist[t] = 0;
   const uint32_t b0 = blockIdx.x * uint32_t(kSortTile);
+  uint32_t key[kSortPer];
 #pragma unroll
   for (int j = 0; j < kSortPer; j++) {
-    const uint32_t x = b0 + j * kThreads + threadIdx.x;
-    if (x < n) atomicAdd(&s_hist[255u - ((keys[x] >> shift) & 255u)], 1u);
+    const uint32_t x = b0 + j * kSortThreads + t;
+    key[j] = x < n ? keys[x] : 0u;
   }
   __syncthreads();
-  counts[size_t(threadIdx.x) * nblk + blockIdx.x] = s_hist[threadIdx.x];
+#pragma unroll
+  for (int j = 0; j < kSortPer; j++)
+    if (b0 + j * kSortThreads + t < n) atomicAdd(&s_hist[255u - ((key[j] >> shift) & 255u)], 1u);
+  __syncthreads();
+  if (t < 256) counts[size_t(blockIdx.x) * 256 + t] = s_hist[t];
 }
 
-// Stable scatter of one 8-bit digit.  Elements are taken round by round
-// (round j holds x = b0 + j*256 + t), waves in order inside a round, lanes in
-// order inside a wave, so equal digits keep their input order.
-__global__ __launch_bounds__(kThreads) void gd_sort_scatter_kernel(const uint32_t* __restrict__ keys_in,
-                                                                   const int32_t* __restrict__ idx_in, uint32_t n,
-                                                                   int shift, const uint32_t* __restrict__ counts,
-                                                                   uint32_t nblk, uint32_t* __restrict__ keys_out,
-                                                                   int32_t* __restrict__ idx_out) {
-  __shared__ uint32_t s_run[256];   // next output slot per bin for this workgroup
-  __shared__ uint32_t s_scan[256];
+// A wave owns 512 consecutive pairs of the tile and takes them 64 at a time, so
+// the order wave, round, lane is the input order and equal digits keep it.  Per
+// round the lanes of a wave that share a bin are found with ballots; the wave
+// keeps its own running count per bin in its row of s_cnt (no workgroup barrier
+// inside the loop).  One pass over the 16 rows gives every wave its first place
+// per bin within the tile; the pairs are then put in that order in LDS, so that
+// consecutive lanes write consecutive slots of a bin's run (scattering straight
+// from registers costs one address per lane and made the pass twice as long).
+__global__ __launch_bounds__(kSortThreads) void gd_sort_pass_kernel(const SortArgs a) {
+  extern __shared__ uint32_t s_stage[];          // [kSortTile] keys, then [kSortTile] indices
+  __shared__ uint32_t s_cnt[kSortWaves][256];    // per wave: pairs per bin, then the wave's first place per bin
+  __shared__ uint32_t s_first[256];              // first place of the bin within the tile
+  __shared__ uint32_t s_slot[256];               // first global slot of the bin's pairs of this tile
+  __shared__ uint32_t s_part[8];
+  uint32_t* s_key = s_stage;
+  uint32_t* s_id = s_stage + kSortTile;
   const uint32_t t = threadIdx.x;
-  {
-    // bin t: total over all workgroups and the part that precedes this one
-    uint32_t total = 0, before = 0;
-    const uint32_t* row = counts + size_t(t) * nblk;
-    for (uint32_t b = 0; b < nblk; b++) {
-      const uint32_t c = row[b];
-      total += c;
-      if (b < blockIdx.x) before += c;
-    }
-    s_scan[t] = total;
-    __syncthreads();
-    for (int o = 1; o < 256; o <<= 1) {
-      const uint32_t v = t >= uint32_t(o) ? s_scan[t - o] : 0u;
-      __syncthreads();
-      s_scan[t] += v;
-      __syncthreads();
-    }
-    s_run[t] = s_scan[t] - total + before;
-    __syncthreads();
-  }
   const uint32_t lane = t & (kWave - 1), wave = t / kWave;
+  const uint32_t n = a.n;
   const uint32_t b0 = blockIdx.x * uint32_t(kSortTile);
+  const uint32_t x0 = b0 + wave * uint32_t(kSortPer * kWave) + lane;
+  uint32_t key[kSortPer];
+  int32_t id[kSortPer];
+#pragma unroll
   for (int j = 0; j < kSortPer; j++) {
-    const uint32_t x = b0 + j * kThreads + t;
-    const bool live = x < n;
-    uint32_t key = 0, bin = 0;
-    int32_t id = 0;
-    if (live) {
-      key = keys_in[x];
-      id = idx_in[x];
-      bin = 255u - ((key >> shift) & 255u);
+    const uint32_t x = x0 + j * kWave;
+    key[j] = x < n ? a.keys_in[x] : 0u;
+    id[j] = x < n ? a.idx_in[x] : 0;
+  }
+  // bin t (first 256 lanes): pairs in all tiles, in the tiles before this one, in this one.
+  // The first 32 tiles are read with independent loads.
+  uint32_t total = 0, before = 0, mine = 0;
+  if (t < 256) {
+    constexpr uint32_t kFlat = 32;
+    uint32_t c[kFlat];
+#pragma unroll
+    for (uint32_t q = 0; q < kFlat; q++) c[q] = q < a.nblk ? a.counts[size_t(q) * 256 + t] : 0u;
+#pragma unroll
+    for (uint32_t q = 0; q < kFlat; q++) {
+      total += c[q];
+      before += q < blockIdx.x ? c[q] : 0u;
+      mine += q == blockIdx.x ? c[q] : 0u;
     }
-    // lanes of this wave holding the same bin
+    for (uint32_t q = kFlat; q < a.nblk; q++) {
+      const uint32_t v = a.counts[size_t(q) * 256 + t];
+      total += v;
+      before += q < blockIdx.x ? v : 0u;
+      mine += q == blockIdx.x ? v : 0u;
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < 256 / kWave; q++) s_cnt[wave][q * kWave + lane] = 0;  // own row: no barrier needed before use
+
+  uint32_t place[kSortPer], bin[kSortPer];
+#pragma unroll
+  for (int j = 0; j < kSortPer; j++) {
+    const bool live = x0 + j * kWave < n;
+    bin[j] = 255u - ((key[j] >> a.shift) & 255u);
     uint64_t same = __ballot(live);
 #pragma unroll
     for (int b = 0; b < 8; b++) {
-      const uint64_t m = __ballot((bin >> b) & 1u);
-      same &= ((bin >> b) & 1u) ? m : ~m;
+      const uint64_t m = __ballot((bin[j] >> b) & 1u);
+      same &= ((bin[j] >> b) & 1u) ? m : ~m;
     }
     const uint32_t rank = __popcll(same & ((uint64_t(1) << lane) - 1));
-    const uint32_t cnt = __popcll(same);
-    uint32_t slot = 0;
-    for (uint32_t w = 0; w < kThreads / kWave; w++) {
-      if (wave == w && live && rank == 0) {
-        slot = s_run[bin];
-        s_run[bin] = slot + cnt;
-      }
-      __syncthreads();
+    uint32_t base = 0;
+    if (live && rank == 0) {
+      base = s_cnt[wave][bin[j]];
+      s_cnt[wave][bin[j]] = base + uint32_t(__popcll(same));
     }
-    // the first lane of each group read the base; hand it to the others
-    const int leader = live ? __builtin_ctzll(same) : int(lane);
-    slot = __shfl(slot, leader, kWave);
-    if (live) {
-      keys_out[slot + rank] = key;
-      idx_out[slot + rank] = id;
+    base = __shfl(base, live ? __builtin_ctzll(same) : int(lane), kWave);
+    place[j] = base + rank;
+  }
+
+  // Exclusive scans over the 256 bins, of the global totals and of this tile's
+  // counts: within each of the first four waves, then across them.
+  uint32_t incl_g = total, incl_l = mine;
+#pragma unroll
+  for (int o = 1; o < kWave; o <<= 1) {
+    const uint32_t vg = __shfl_up(incl_g, o, kWave), vl = __shfl_up(incl_l, o, kWave);
+    if (lane >= uint32_t(o)) { incl_g += vg; incl_l += vl; }
+  }
+  if (t < 256 && lane == kWave - 1) { s_part[wave] = incl_g; s_part[4 + wave] = incl_l; }
+  __syncthreads();  // also: every wave's row of s_cnt is complete
+  if (t < 256) {
+    uint32_t slot = incl_g - total + before, first = incl_l - mine;
+    for (uint32_t w = 0; w < wave; w++) { slot += s_part[w]; first += s_part[4 + w]; }
+    s_slot[t] = slot;
+    s_first[t] = first;
+    uint32_t run = first;
+#pragma unroll
+    for (int w = 0; w < kSortWaves; w++) {
+      const uint32_t c = s_cnt[w][t];
+      s_cnt[w][t] = run;
+      run += c;
     }
   }
-}
-
-__global__ __launch_bounds__(kThreads) void gd_copy_idx_kernel(const int32_t* __restrict__ src, int32_t* __restrict__ dst,
-                                                               uint32_t n) {
-  const uint32_t x = blockIdx.x * kThreads + threadIdx.x;
-  if (x < n) dst[x] = src[x];
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < kSortPer; j++) {
+    if (x0 + j * kWave < n) {
+      const uint32_t p = s_cnt[wave][bin[j]] + place[j];
+      s_key[p] = key[j];
+      s_id[p] = uint32_t(id[j]);
+    }
+  }
+  __syncthreads();
+  const uint32_t live_n = n - b0 < uint32_t(kSortTile) ? n - b0 : uint32_t(kSortTile);
+  if (a.msg && blockIdx.x == 0 && t == 0) *reinterpret_cast<int32_t*>(a.msg) = int32_t(4 + a.keep * 8);
+#pragma unroll
+  for (int j = 0; j < kSortPer; j++) {
+    const uint32_t p = j * kSortThreads + t;
+    if (p < live_n) {
+      const uint32_t k = s_key[p];
+      const int32_t i = int32_t(s_id[p]);
+      const uint32_t b = 255u - ((k >> a.shift) & 255u);
+      const uint32_t slot = s_slot[b] + (p - s_first[b]);
+      if (a.msg) {
+        // generate_S_value, gd_body.h:80-99, for the pairs that survive the cut
+        if (slot < a.keep) {
+          reinterpret_cast<int32_t*>(a.msg + 4)[slot] = i;
+          reinterpret_cast<float*>(a.msg + 4 + size_t(a.keep) * 4)[slot] = a.r[i];
+          a.r[i] = 0.0f;
+        }
+      } else {
+        a.keys_out[slot] = k;
+        a.idx_out[slot] = i;
+      }
+    }
+  }
 }
 
 // ---- decode -----------------------------------------------------------------
@@ -477,21 +552,36 @@ __global__ __launch_bounds__(kThreads) void gd_scatter_kernel(const int32_t* __r
 inline uint32_t cdiv(uint64_t a, uint64_t b) { return static_cast<uint32_t>((a + b - 1) / b); }
 inline size_t align256(size_t x) { return (x + 255) & ~size_t(255); }
 
-// Sorts (keys, idx) by key descending, stable, `n` pairs; result left in
-// (keys_a, idx_a).  counts holds 256 * nblk words.
-int sort_pairs_desc(uint32_t* keys_a, int32_t* idx_a, uint32_t* keys_b, int32_t* idx_b, uint32_t* counts, uint32_t n,
-                    hipStream_t st) {
+// The four passes of the cut path: (keys_a, idx_a) hold the candidates in index
+// order.  The last pass writes the `keep` largest into the message `msg` and
+// clears their residual entries.
+int sort_and_cut(uint32_t* keys_a, int32_t* idx_a, uint32_t* keys_b, int32_t* idx_b, uint32_t* counts, uint32_t n,
+                 uint8_t* msg, float* r, uint32_t keep, hipStream_t st) {
+  static std::once_flag once;
+  static hipError_t attr_rc = hipSuccess;
+  constexpr int kStageBytes = 2 * kSortTile * int(sizeof(uint32_t));
+  std::call_once(once, [] {
+    attr_rc = hipFuncSetAttribute(reinterpret_cast<const void*>(&gd_sort_pass_kernel),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, kStageBytes);
+  });
+  HPX_HIP(attr_rc);
   const uint32_t nblk = cdiv(n, kSortTile);
   for (int pass = 0; pass < 4; pass++) {
-    const int shift = pass * 8;
-    HPX_LAUNCH("gd_sort_count_kernel", gd_sort_count_kernel, dim3(nblk), dim3(kThreads), st, keys_a, n, shift, counts, nblk);
-    HPX_LAUNCH("gd_sort_scatter_kernel", gd_sort_scatter_kernel, dim3(nblk), dim3(kThreads), st, keys_a, idx_a, n, shift, counts, nblk,
-                       keys_b, idx_b);
+    SortArgs a;
+    a.keys_in = keys_a; a.idx_in = idx_a; a.n = n; a.shift = pass * 8;
+    a.counts = counts; a.nblk = nblk;
+    a.keys_out = keys_b; a.idx_out = idx_b;
+    a.msg = pass == 3 ? msg : nullptr;
+    a.r = r; a.keep = keep;
+    HPX_LAUNCH("gd_sort_count_kernel", gd_sort_count_kernel, dim3(nblk), dim3(kSortThreads), st, keys_a, n, a.shift, counts);
+    if (hpx::g_prof_on) hpx::prof_begin("gd_sort_pass_kernel", st);
+    hipLaunchKernelGGL(gd_sort_pass_kernel, dim3(nblk), dim3(kSortThreads), kStageBytes, st, a);
+    if (hpx::g_prof_on) hpx::prof_end(st);
     HPX_HIP(hipGetLastError());
     std::swap(keys_a, keys_b);
     std::swap(idx_a, idx_b);
   }
-  return HPX_OK;  // four passes: data is back in the caller's (keys_a, idx_a)
+  return HPX_OK;
 }
 
 int gd_encode_one(const float* g, int32_t N, float* r, uint8_t* out, double sample_rate, double drop_ratio,
@@ -517,14 +607,25 @@ int gd_encode_one(const float* g, int32_t N, float* r, uint8_t* out, double samp
   const size_t o_off = off; off += align256(sizeof(uint32_t) * size_t(ntiles));
   const size_t o_ctot = off; off += align256(sizeof(uint32_t) * kMaxChunks);
   const size_t o_coff = off; off += align256(sizeof(uint32_t) * kMaxChunks);
-  // Room for the cut path (sorted copies of the candidates) is reserved for a
-  // typical overshoot so that path normally needs no reallocation.
-  uint64_t cap = uint64_t(expected) * 2 > uint64_t(expected) + 65536 ? uint64_t(expected) * 2 : uint64_t(expected) + 65536;
-  if (cap > n) cap = n;
-  auto cut_bytes = [](uint64_t total) {
-    return 4 * align256(sizeof(uint32_t) * size_t(total)) + align256(sizeof(uint32_t) * 256 * size_t(cdiv(total, kSortTile)));
+  // Room for the cut path (two copies of the candidates' keys and indices, and
+  // the sort's counts) is laid out for a typical overshoot before anything is
+  // launched: the expand kernel fills it without the host knowing the count.
+  uint64_t cap64 = uint64_t(expected) * 2 > uint64_t(expected) + 65536 ? uint64_t(expected) * 2 : uint64_t(expected) + 65536;
+  if (cap64 > n) cap64 = n;
+  const uint32_t cap = static_cast<uint32_t>(cap64);
+  struct CutLayout { size_t ka, kb, ia, ib, sc, end; };
+  auto cut_layout = [](size_t at, uint64_t pairs) {
+    CutLayout c;
+    c.ka = at; at += align256(sizeof(uint32_t) * size_t(pairs));
+    c.kb = at; at += align256(sizeof(uint32_t) * size_t(pairs));
+    c.ia = at; at += align256(sizeof(int32_t) * size_t(pairs));
+    c.ib = at; at += align256(sizeof(int32_t) * size_t(pairs));
+    c.sc = at; at += align256(sizeof(uint32_t) * 256 * size_t(cdiv(pairs, kSortTile)));
+    c.end = at;
+    return c;
   };
-  int rc = hpx::ensure_workspace(ws, off + cut_bytes(cap));
+  CutLayout cl = cut_layout(off, cap);
+  int rc = hpx::ensure_workspace(ws, cl.end);
   if (rc != HPX_OK) return rc;
   uint8_t* base = ws->dev;
   GdState* state = reinterpret_cast<GdState*>(base + o_state);
@@ -553,32 +654,27 @@ int gd_encode_one(const float* g, int32_t N, float* r, uint8_t* out, double samp
   HPX_LAUNCH("gd_scan_kernel", gd_scan_kernel, dim3(nchunks), dim3(kSelThreads), st, blk_cnt, blk_off, ntiles, chunk_tot,
              chunk_off, state, h_total);
   HPX_HIP(hipGetLastError());
-  // Common case (nothing to cut) queued before the host knows the count.
-  int32_t* out_idx = reinterpret_cast<int32_t*>(out + 4);
+  // Queued before the host knows the count: the finish if nothing has to be cut,
+  // else the candidate list and keys of the cut path.
   const uint32_t lim = static_cast<uint32_t>(expected);
   HPX_LAUNCH("gd_expand_kernel", gd_expand_kernel, dim3(cdiv(ntiles, kThreads / kWave)), dim3(kThreads), st, masks, blk_off,
-             chunk_off, ntiles, state, out_idx, lim, out, r);
+             chunk_off, ntiles, state, lim, out, r, reinterpret_cast<int32_t*>(base + cl.ia),
+             reinterpret_cast<uint32_t*>(base + cl.ka), cap);
   HPX_HIP(hipGetLastError());
   HPX_HIP(hipStreamSynchronize(st));
   const uint32_t total = *reinterpret_cast<volatile uint32_t*>(h_total);
   if (total <= lim) return HPX_OK;
 
   // More candidates than `expected`: order them by |r| descending and keep the first `expected`.
-  const uint32_t sblk = cdiv(total, kSortTile);
-  size_t off2 = off;
-  const size_t o_ka = off2; off2 += align256(sizeof(uint32_t) * size_t(total));
-  const size_t o_kb = off2; off2 += align256(sizeof(uint32_t) * size_t(total));
-  const size_t o_ia = off2; off2 += align256(sizeof(int32_t) * size_t(total));
-  const size_t o_ib = off2; off2 += align256(sizeof(int32_t) * size_t(total));
-  const size_t o_sc = off2; off2 += align256(sizeof(uint32_t) * 256 * size_t(sblk));
-  if (off2 > ws->dev_bytes) {
+  if (total > cap) {
     // Far more candidates than reserved for.  Growing would discard the masks;
-    // build the larger block and carry them over.
+    // build the larger block, carry them over and list the candidates again.
+    cl = cut_layout(off, total);
     uint8_t* old = ws->dev;
     const size_t old_bytes = ws->dev_bytes;
     ws->dev = nullptr;
     ws->dev_bytes = 0;
-    rc = hpx::ensure_workspace(ws, off2);
+    rc = hpx::ensure_workspace(ws, cl.end);
     if (rc != HPX_OK) { (void)hipFree(old); return rc; }
     HPX_HIP(hipMemcpyAsync(ws->dev, old, off < old_bytes ? off : old_bytes, hipMemcpyDeviceToDevice, st));
     HPX_HIP(hipStreamSynchronize(st));
@@ -588,21 +684,18 @@ int gd_encode_one(const float* g, int32_t N, float* r, uint8_t* out, double samp
     masks = reinterpret_cast<uint64_t*>(base + o_masks);
     blk_off = reinterpret_cast<uint32_t*>(base + o_off);
     chunk_off = reinterpret_cast<uint32_t*>(base + o_coff);
+    HPX_LAUNCH("gd_expand_kernel", gd_expand_kernel, dim3(cdiv(ntiles, kThreads / kWave)), dim3(kThreads), st, masks, blk_off,
+               chunk_off, ntiles, state, 0u, out, r, reinterpret_cast<int32_t*>(base + cl.ia),
+               reinterpret_cast<uint32_t*>(base + cl.ka), total);
+    HPX_HIP(hipGetLastError());
   }
-  uint32_t* ka = reinterpret_cast<uint32_t*>(base + o_ka);
-  uint32_t* kb = reinterpret_cast<uint32_t*>(base + o_kb);
-  int32_t* ia = reinterpret_cast<int32_t*>(base + o_ia);
-  int32_t* ib = reinterpret_cast<int32_t*>(base + o_ib);
-  uint32_t* sc = reinterpret_cast<uint32_t*>(base + o_sc);
-  HPX_LAUNCH("gd_expand_kernel", gd_expand_kernel, dim3(cdiv(ntiles, kThreads / kWave)), dim3(kThreads), st, masks, blk_off,
-             chunk_off, ntiles, state, ia, total, static_cast<uint8_t*>(nullptr), static_cast<float*>(nullptr));
-  HPX_LAUNCH("gd_keys_kernel", gd_keys_kernel, dim3(cdiv(total, kThreads)), dim3(kThreads), st, ia, r, total, ka);
-  HPX_HIP(hipGetLastError());
-  rc = sort_pairs_desc(ka, ia, kb, ib, sc, total, st);
+  uint32_t* ka = reinterpret_cast<uint32_t*>(base + cl.ka);
+  uint32_t* kb = reinterpret_cast<uint32_t*>(base + cl.kb);
+  int32_t* ia = reinterpret_cast<int32_t*>(base + cl.ia);
+  int32_t* ib = reinterpret_cast<int32_t*>(base + cl.ib);
+  uint32_t* sc = reinterpret_cast<uint32_t*>(base + cl.sc);
+  rc = sort_and_cut(ka, ia, kb, ib, sc, total, out, r, lim, st);
   if (rc != HPX_OK) return rc;
-  if (lim > 0) HPX_LAUNCH("gd_copy_idx_kernel", gd_copy_idx_kernel, dim3(cdiv(lim, kThreads)), dim3(kThreads), st, ia, out_idx, lim);
-  HPX_LAUNCH("gd_gather_kernel", gd_gather_kernel, dim3(cdiv(lim > 0 ? lim : 1, kThreads)), dim3(kThreads), st, out, r, lim);
-  HPX_HIP(hipGetLastError());
   return HPX_OK;
 }
 

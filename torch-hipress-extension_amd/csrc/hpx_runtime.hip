@@ -5,6 +5,7 @@
 #include <map>
 #include <memory>
 #include <algorithm>
+#include <atomic>
 #include <cstdlib>
 #include <cstring>
 #include <utility>
@@ -48,6 +49,7 @@ int ensure_workspace(Workspace* ws, size_t dev_bytes) {
     HPX_HIP(hipMalloc(reinterpret_cast<void**>(&ws->state), kStateWords * sizeof(uint32_t)));
     HPX_HIP(hipMemset(ws->state, 0, kStateWords * sizeof(uint32_t)));
     HPX_HIP(hipHostMalloc(reinterpret_cast<void**>(&ws->pinned), kPinnedBytes, hipHostMallocDefault));
+    std::memset(ws->pinned, 0, kPinnedBytes);
   }
   if (dev_bytes > ws->dev_bytes) {
     // Work already queued on this stream may still use the old block.
@@ -109,12 +111,51 @@ int ensure_slots(Workspace* ws, size_t words) {
   return HPX_OK;
 }
 
+int ensure_barrier(Workspace* ws) {
+  if (ws->bar) return HPX_OK;
+  HPX_HIP(hipDeviceGetAttribute(&ws->num_cus, hipDeviceAttributeMultiprocessorCount, ws->device));
+  HPX_HIP(hipMalloc(reinterpret_cast<void**>(&ws->bar), kBarWords * sizeof(uint32_t)));
+  HPX_HIP(hipMemset(ws->bar, 0, kBarWords * sizeof(uint32_t)));
+  ws->bar_gen = 0;
+  return HPX_OK;
+}
+
+namespace {
+struct OptionDef {
+  const char* name;
+  const char* env;
+  int64_t def;
+};
+const OptionDef kOptions[kOptCount] = {
+    {"stream_store_max_bytes", "HPX_STREAM_STORE_MAX_BYTES", int64_t(kStreamStoreMaxBytes)},
+    {"terngrad_resident_min", "HPX_TERNGRAD_RESIDENT_MIN", int64_t(1) << 21},
+    {"terngrad_barrier_ms", "HPX_TERNGRAD_BARRIER_MS", 2000},
+};
+std::atomic<int64_t> g_opt[kOptCount];
+std::once_flag g_opt_once;
+void options_init() {
+  std::call_once(g_opt_once, [] {
+    for (int i = 0; i < kOptCount; i++) {
+      const char* e = std::getenv(kOptions[i].env);
+      g_opt[i].store(e ? std::strtoll(e, nullptr, 10) : kOptions[i].def);
+    }
+  });
+}
+int option_index(const char* name) {
+  for (int i = 0; i < kOptCount; i++)
+    if (std::strcmp(name, kOptions[i].name) == 0) return i;
+  return -1;
+}
+}  // namespace
+
+int64_t option(Option o) {
+  options_init();
+  return g_opt[o].load(std::memory_order_relaxed);
+}
+
 size_t stream_store_max_bytes() {
-  static const size_t v = [] {
-    const char* e = std::getenv("HPX_STREAM_STORE_MAX_MB");
-    return e ? size_t(std::strtoull(e, nullptr, 10)) << 20 : kStreamStoreMaxBytes;
-  }();
-  return v;
+  const int64_t v = option(kOptStreamStoreMaxBytes);
+  return v < 0 ? 0 : size_t(v);
 }
 
 int classify_outputs(int count, float* const* outs, const int32_t* sizes) {
@@ -160,11 +201,32 @@ HPX_API int hpx_release_workspaces(void) {
     if (ws->dev && hipFree(ws->dev) != hipSuccess) rc = HPX_ERR_HIP;
     if (ws->state && hipFree(ws->state) != hipSuccess) rc = HPX_ERR_HIP;
     if (ws->slots && hipFree(ws->slots) != hipSuccess) rc = HPX_ERR_HIP;
+    if (ws->bar && hipFree(ws->bar) != hipSuccess) rc = HPX_ERR_HIP;
     if (ws->pinned && hipHostFree(ws->pinned) != hipSuccess) rc = HPX_ERR_HIP;
   }
   hpx::g_ws.clear();
   if (cur >= 0) (void)hipSetDevice(cur);
   return rc;
+}
+
+HPX_API int hpx_set_option(const char* name, int64_t value) {
+  hpx::clear_error();
+  HPX_ARG(name, "hpx_set_option: null name");
+  hpx::options_init();
+  const int i = hpx::option_index(name);
+  HPX_ARG(i >= 0, "hpx_set_option: unknown option '%s'", name);
+  hpx::g_opt[i].store(value);
+  return HPX_OK;
+}
+
+HPX_API int hpx_get_option(const char* name, int64_t* value) {
+  hpx::clear_error();
+  HPX_ARG(name && value, "hpx_get_option: null argument");
+  hpx::options_init();
+  const int i = hpx::option_index(name);
+  HPX_ARG(i >= 0, "hpx_get_option: unknown option '%s'", name);
+  *value = hpx::g_opt[i].load();
+  return HPX_OK;
 }
 
 HPX_API int hpx_profile_enable(int on) {

@@ -15,12 +15,20 @@
 //     draws once per slot after one discarded draw (terngrad_body.h:88-96), so
 //     slot j of byte i uses x = A_{j+2} * (seed + i) + C_{j+2}: a lane stepping
 //     through bytes at a fixed stride advances each draw by a constant.
-//   * u = float(double(x) / 4294967295.0) is evaluated as
-//     float(double(x) * 0x1.00000001p-32); the two agree for all 2^32 inputs
-//     (checked exhaustively on the CPU), and the product needs no division.
+//   * u = float(double(x) / 4294967295.0) is evaluated without fp64 (which
+//     runs at a quarter of the fp32 rate and made the quantise pass
+//     ALU-bound): with A = float(x & ~0xFF) and lo = float(x & 0xFF),
+//     u = (A + fma(A, 0x1.ffff88p-33, lo)) * 2^-32 for all 2^32 inputs
+//     (checked exhaustively on the CPU).  A + lo alone is RNE(x); the fused
+//     term adds the quotient's excess over x * 2^-32, which turns ties into
+//     round-up, and the constant is chosen so that the two inputs where the
+//     fp64 quotient itself lands on a tie (0xFFFFFD7F, 0xFFFFFF7F) come out
+//     as the reference's double rounding leaves them.
 //   * min and max are the FIRST smallest / largest element as
 //     thrust::minmax_element returns them, which only matters for the sign of
 //     a zero extreme; it is recovered from the first zero of the tensor.
+#include <cstdlib>
+#include <mutex>
 #include <unordered_map>
 #include <vector>
 
@@ -177,6 +185,27 @@ __global__ __launch_bounds__(kThreads) void terngrad_minmax_kernel(const EncArgs
   }
 }
 
+// 1 / (gap + 1e-8) in fp64, rounded to fp32 (terngrad_body.h:204-206).
+__device__ __forceinline__ float inverse_gap(float mn, float mx, uint32_t bits) {
+  const float gap = (mx - mn) / (float(1 << bits) - 1.0f);
+  return static_cast<float>(1.0 / (static_cast<double>(gap) + 1e-8));
+}
+
+// The 10-byte header: bitwidth, tail, min, max (terngrad_body.h:219-224).
+__device__ __forceinline__ void write_header(uint8_t* o, uint32_t bits, uint32_t n, float mn, float mx) {
+  const uint32_t dpb = 8u / bits;
+  uint32_t tail = n % dpb;
+  tail = tail == 0 ? 0 : dpb - tail;
+  const uint32_t mb = __float_as_uint(mn), xb = __float_as_uint(mx);
+  o[0] = uint8_t(bits);
+  o[1] = uint8_t(tail);
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    o[2 + i] = uint8_t(mb >> (8 * i));
+    o[6 + i] = uint8_t(xb >> (8 * i));
+  }
+}
+
 // Prologue of the quantise kernel: folds the tensor's 64 slots into min and max
 // (thrust::minmax_element semantics: a zero extreme takes the sign of the first
 // zero element of the tensor), derives gap and 1/(gap + 1e-8) as the reference
@@ -217,28 +246,16 @@ __device__ __forceinline__ void load_scalars(const EncArgs<CAP>& a, int s, bool 
     }
   }
   const uint32_t bits = a.seg[s].bits;
-  const float gap = (mx - mn) / (float(1 << bits) - 1.0f);
-  gi_out = static_cast<float>(1.0 / (static_cast<double>(gap) + 1e-8));
+  gi_out = inverse_gap(mn, mx, bits);
   mn_out = mn;
-  if (first_tile && threadIdx.x == 0) {
-    const uint32_t dpb = 8u / bits;
-    uint32_t tail = n % dpb;
-    tail = tail == 0 ? 0 : dpb - tail;
-    uint8_t* o = a.seg[s].out;
-    const uint32_t mb = __float_as_uint(mn), xb = __float_as_uint(mx);
-    o[0] = uint8_t(bits);
-    o[1] = uint8_t(tail);
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      o[2 + i] = uint8_t(mb >> (8 * i));
-      o[6 + i] = uint8_t(xb >> (8 * i));
-    }
-  }
+  if (first_tile && threadIdx.x == 0) write_header(a.seg[s].out, bits, n, mn, mx);
 }
 
-// float(double(x) / 4294967295.0) without the division (see the file header).
-__device__ __forceinline__ float u01(uint32_t x) {
-  return static_cast<float>(static_cast<double>(x) * 0x1.00000001p-32);
+// 2^32 * float(double(x) / 4294967295.0), in fp32 only (see the file header).
+__device__ __forceinline__ float u01_scaled(uint32_t x) {
+  const float hi = static_cast<float>(x & 0xFFFFFF00u);  // 24 significant bits: exact
+  const float lo = static_cast<float>(x & 0xFFu);
+  return hi + __builtin_fmaf(hi, 0x1.ffff88p-33f, lo);
 }
 
 template <int B, bool RANDOM>
@@ -246,12 +263,63 @@ __device__ __forceinline__ uint32_t quant_one(float x, float mn, float gi, uint3
   float th = (x - mn) * gi;
   int32_t t;
   if (RANDOM) {
-    th += u01(draw);
+    th = __builtin_fmaf(u01_scaled(draw), 0x1p-32f, th);  // th + u: the scaling by 2^-32 is exact
     t = static_cast<int32_t>(th);  // truncation, terngrad_body.h:94
   } else {
     t = static_cast<int32_t>(__builtin_rintf(th));  // nearbyint, terngrad_body.h:53
   }
   return static_cast<uint32_t>(t) & 0xFFu;
+}
+
+// Quantises one unit held in registers and returns its BPU packed bytes; advances
+// the lane's draws by `stride_bytes` output bytes.
+template <int B, bool RANDOM, int UNIT = (8 / B > 4 ? 8 / B : 4)>
+__device__ __forceinline__ uint32_t quant_unit(const float4 (&v)[UNIT / 4], float mn, float gi, uint32_t (&draw)[UNIT],
+                                               uint32_t stride_bytes) {
+  constexpr int DPB = 8 / B;
+  uint32_t packed = 0;
+#pragma unroll
+  for (int q = 0; q < UNIT; q++) {
+    const float4 f = v[q / 4];
+    const float x = (q & 3) == 0 ? f.x : (q & 3) == 1 ? f.y : (q & 3) == 2 ? f.z : f.w;
+    const uint32_t t = quant_one<B, RANDOM>(x, mn, gi, RANDOM ? draw[q] : 0u);
+    // Within a byte codes are OR-ed without masking (terngrad_body.h:95):
+    // a code that reaches 1<<B spills into the next slot of the SAME byte.
+    const int jb = q / DPB, j = q % DPB;
+    packed |= ((t << (B * j)) & 0xFFu) << (8 * jb);
+    if (RANDOM) draw[q] += lcg_mul(j + 2) * stride_bytes;
+  }
+  return packed;
+}
+
+// Unit u of a tensor whose end may fall inside it: element-wise from memory.
+template <int B, bool RANDOM, int UNIT = (8 / B > 4 ? 8 / B : 4)>
+__device__ __forceinline__ void quant_unit_ragged(const EncSeg& sg, float mn, float gi, uint32_t u,
+                                                  const uint32_t (&draw)[UNIT]) {
+  constexpr int DPB = 8 / B;
+  constexpr int BPU = UNIT / DPB;
+  const float* __restrict__ xp = sg.x;
+  uint8_t* __restrict__ pay = sg.out + 10;
+  const uint32_t n = static_cast<uint32_t>(sg.n);
+  const uint32_t nbytes = n / DPB;  // bytes the reference's transform covers
+  for (int jb = 0; jb < BPU; jb++) {
+    const uint32_t byte = u * BPU + jb;
+    const size_t e = size_t(byte) * DPB;
+    if (byte < nbytes) {
+      uint32_t qv = 0;
+      for (int j = 0; j < DPB; j++) {
+        const uint32_t t = quant_one<B, RANDOM>(xp[e + j], mn, gi, RANDOM ? draw[jb * DPB + j] : 0u);
+        qv |= t << (B * j);
+      }
+      pay[byte] = uint8_t(qv);
+    } else if (byte == nbytes && (n % DPB)) {
+      // Partial last byte: always round-to-nearest, stored at the last byte
+      // of the caller's buffer (terngrad_body.h:288-296).
+      uint32_t qv = 0;
+      for (uint32_t j = 0; j < n % DPB; j++) qv |= quant_one<B, false>(xp[e + j], mn, gi, 0u) << (B * j);
+      sg.out[sg.out_size - 1] = uint8_t(qv);
+    }
+  }
 }
 
 // One tile of the quantise stream.  A unit is UNIT = max(4, 8/B) consecutive
@@ -265,7 +333,6 @@ __device__ __forceinline__ void quant_tile(const EncSeg& sg, const float mn, con
   const float* __restrict__ xp = sg.x;
   uint8_t* __restrict__ pay = sg.out + 10;
   const uint32_t n = static_cast<uint32_t>(sg.n);
-  const uint32_t nbytes = n / DPB;  // bytes the reference's transform covers
   const uint32_t u0 = tile_in_seg * uint32_t(kThreads * kQIters) + threadIdx.x;
 
   // Draw for slot j of byte (u*BPU + jb): A_{j+2} * (seed + byte) + C_{j+2}.
@@ -290,47 +357,16 @@ __device__ __forceinline__ void quant_tile(const EncSeg& sg, const float mn, con
         v[k][h] = ld4_stream(xp + size_t(u0 + k * kThreads) * UNIT + h * 4);
 #pragma unroll
     for (int k = 0; k < kQIters; k++) {
-      const uint32_t u = u0 + k * kThreads;
-      uint32_t packed = 0;
+      const uint32_t packed = quant_unit<B, RANDOM>(v[k], mn, gi, draw, kStrideBytes);
 #pragma unroll
-      for (int q = 0; q < UNIT; q++) {
-        const float4 f = v[k][q / 4];
-        const float x = (q & 3) == 0 ? f.x : (q & 3) == 1 ? f.y : (q & 3) == 2 ? f.z : f.w;
-        const uint32_t t = quant_one<B, RANDOM>(x, mn, gi, RANDOM ? draw[q] : 0u);
-        // Within a byte codes are OR-ed without masking (terngrad_body.h:95):
-        // a code that reaches 1<<B spills into the next slot of the SAME byte.
-        const int jb = q / DPB, j = q % DPB;
-        packed |= ((t << (B * j)) & 0xFFu) << (8 * jb);
-        if (RANDOM) draw[q] += lcg_mul(j + 2) * kStrideBytes;
-      }
-#pragma unroll
-      for (int jb = 0; jb < BPU; jb++) pay[size_t(u) * BPU + jb] = uint8_t(packed >> (8 * jb));
+      for (int jb = 0; jb < BPU; jb++) pay[size_t(u0 + k * kThreads) * BPU + jb] = uint8_t(packed >> (8 * jb));
     }
     return;
   }
   // Tile holding the end of the tensor.
   for (int k = 0; k < kQIters; k++) {
     const uint32_t u = u0 + k * kThreads;
-    if (u < units_total) {
-      for (int jb = 0; jb < BPU; jb++) {
-        const uint32_t byte = u * BPU + jb;
-        const size_t e = size_t(byte) * DPB;
-        if (byte < nbytes) {
-          uint32_t qv = 0;
-          for (int j = 0; j < DPB; j++) {
-            const uint32_t t = quant_one<B, RANDOM>(xp[e + j], mn, gi, RANDOM ? draw[jb * DPB + j] : 0u);
-            qv |= t << (B * j);
-          }
-          pay[byte] = uint8_t(qv);
-        } else if (byte == nbytes && (n % DPB)) {
-          // Partial last byte: always round-to-nearest, stored at the last byte
-          // of the caller's buffer (terngrad_body.h:288-296).
-          uint32_t qv = 0;
-          for (uint32_t j = 0; j < n % DPB; j++) qv |= quant_one<B, false>(xp[e + j], mn, gi, 0u) << (B * j);
-          sg.out[sg.out_size - 1] = uint8_t(qv);
-        }
-      }
-    }
+    if (u < units_total) quant_unit_ragged<B, RANDOM>(sg, mn, gi, u, draw);
     if (RANDOM) {
 #pragma unroll
       for (int q = 0; q < UNIT; q++) draw[q] += lcg_mul(q % DPB + 2) * kStrideBytes;
@@ -356,6 +392,314 @@ __global__ __launch_bounds__(kThreads) void terngrad_quant_kernel(const EncArgs<
     case 2: quant_dispatch<2>(a.seg[s], mn, gi, t); break;
     case 4: quant_dispatch<4>(a.seg[s], mn, gi, t); break;
     default: quant_dispatch<8>(a.seg[s], mn, gi, t); break;
+  }
+}
+
+// ---- resident encode ------------------------------------------------------------
+// One launch for one large tensor.  The chip's register files and LDS together
+// hold more than 128 MB, so a tensor of up to ~33M elements can stay on chip
+// between the min/max pass and the quantise pass: every workgroup (one per CU,
+// 1024 lanes) loads its contiguous share once, 24 float4 per lane into registers
+// and the rest into LDS, publishes its extremes, waits at a grid-wide barrier and
+// then quantises out of registers.  The tensor is read from HBM once instead of
+// twice.
+//
+// The barrier is a two-level arrival count on monotonic counters (they are never
+// reset; launch number `gen` waits for gen * arrivals).  All workgroups of the grid
+// must be resident together, which holds because the grid is one workgroup per
+// CU and a workgroup fits a CU by construction; other work sharing the GPU only
+// delays the barrier.  The wait is bounded by `spin_limit` ticks of the 100 MHz
+// wall clock: on expiry the workgroup raises *host_flag and leaves, so the grid
+// always drains.
+constexpr int kResThreads = 1024;
+constexpr int kResRegGroups = 24;  // float4 per lane held in registers ...
+// ... except at 1 bit with stochastic rounding, whose eight draws per lane need the room.
+constexpr int res_reg_groups(int bits, bool random) { return (bits == 1 && random) ? 14 : kResRegGroups; }
+constexpr int kResLdsGroups = 8;   // float4 per lane held in LDS (128 KiB per workgroup)
+constexpr int kBarGroup = 16;           // workgroups per group; also the largest number of groups
+constexpr int kBarMaxWorkgroups = kBarGroup * kBarGroup;
+constexpr int kBarRecWords = 4;         // 64-bit words per record (three used)
+constexpr int kBarAreaWords = kBarGroup * kBarRecWords;  // one area: 16 records = 64 words = 512 bytes
+// Exchange memory, in 64-bit words: group areas first (members report here), then
+// one area per workgroup (group leaders report here).
+constexpr size_t kBarGroupBase = 0;
+constexpr size_t kBarWgBase = size_t(kBarGroup) * kBarAreaWords;
+constexpr size_t kBarTotalWords = kBarWgBase + size_t(kBarMaxWorkgroups) * kBarAreaWords;
+static_assert(kBarTotalWords * 8 <= hpx::kBarWords * 4, "barrier memory too small");
+
+struct ResArgs {
+  EncSeg seg;
+  uint32_t chunk_units;  // units per workgroup, a multiple of kResThreads
+  uint32_t lds_rows;     // rows of kResThreads units kept in LDS
+  uint32_t gen;          // generation of this launch, counted from 1: the tag of its records
+  uint64_t* bar;         // exchange memory (kBarTotalWords); only ever holds (gen << 32 | key) words
+  uint32_t* host_flag;   // pinned host word, set to 1 when the barrier wait expires
+  uint64_t spin_limit;
+};
+
+// Grid-wide exchange of (max key, min key, first-zero key) and barrier in one.
+// Every lane of wave 0 of every workgroup calls it once per launch with the
+// workgroup's three keys; on success every lane holds the grid-wide maximum of
+// key[lane & 3] (lanes with (lane & 3) == 3 hold nothing of use).
+//
+// The protocol uses only stores and polling loads, no read-modify-write and no
+// fence: a member writes its record (three self-validating words, generation in
+// the high half) into its group's area; the group's leader polls that area with
+// one wave-wide load until all records carry this generation, folds them, and
+// writes the group's record into the area of EVERY workgroup; each workgroup
+// polls its own area until all groups have reported.  A polled line has one
+// reader, a written line at most 16 writers, and the critical path is two
+// store-to-load hand-overs.  (A counter-based barrier - fence, two dependent
+// atomics, a release flag, then reading the reduction slots - took 7 us here;
+// polling one shared word from all 256 workgroups took 10.)
+__device__ __forceinline__ bool grid_exchange(uint64_t* bar, uint32_t gen, uint64_t spin_limit, uint32_t& key) {
+  const uint32_t lane = threadIdx.x;  // < 64
+  const uint32_t nwg = gridDim.x, grp = blockIdx.x / kBarGroup, mem = blockIdx.x % kBarGroup;
+  const uint32_t ngrp = (nwg + kBarGroup - 1) / kBarGroup;
+  const uint32_t left = nwg - grp * kBarGroup;
+  const uint32_t gsz = left < uint32_t(kBarGroup) ? left : uint32_t(kBarGroup);
+  const uint64_t tag = uint64_t(gen) << 32;
+  const uint64_t t0 = wall_clock64();
+  unsigned long long* garea = reinterpret_cast<unsigned long long*>(bar) + kBarGroupBase + size_t(grp) * kBarAreaWords;
+  unsigned long long* warea = reinterpret_cast<unsigned long long*>(bar) + kBarWgBase + size_t(blockIdx.x) * kBarAreaWords;
+  const uint32_t rec = lane / kBarRecWords, word = lane % kBarRecWords;
+
+  if (lane < 3) __hip_atomic_store(&garea[mem * kBarRecWords + lane], tag | key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+
+  bool ok = true;
+  if (mem == 0) {  // group leader
+    uint32_t k = 0;
+    for (;;) {
+      const unsigned long long v = __hip_atomic_load(&garea[lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const bool valid = word == 3 || rec >= gsz || uint32_t(v >> 32) == gen;
+      k = (word == 3 || rec >= gsz) ? 0u : uint32_t(v);
+      if (__ballot(valid) == ~0ull) break;
+      if (wall_clock64() - t0 > spin_limit) { ok = false; break; }
+      __builtin_amdgcn_s_sleep(1);
+    }
+    if (ok) {
+#pragma unroll
+      for (int o = kBarRecWords; o < kWave; o <<= 1) { const uint32_t t = __shfl_xor(k, o, 64); k = t > k ? t : k; }
+      // lane l now holds the group's key (l & 3); lanes 0..2 of each quad of lanes write it out
+      unsigned long long* wbase = reinterpret_cast<unsigned long long*>(bar) + kBarWgBase + size_t(grp) * kBarRecWords;
+      if (word < 3) {
+        for (uint32_t w = rec; w < nwg; w += kWave / kBarRecWords)
+          __hip_atomic_store(&wbase[size_t(w) * kBarAreaWords + word], tag | k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+  }
+  ok = __builtin_amdgcn_readfirstlane(ok ? 1 : 0) != 0;
+  if (!ok) return false;
+
+  uint32_t k = 0;
+  for (;;) {
+    const unsigned long long v = __hip_atomic_load(&warea[lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const bool valid = word == 3 || rec >= ngrp || uint32_t(v >> 32) == gen;
+    k = (word == 3 || rec >= ngrp) ? 0u : uint32_t(v);
+    if (__ballot(valid) == ~0ull) break;
+    if (wall_clock64() - t0 > spin_limit) return false;
+    __builtin_amdgcn_s_sleep(1);
+  }
+#pragma unroll
+  for (int o = kBarRecWords; o < kWave; o <<= 1) { const uint32_t t = __shfl_xor(k, o, 64); k = t > k ? t : k; }
+  key = k;
+  return true;
+}
+
+__device__ __forceinline__ void acc_zero(float v, uint32_t idx, float& mn, float& mx, uint32_t& fz) {
+  mn = v < mn ? v : mn;
+  mx = v > mx ? v : mx;
+  fz = (v == 0.0f && idx < fz) ? idx : fz;
+}
+__device__ __forceinline__ void acc_zero4(float4 v, uint32_t idx, float& mn, float& mx, uint32_t& fz) {
+  acc_zero(v.x, idx, mn, mx, fz); acc_zero(v.y, idx + 1, mn, mx, fz);
+  acc_zero(v.z, idx + 2, mn, mx, fz); acc_zero(v.w, idx + 3, mn, mx, fz);
+}
+
+template <int B, bool RANDOM>
+__global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const ResArgs a) {
+  constexpr int DPB = 8 / B;
+  constexpr int UNIT = DPB > 4 ? DPB : 4;
+  constexpr int H = UNIT / 4;
+  constexpr int BPU = UNIT / DPB;
+  constexpr int KU = res_reg_groups(B, RANDOM) / H;  // unit rows held in registers
+  constexpr int kWaves = kResThreads / kWave;
+  extern __shared__ float4 s_rows[];  // [lds_rows][H][kResThreads]
+  __shared__ float s_mn[kWaves], s_mx[kWaves];
+  __shared__ uint32_t s_fz[kWaves];
+  __shared__ uint32_t s_k[4];
+
+  const float* __restrict__ xp = a.seg.x;
+  const uint32_t n = static_cast<uint32_t>(a.seg.n);
+  const uint32_t full_units = n / UNIT;
+  const uint32_t wg_u0 = blockIdx.x * a.chunk_units;
+  const uint32_t wg_lim = wg_u0 + a.chunk_units;
+  const uint32_t wg_end = wg_lim < full_units ? wg_lim : full_units;  // <= wg_u0 for a workgroup without a share
+  // A wave's register rows are 24 consecutive 64-unit pieces (24 KiB of contiguous
+  // input per wave: measurably faster than rows spread over the workgroup's
+  // share); the LDS rows follow all register rows.
+  constexpr uint32_t rs = kWave;
+  const uint32_t u0 = wg_u0 + (threadIdx.x / kWave) * (KU * kWave) + (threadIdx.x & (kWave - 1));
+  const uint32_t l0 = wg_u0 + KU * kResThreads + threadIdx.x;
+  constexpr uint32_t stride_bytes = rs * BPU;
+  const float qnan = __builtin_nanf("");  // compares false both ways: ignored by min and max
+
+  // ---- pass 1: load the share, reduce ------------------------------------------
+  float4 v[KU][H];
+  if (wg_u0 + uint32_t(KU * kResThreads) <= wg_end) {
+#pragma unroll
+    for (int k = 0; k < KU; k++)
+#pragma unroll
+      for (int h = 0; h < H; h++) v[k][h] = ld4_stream(xp + size_t(u0 + k * rs) * UNIT + h * 4);
+  } else {
+#pragma unroll
+    for (int k = 0; k < KU; k++) {
+      const uint32_t u = u0 + k * rs;
+#pragma unroll
+      for (int h = 0; h < H; h++)
+        v[k][h] = u < wg_end ? ld4_stream(xp + size_t(u) * UNIT + h * 4) : make_float4(qnan, qnan, qnan, qnan);
+    }
+  }
+  float mn = __builtin_inff(), mx = -__builtin_inff();
+  uint32_t fz = 0xFFFFFFFFu;
+  for (uint32_t r = 0; r < a.lds_rows; r++) {
+    const uint32_t u = l0 + r * kResThreads;
+#pragma unroll
+    for (int h = 0; h < H; h++) {
+      const float4 f = u < wg_end ? ld4_stream(xp + size_t(u) * UNIT + h * 4) : make_float4(qnan, qnan, qnan, qnan);
+      s_rows[(r * H + h) * kResThreads + threadIdx.x] = f;
+      acc_zero4(f, u * UNIT + h * 4, mn, mx, fz);
+    }
+  }
+  // Register rows: min, max and min |x| per element; the index of the first zero is
+  // only worked out by lanes that met one.
+  float am = __builtin_inff();
+#pragma unroll
+  for (int k = 0; k < KU; k++)
+#pragma unroll
+    for (int h = 0; h < H; h++) {
+      acc3(v[k][h].x, mn, mx, am); acc3(v[k][h].y, mn, mx, am);
+      acc3(v[k][h].z, mn, mx, am); acc3(v[k][h].w, mn, mx, am);
+    }
+  if (am == 0.0f) {
+    float d0 = 0.f, d1 = 0.f;
+#pragma unroll
+    for (int k = 0; k < KU; k++)
+#pragma unroll
+      for (int h = 0; h < H; h++) acc_zero4(v[k][h], (u0 + k * rs) * UNIT + h * 4, d0, d1, fz);
+  }
+  if (blockIdx.x == 0 && threadIdx.x == 0)
+    for (uint32_t e = full_units * UNIT; e < n; e++) acc_zero(xp[e], e, mn, mx, fz);
+
+  mn = wave_min(mn);
+  mx = wave_max(mx);
+  fz = wave_min_u32(fz);
+  if ((threadIdx.x & (kWave - 1)) == 0) {
+    s_mn[threadIdx.x / kWave] = mn; s_mx[threadIdx.x / kWave] = mx; s_fz[threadIdx.x / kWave] = fz;
+  }
+  __syncthreads();
+  if (threadIdx.x < kWave) {
+    if (threadIdx.x == 0) {
+#pragma unroll
+      for (int i = 1; i < kWaves; i++) {
+        mn = s_mn[i] < mn ? s_mn[i] : mn;
+        mx = s_mx[i] > mx ? s_mx[i] : mx;
+        fz = s_fz[i] < fz ? s_fz[i] : fz;
+      }
+    }
+    mn = __shfl(mn, 0, 64);
+    mx = __shfl(mx, 0, 64);
+    fz = __shfl(fz, 0, 64);
+    const bool has = mx >= mn;  // false only for a workgroup whose share is empty
+    // lane 0: largest key of x; lane 1: largest complemented key (the minimum);
+    // lane 2: complemented index of the first zero, 0 for none
+    uint32_t key = threadIdx.x == 0 ? (has ? okey(mx) : 0u)
+                 : threadIdx.x == 1 ? (has ? ~okey(mn) : 0u)
+                                    : (fz != 0xFFFFFFFFu ? 0xFFFFFFFEu - fz : 0u);
+#ifndef RES_EXP
+#define RES_EXP 0
+#endif
+#if RES_EXP == 1
+    const bool ok = false;
+#elif RES_EXP == 2
+    const bool ok = grid_exchange(a.bar, a.gen, a.spin_limit, key) && mn == 12345.f;
+#elif RES_EXP == 3
+    const bool ok = true;
+#else
+    const bool ok = grid_exchange(a.bar, a.gen, a.spin_limit, key);
+#endif
+    if (threadIdx.x < 3) s_k[threadIdx.x] = key;
+    if (threadIdx.x == 0) {
+      if (!ok && !RES_EXP) __hip_atomic_store(a.host_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      s_k[3] = ok ? 1u : 0u;
+    }
+  }
+  __syncthreads();
+  if (s_k[3] == 0u) return;
+
+  // ---- pass 2: quantise from registers -------------------------------------------
+  mx = from_okey(s_k[0]);
+  mn = from_okey(~s_k[1]);
+  if ((mn == 0.0f || mx == 0.0f) && s_k[2] != 0u) {
+    // thrust::minmax_element returns the first extreme: a zero extreme carries the
+    // sign of the first zero of the tensor.
+    const float zv = xp[0xFFFFFFFEu - s_k[2]];
+    if (mn == 0.0f) mn = zv;
+    if (mx == 0.0f) mx = zv;
+  }
+  const float gi = inverse_gap(mn, mx, B);
+  if (blockIdx.x == 0 && threadIdx.x == 0) write_header(a.seg.out, B, n, mn, mx);
+
+  uint8_t* __restrict__ pay = a.seg.out + 10;
+  uint32_t draw[UNIT];
+  if (RANDOM) {
+    const uint32_t x0 = a.seg.seed + u0 * BPU;
+#pragma unroll
+    for (int q = 0; q < UNIT; q++) {
+      const int jb = q / DPB, j = q % DPB;
+      draw[q] = lcg_mul(j + 2) * (x0 + jb) + lcg_add(j + 2);
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < KU; k++) {
+    const uint32_t u = u0 + k * rs;
+    const uint32_t packed = quant_unit<B, RANDOM>(v[k], mn, gi, draw, stride_bytes);
+    if (u < wg_end) {
+#pragma unroll
+      for (int jb = 0; jb < BPU; jb++) pay[size_t(u) * BPU + jb] = uint8_t(packed >> (8 * jb));
+    }
+  }
+  if (RANDOM) {
+    uint32_t x0 = a.seg.seed + l0 * BPU;
+    // Keeps the compiler from preparing these draws before the register rows are
+    // done, where they would cost registers the rows need.
+    __asm__ volatile("" : "+v"(x0));
+#pragma unroll
+    for (int q = 0; q < UNIT; q++) {
+      const int jb = q / DPB, j = q % DPB;
+      draw[q] = lcg_mul(j + 2) * (x0 + jb) + lcg_add(j + 2);
+    }
+  }
+  for (uint32_t r = 0; r < a.lds_rows; r++) {
+    const uint32_t u = l0 + r * kResThreads;
+    float4 f[H];
+#pragma unroll
+    for (int h = 0; h < H; h++) f[h] = s_rows[(r * H + h) * kResThreads + threadIdx.x];
+    const uint32_t packed = quant_unit<B, RANDOM>(f, mn, gi, draw, uint32_t(kResThreads) * BPU);
+    if (u < wg_end) {
+#pragma unroll
+      for (int jb = 0; jb < BPU; jb++) pay[size_t(u) * BPU + jb] = uint8_t(packed >> (8 * jb));
+    }
+  }
+  // The unit that holds the end of the tensor, if the length is not a whole number of units.
+  if (blockIdx.x == 0 && threadIdx.x == 0 && full_units * UNIT < n) {
+    uint32_t d[UNIT];
+#pragma unroll
+    for (int q = 0; q < UNIT; q++) {
+      const int jb = q / DPB, j = q % DPB;
+      d[q] = lcg_mul(j + 2) * (a.seg.seed + full_units * BPU + jb) + lcg_add(j + 2);
+    }
+    quant_unit_ragged<B, RANDOM>(a.seg, mn, gi, full_units, d);
   }
 }
 
@@ -610,6 +954,57 @@ __global__ __launch_bounds__(kThreads) void terngrad_decode_multi_kernel(const M
 
 inline int32_t ceil_div(int64_t a, int64_t b) { return static_cast<int32_t>((a + b - 1) / b); }
 
+uint64_t resident_spin_limit() {
+  const int64_t ms = hpx::option(hpx::kOptTerngradBarrierMs);
+  return uint64_t(ms < 0 ? 0 : ms) * 100000ull;  // wall_clock64 ticks at 100 MHz
+}
+
+// Fills chunk_units / lds_rows when tensor (n, bits) fits the chip; false otherwise.
+bool resident_plan(int32_t n, int bits, bool random, const hpx::Workspace* ws, ResArgs& ra) {
+  const int64_t min_elems = hpx::option(hpx::kOptTerngradResidentMin);
+  if (min_elems < 0 || n < min_elems || ws->num_cus <= 0 || ws->num_cus > kBarMaxWorkgroups) return false;
+  const int unit = (8 / bits) > 4 ? (8 / bits) : 4;
+  const int h = unit / 4;
+  const int64_t full_units = n / unit;
+  const int64_t per_wg = (full_units + ws->num_cus - 1) / ws->num_cus;
+  int64_t rows = (per_wg + kResThreads - 1) / kResThreads;
+  if (rows < 1) rows = 1;
+  const int reg_rows = res_reg_groups(bits, random) / h, lds_rows_max = kResLdsGroups / h;
+  if (rows > reg_rows + lds_rows_max) return false;
+  ra.chunk_units = static_cast<uint32_t>(rows * kResThreads);
+  ra.lds_rows = rows > reg_rows ? static_cast<uint32_t>(rows - reg_rows) : 0u;
+  return true;
+}
+
+template <int B, bool RANDOM>
+int launch_resident_as(const ResArgs& ra, int num_cus, hipStream_t st) {
+  constexpr int H = ((8 / B) > 4 ? (8 / B) : 4) / 4;
+  static std::once_flag once;  // per instantiation
+  static hipError_t attr_rc = hipSuccess;
+  std::call_once(once, [] {
+    attr_rc = hipFuncSetAttribute(reinterpret_cast<const void*>(&terngrad_resident_kernel<B, RANDOM>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  kResLdsGroups * kResThreads * int(sizeof(float4)));
+  });
+  HPX_HIP(attr_rc);
+  const size_t lds = size_t(ra.lds_rows) * H * kResThreads * sizeof(float4);
+  if (hpx::g_prof_on) hpx::prof_begin("terngrad_resident_kernel", st);
+  hipLaunchKernelGGL((terngrad_resident_kernel<B, RANDOM>), dim3(num_cus), dim3(kResThreads), lds, st, ra);
+  if (hpx::g_prof_on) hpx::prof_end(st);
+  HPX_HIP(hipGetLastError());
+  return HPX_OK;
+}
+
+int launch_resident(const ResArgs& ra, int num_cus, hipStream_t st) {
+  const bool r = ra.seg.random != 0;
+  switch (ra.seg.bits) {
+    case 1: return r ? launch_resident_as<1, true>(ra, num_cus, st) : launch_resident_as<1, false>(ra, num_cus, st);
+    case 2: return r ? launch_resident_as<2, true>(ra, num_cus, st) : launch_resident_as<2, false>(ra, num_cus, st);
+    case 4: return r ? launch_resident_as<4, true>(ra, num_cus, st) : launch_resident_as<4, false>(ra, num_cus, st);
+    default: return r ? launch_resident_as<8, true>(ra, num_cus, st) : launch_resident_as<8, false>(ra, num_cus, st);
+  }
+}
+
 template <int CAP>
 int launch_encode(int count, const float* const* ins, const int32_t* in_sizes, uint8_t* const* outs,
                   const int32_t* out_sizes, const uint8_t* bitwidths, const int32_t* enable_randoms,
@@ -784,6 +1179,8 @@ HPX_API int hpx_terngrad_encode(int count, const float* const* ins, const int32_
   if (rc != HPX_OK) return rc;
   rc = hpx::ensure_slots(ws, size_t(count) * kSlotsPerTensor);
   if (rc != HPX_OK) return rc;
+  rc = hpx::ensure_barrier(ws);
+  if (rc != HPX_OK) return rc;
   if (++ws->epoch == 0) {
     // The 32-bit tag wrapped: start over from cleared slots.
     HPX_HIP(hipStreamSynchronize(st));
@@ -791,11 +1188,66 @@ HPX_API int hpx_terngrad_encode(int count, const float* const* ins, const int32_
     ws->epoch = 1;
   }
 
-  if (count <= kCapSmall)
-    return launch_encode<kCapSmall>(count, ins, in_sizes, outs, out_sizes, bitwidths, enable_randoms, seeds, ws->slots,
+  // Large tensors take the single-launch resident kernel, the rest the tiled pair.
+  volatile uint32_t* expired = reinterpret_cast<volatile uint32_t*>(ws->pinned + hpx::kPinnedFlagOffset);
+  if (*expired) {
+    *expired = 0;
+    ws->barrier_broken = true;
+    hpx::set_error("hpx_terngrad_encode: the grid barrier of an earlier resident encode on this stream expired; "
+                   "that call's output is invalid. The resident path is now off for this stream.");
+    return HPX_ERR_HIP;
+  }
+  std::vector<int> tiled;
+  tiled.reserve(count);
+  int nres = 0;
+  for (int i = 0; i < count; i++) {
+    ResArgs ra;
+    if (ws->barrier_broken || !resident_plan(in_sizes[i], bitwidths[i], enable_randoms[i] != 0, ws, ra)) {
+      tiled.push_back(i);
+      continue;
+    }
+    const uint64_t seed = seeds ? seeds[i] : hpx::clock_seed();
+    ra.seg = EncSeg{ins[i], outs[i], in_sizes[i], out_sizes[i], static_cast<uint32_t>(seed), bitwidths[i],
+                    static_cast<uint8_t>(enable_randoms[i] != 0), 0};
+    if (++ws->bar_gen == 0) {
+      // The 32-bit generation wrapped: start over from cleared exchange memory.
+      HPX_HIP(hipStreamSynchronize(st));
+      HPX_HIP(hipMemset(ws->bar, 0, hpx::kBarWords * sizeof(uint32_t)));
+      ws->bar_gen = 1;
+    }
+    ra.gen = ws->bar_gen;
+    ra.bar = reinterpret_cast<uint64_t*>(ws->bar);
+    ra.host_flag = const_cast<uint32_t*>(expired);
+    ra.spin_limit = resident_spin_limit();
+    rc = launch_resident(ra, ws->num_cus, st);
+    if (rc != HPX_OK) return rc;
+    nres++;
+  }
+  if (tiled.empty()) return HPX_OK;
+  if (int(tiled.size()) == count) {
+    if (count <= kCapSmall)
+      return launch_encode<kCapSmall>(count, ins, in_sizes, outs, out_sizes, bitwidths, enable_randoms, seeds,
+                                      ws->slots, ws->epoch, st);
+    return launch_encode<kCapLarge>(count, ins, in_sizes, outs, out_sizes, bitwidths, enable_randoms, seeds, ws->slots,
                                     ws->epoch, st);
-  return launch_encode<kCapLarge>(count, ins, in_sizes, outs, out_sizes, bitwidths, enable_randoms, seeds, ws->slots,
-                                  ws->epoch, st);
+  }
+  const int m = int(tiled.size());
+  std::vector<const float*> t_in(m);
+  std::vector<uint8_t*> t_out(m);
+  std::vector<int32_t> t_isz(m), t_osz(m), t_rnd(m);
+  std::vector<uint8_t> t_bits(m);
+  std::vector<uint64_t> t_seed(m);
+  for (int k = 0; k < m; k++) {
+    const int i = tiled[k];
+    t_in[k] = ins[i]; t_out[k] = outs[i]; t_isz[k] = in_sizes[i]; t_osz[k] = out_sizes[i];
+    t_rnd[k] = enable_randoms[i]; t_bits[k] = bitwidths[i];
+    t_seed[k] = seeds ? seeds[i] : hpx::clock_seed();
+  }
+  if (m <= kCapSmall)
+    return launch_encode<kCapSmall>(m, t_in.data(), t_isz.data(), t_out.data(), t_osz.data(), t_bits.data(),
+                                    t_rnd.data(), t_seed.data(), ws->slots, ws->epoch, st);
+  return launch_encode<kCapLarge>(m, t_in.data(), t_isz.data(), t_out.data(), t_osz.data(), t_bits.data(), t_rnd.data(),
+                                  t_seed.data(), ws->slots, ws->epoch, st);
 }
 
 HPX_API int hpx_terngrad_decode(int count, float* const* outs, const int32_t* out_sizes,
