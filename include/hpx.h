@@ -120,7 +120,10 @@ int hpx_tbq_decode(int count, float* const* outs, const int32_t* sizes,
  * 1 bit) is encoded by one launch that keeps it in registers and LDS between the
  * min/max pass and the quantise pass, with a grid-wide barrier in between.  That
  * barrier needs every CU of the device to be reachable from `stream` (no CU
- * mask); its wait is bounded, and if it ever expires the call's output is
+ * mask), and two such kernels must never run at once, so per device only the
+ * first stream that encodes a large tensor uses this kernel (other streams keep
+ * to the two-launch path).  The wait is bounded: if it ever expires (the GPU is
+ * shared with another process's barrier kernels, say) the call's output is
  * invalid, the NEXT hpx_terngrad_encode on the stream returns -2 once and the
  * stream falls back to the two-launch path for good. */
 int hpx_terngrad_encode(int count, const float* const* ins, const int32_t* in_sizes,

@@ -288,6 +288,11 @@ def test_resident_barrier_expiry_is_reported(tg, oracle_cpu, capi):
     rng = np.random.default_rng(5)
     x = rng.normal(0, 1e-2, 3_000_000).astype(np.float32)
     side = torch.cuda.Stream()
+    # Only one stream per device may launch barrier kernels (the first that asks): forget the
+    # workspaces so that the side stream becomes that stream here, and again afterwards so that the
+    # stream of the other tests gets the resident path back.
+    torch.cuda.synchronize()
+    assert capi.load().hpx_release_workspaces() == 0
     old_ms = capi.set_option("terngrad_barrier_ms", 0)
     try:
         with torch.cuda.stream(side):
@@ -303,3 +308,28 @@ def test_resident_barrier_expiry_is_reported(tg, oracle_cpu, capi):
             assert_bits_equal(host(out), ref, "message after fallback")
     finally:
         capi.set_option("terngrad_barrier_ms", old_ms)
+        torch.cuda.synchronize()
+        assert capi.load().hpx_release_workspaces() == 0
+
+
+def test_resident_kernel_belongs_to_one_stream(tg, oracle_cpu, capi):
+    # A second stream encoding a large tensor takes the two-launch path (same bytes out).
+    rng = np.random.default_rng(6)
+    x = rng.normal(0, 1e-2, 3_000_000).astype(np.float32)
+    rc, ref = oracle_cpu.terngrad_encode(x, 2, 1, 9)
+    dx = dev(x)
+    L = capi.load()
+    out0 = tg.encode([dx], [2], [1], [9])[0]
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    L.hpx_profile_reset(); L.hpx_profile_enable(1)
+    try:
+        with torch.cuda.stream(side):
+            out1 = tg.encode([dx], [2], [1], [9])[0]
+            side.synchronize()
+        assert capi.profile_query("terngrad_resident_kernel")[1] == 0
+        assert capi.profile_query("terngrad_quant_kernel")[1] == 1
+    finally:
+        L.hpx_profile_enable(0); L.hpx_profile_reset()
+    assert_bits_equal(host(out0), ref, "owning stream")
+    assert_bits_equal(host(out1), ref, "second stream")

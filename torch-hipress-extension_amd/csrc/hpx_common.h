@@ -86,6 +86,11 @@ int ensure_workspace(Workspace* ws, size_t dev_bytes);
 int ensure_slots(Workspace* ws, size_t words);
 // Zeroed barrier exchange memory and the CU count of the device (both created once).
 int ensure_barrier(Workspace* ws);
+// Kernels that wait at a grid-wide barrier need every CU for themselves: two of them
+// running at once on different streams could each hold CUs the other is waiting
+// for.  So only one stream per device may launch them: the first that asks.
+// Returns whether `ws` is (now) that stream's workspace.
+bool claim_barrier_kernels(Workspace* ws);
 
 uint64_t clock_seed();
 

@@ -111,6 +111,18 @@ int ensure_slots(Workspace* ws, size_t words) {
   return HPX_OK;
 }
 
+static std::map<int, Workspace*> g_barrier_owner;  // guarded by g_ws_mu
+
+bool claim_barrier_kernels(Workspace* ws) {
+  std::lock_guard<std::mutex> g(g_ws_mu);
+  auto it = g_barrier_owner.find(ws->device);
+  if (it == g_barrier_owner.end()) {
+    g_barrier_owner[ws->device] = ws;
+    return true;
+  }
+  return it->second == ws;
+}
+
 int ensure_barrier(Workspace* ws) {
   if (ws->bar) return HPX_OK;
   HPX_HIP(hipDeviceGetAttribute(&ws->num_cus, hipDeviceAttributeMultiprocessorCount, ws->device));
@@ -205,6 +217,7 @@ HPX_API int hpx_release_workspaces(void) {
     if (ws->pinned && hipHostFree(ws->pinned) != hipSuccess) rc = HPX_ERR_HIP;
   }
   hpx::g_ws.clear();
+  hpx::g_barrier_owner.clear();
   if (cur >= 0) (void)hipSetDevice(cur);
   return rc;
 }

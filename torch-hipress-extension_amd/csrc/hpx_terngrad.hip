@@ -1199,10 +1199,10 @@ HPX_API int hpx_terngrad_encode(int count, const float* const* ins, const int32_
   }
   std::vector<int> tiled;
   tiled.reserve(count);
-  int nres = 0;
   for (int i = 0; i < count; i++) {
     ResArgs ra;
-    if (ws->barrier_broken || !resident_plan(in_sizes[i], bitwidths[i], enable_randoms[i] != 0, ws, ra)) {
+    if (ws->barrier_broken || !resident_plan(in_sizes[i], bitwidths[i], enable_randoms[i] != 0, ws, ra) ||
+        !hpx::claim_barrier_kernels(ws)) {
       tiled.push_back(i);
       continue;
     }
@@ -1221,7 +1221,6 @@ HPX_API int hpx_terngrad_encode(int count, const float* const* ins, const int32_
     ra.spin_limit = resident_spin_limit();
     rc = launch_resident(ra, ws->num_cus, st);
     if (rc != HPX_OK) return rc;
-    nres++;
   }
   if (tiled.empty()) return HPX_OK;
   if (int(tiled.size()) == count) {
