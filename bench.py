@@ -37,9 +37,10 @@ N_DGC = 138_357_544
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, each scaled by what the same
 # counter reads for a plain copy of known size.
 MEASURED_TRAFFIC_BYTES = {  # profiles/terngrad_25M_pmc_fetch_write.txt (FETCH x1.99949 + WRITE x1.0, KiB -> bytes)
+    "terngrad_resident_kernel": int((50274.6 * 1.99948 + 6383.5) * 1024),
     "terngrad_minmax_kernel": int((49946.2 * 1.99949 + 122.1) * 1024),
     "terngrad_quant_kernel": int((49957.5 * 1.99949 + 6434.6) * 1024),
-    "terngrad_decode_kernel": int((3573.3 * 1.99949 + 99909.5) * 1024),
+    "terngrad_decode_kernel": int((3571.8 * 1.99948 + 99904.3) * 1024),
 }
 
 
@@ -289,30 +290,42 @@ def extra(torch, np, capi, L, stream, gen):
     r0 = torch.randn(n, device="cuda", generator=gen) * 1e-4
     r = r0.clone()
     out = torch.zeros(4 + 8 * int(np.ceil(n * (1 - 0.999))), dtype=torch.uint8, device="cuda")
-    gd = Call(L.hpx_gd_encode, 1, capi.ptr_array([g.data_ptr()]), capi.i32_array([n]), capi.ptr_array([r.data_ptr()]),
-              capi.ptr_array([out.data_ptr()]), capi.f64_array([0.01]), capi.f64_array([0.999]), capi.u64_array([0]), stream)
-    times = []
     scrub = torch.empty(160_000_000, device="cuda")  # 640 MB, larger than L2 + Infinity Cache
-    for it in range(12):
-        r.copy_(r0)                      # every repetition sees the configuration's residual
-        scrub.sum()                      # push the copy's dirty lines out of the caches: inputs are in HBM when the clock starts
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        gd()
-        torch.cuda.synchronize()
-        times.append(time.perf_counter() - t0)
-    sec = float(np.median(times[2:]))
-    k = (int(out[:4].cpu().numpy().view(np.int32)[0]) - 4) // 8
-    r.copy_(r0)
-    scrub.sum()
-    kt = kernel_times(torch, capi, gd, ["gd_sample_kernel", "gd_select_kernel", "gd_threshold_kernel", "gd_stream_kernel", "gd_scan_kernel",
-                                        "gd_expand_kernel", "gd_sort_pass_kernel"], reps=1)
+    sort_kernels = ["gd_sort_count_kernel", "gd_sort_pass_kernel", "gd_gather_kernel"]
+    all_kernels = ["gd_sample_kernel", "gd_select_kernel", "gd_threshold_kernel", "gd_stream_kernel", "gd_scan_kernel",
+                   "gd_expand_kernel"] + sort_kernels
+    # Whether the sampled threshold lets through more than the `expected` entries (and the call has to sort and
+    # cut) depends on the sample, i.e. on the seed: time several seeds and report each.
+    per_seed = []
+    kt = None
+    for seed in (0, 1 << 24, 2 << 24, 3 << 24, 4 << 24, 5 << 24, 6 << 24, 7 << 24):  # seeds closer than the sample size share most of their sample
+        gd = Call(L.hpx_gd_encode, 1, capi.ptr_array([g.data_ptr()]), capi.i32_array([n]), capi.ptr_array([r.data_ptr()]),
+                  capi.ptr_array([out.data_ptr()]), capi.f64_array([0.01]), capi.f64_array([0.999]), capi.u64_array([seed]), stream)
+        times = []
+        for it in range(7):
+            r.copy_(r0)                      # every repetition sees the configuration's residual
+            scrub.sum()                      # push the copy's dirty lines out of the caches: inputs are in HBM when the clock starts
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            gd()
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+        k = (int(out[:4].cpu().numpy().view(np.int32)[0]) - 4) // 8
+        r.copy_(r0)
+        scrub.sum()
+        kts = kernel_times(torch, capi, gd, all_kernels, reps=1)
+        cut = kts["gd_sort_pass_kernel"] is not None
+        per_seed.append({"seed": seed, "encode_ms": round(float(np.median(times[2:])) * 1e3, 4), "selected": k, "cut": cut})
+        if kt is None or (cut and kt["gd_sort_pass_kernel"] is None):
+            kt = kts
+    sec = float(np.mean([p["encode_ms"] for p in per_seed])) * 1e-3
     dout = torch.zeros(n, device="cuda")
     gdr = Call(L.hpx_gd_decode, 1, capi.ptr_array([out.data_ptr()]), capi.i32_array([out.numel()]),
                capi.ptr_array([dout.data_ptr()]), capi.i32_array([n]), capi.i32_array([1]), stream)
     sec_dec = timed(torch, gdr, 20, 3)
     res["dgc_top0.1pct_138M"] = {
-        "encode_ms": round(sec * 1e3, 4), "encode_GBps_of_gradient": round(4.0 * n / sec / 1e9, 1), "selected": k,
+        "encode_ms": round(sec * 1e3, 4), "encode_ms_is": "mean over the seeds below", "per_seed": per_seed,
+        "encode_GBps_of_gradient": round(4.0 * n / sec / 1e9, 1),
         "algorithmic_bytes": 12.0 * n + 8 * k + 4, "frac_of_hbm_peak": round((12.0 * n + 8 * k + 4) / sec / 1e9 / HBM_PEAK_GBS, 4),
         "stream_kernel_frac_of_hbm_peak": round(12.0 * n / kt["gd_stream_kernel"] / 1e9 / HBM_PEAK_GBS, 4) if kt["gd_stream_kernel"] else None,
         "decode_add_ms": round(sec_dec * 1e3, 4), "kernel_us_per_launch": {k_: round(v * 1e6, 1) for k_, v in kt.items() if v}}

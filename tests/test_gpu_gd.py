@@ -122,6 +122,23 @@ def test_far_more_candidates_than_reserved(gd, oracle_cpu):
     assert info["threshold"] < 3e-7 and info["candidates"] > 390_000 and info["kept"] == oracle_cpu.gd_sizes(n, sr, dr)[1]
 
 
+def test_cut_branch_many_ties(gd, oracle_cpu):
+    # Values on a coarse grid, threshold forced tiny through the sampled positions: nearly every
+    # element is a candidate, thousands share each |r|, and the cut keeps them in ascending index
+    # order within a value (the sort has to be stable across its tiles and passes).
+    rng = np.random.default_rng(11)
+    n, sr, dr, seed = 300_000, 0.01, 0.99, 21
+    g = (np.round(rng.laplace(0, 1e-3, n) * 2000) / 2000).astype(np.float32)
+    g[g == 0] = np.float32(0.0005)
+    sampled = np.array([oracle_cpu.gd_sample_index(seed, x, n) for x in range(3000)])
+    g[sampled] = (1e-7 * (1 + np.arange(3000) / 3000.0)).astype(np.float32)
+    out, msg, info = _check_encode(gd, oracle_cpu, g, np.zeros(n, np.float32), sr, dr, seed)
+    kept = oracle_cpu.gd_sizes(n, sr, dr)[1]
+    assert info["candidates"] > 290_000 and info["kept"] == kept
+    vals = msg[4 + 4 * kept:].view(np.float32)
+    assert np.unique(np.abs(vals)).size < 40      # ties dominate
+
+
 def test_nothing_selected(gd, oracle_cpu):
     n = 50_000
     _check_encode(gd, oracle_cpu, np.zeros(n, np.float32), np.zeros(n, np.float32), 0.05, 0.99, 0)

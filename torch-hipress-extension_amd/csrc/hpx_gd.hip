@@ -333,11 +333,14 @@ __global__ __launch_bounds__(kThreads) void gd_expand_kernel(const uint64_t* __r
   uint32_t pos = chunk_off[tile / kScanChunk] + tile_off[tile] + incl - c;
   const uint32_t e0 = tile * uint32_t(kTile) + lane * kWave;
   if (cut) {
+    const uint32_t thr_bits = st->thr_bits;
     while (m) {
       const uint32_t e = e0 + uint32_t(__builtin_ctzll(m));
       m &= m - 1;
       cand[pos] = int32_t(e);
-      keys[pos] = __float_as_uint(__builtin_fabsf(r[e]));
+      // Sort key: distance of |r| above the threshold in fp32 bit patterns (same order as |r|;
+      // the high digits of such keys are mostly zero, which lets the sort skip its last pass).
+      keys[pos] = __float_as_uint(__builtin_fabsf(r[e])) - thr_bits;
       pos++;
     }
     return;
@@ -354,11 +357,27 @@ __global__ __launch_bounds__(kThreads) void gd_expand_kernel(const uint64_t* __r
   }
 }
 
+// generate_S_value, gd_body.h:80-99, plus the header (gd_body.h:193-201), for a
+// message whose k indices are already in place (the cut path).  A launch of its
+// own with one lane per entry: done by the few workgroups of the last sort pass
+// these random accesses to r took three times as long.
+__global__ __launch_bounds__(kThreads) void gd_gather_kernel(uint8_t* __restrict__ out, float* __restrict__ r, uint32_t k) {
+  const int32_t* idx = reinterpret_cast<const int32_t*>(out + 4);
+  float* val = reinterpret_cast<float*>(out + 4 + size_t(k) * 4);
+  const uint32_t x = blockIdx.x * kThreads + threadIdx.x;
+  if (x == 0) *reinterpret_cast<int32_t*>(out) = int32_t(4 + k * 8);
+  if (x < k) {
+    const int32_t i = idx[x];
+    val[x] = r[i];
+    r[i] = 0.0f;
+  }
+}
+
 // ---- cut to the `expected` largest |r| (gd_body.h:176-187) ------------------
 // Stable LSD radix sort of (key, index) pairs, 8 bits per pass, descending
 // (bin = 255 - digit).  A pass is a count launch and a scatter launch over tiles
 // of 8192 pairs (1024 lanes x 8), counts[tile * 256 + bin]; the last pass writes
-// the message instead of a sorted list.  (Counting a pass's digits where its
+// the message's index block instead of a sorted list.  (Counting a pass's digits where its
 // input is written, with global atomics, saves the count launches but was five
 // times slower: some 10^5 scattered atomics cost more than the launches.)
 struct SortArgs {
@@ -370,15 +389,29 @@ struct SortArgs {
   uint32_t nblk;
   uint32_t* keys_out;       // not used by the last pass
   int32_t* idx_out;
-  uint8_t* msg;             // last pass only: the message, of which the first `keep` pairs are written
-  float* r;
+  uint8_t* msg;             // last pass only: the message, whose index block gets the first `keep` indices
   uint32_t keep;
 };
 
+// Lanes of the wave whose `bin` equals this lane's, among the lanes in `live`.
+__device__ __forceinline__ uint64_t match_bin(uint32_t bin, bool live) {
+  uint64_t same = __ballot(live);
+#pragma unroll
+  for (int b = 0; b < 8; b++) {
+    const uint64_t m = __ballot((bin >> b) & 1u);
+    same &= ((bin >> b) & 1u) ? m : ~m;
+  }
+  return same;
+}
+
+// One LDS atomic per distinct bin of a wave's 64 keys, not one per key: the top
+// digit of keys that are all just above one threshold is the same for nearly all
+// of them, and 8192 atomics on one LDS word took longer than the rest of the pass.
 __global__ __launch_bounds__(kSortThreads) void gd_sort_count_kernel(const uint32_t* __restrict__ keys, uint32_t n,
                                                                      int shift, uint32_t* __restrict__ counts) {
   __shared__ uint32_t s_hist[256];
   const uint32_t t = threadIdx.x;
+  const uint32_t lane = t & (kWave - 1);
   if (t < 256) s_hist[t] = 0;
   const uint32_t b0 = blockIdx.x * uint32_t(kSortTile);
   uint32_t key[kSortPer];
@@ -389,8 +422,12 @@ __global__ __launch_bounds__(kSortThreads) void gd_sort_count_kernel(const uint3
   }
   __syncthreads();
 #pragma unroll
-  for (int j = 0; j < kSortPer; j++)
-    if (b0 + j * kSortThreads + t < n) atomicAdd(&s_hist[255u - ((key[j] >> shift) & 255u)], 1u);
+  for (int j = 0; j < kSortPer; j++) {
+    const bool live = b0 + j * kSortThreads + t < n;
+    const uint32_t bin = 255u - ((key[j] >> shift) & 255u);
+    const uint64_t same = match_bin(bin, live);
+    if (live && (same & ((uint64_t(1) << lane) - 1)) == 0) atomicAdd(&s_hist[bin], uint32_t(__popcll(same)));
+  }
   __syncthreads();
   if (t < 256) counts[size_t(blockIdx.x) * 256 + t] = s_hist[t];
 }
@@ -445,6 +482,17 @@ __global__ __launch_bounds__(kSortThreads) void gd_sort_pass_kernel(const SortAr
       mine += q == blockIdx.x ? v : 0u;
     }
   }
+  if (a.msg) {
+    // Last pass: if every key has the same digit the input is already in order.
+    if (__syncthreads_or(t < 256 && total == n)) {
+#pragma unroll
+      for (int j = 0; j < kSortPer; j++) {
+        const uint32_t x = x0 + j * kWave;
+        if (x < n && x < a.keep) reinterpret_cast<int32_t*>(a.msg + 4)[x] = id[j];
+      }
+      return;
+    }
+  }
 #pragma unroll
   for (int q = 0; q < 256 / kWave; q++) s_cnt[wave][q * kWave + lane] = 0;  // own row: no barrier needed before use
 
@@ -453,12 +501,7 @@ __global__ __launch_bounds__(kSortThreads) void gd_sort_pass_kernel(const SortAr
   for (int j = 0; j < kSortPer; j++) {
     const bool live = x0 + j * kWave < n;
     bin[j] = 255u - ((key[j] >> a.shift) & 255u);
-    uint64_t same = __ballot(live);
-#pragma unroll
-    for (int b = 0; b < 8; b++) {
-      const uint64_t m = __ballot((bin[j] >> b) & 1u);
-      same &= ((bin[j] >> b) & 1u) ? m : ~m;
-    }
+    const uint64_t same = match_bin(bin[j], live);
     const uint32_t rank = __popcll(same & ((uint64_t(1) << lane) - 1));
     uint32_t base = 0;
     if (live && rank == 0) {
@@ -503,7 +546,6 @@ __global__ __launch_bounds__(kSortThreads) void gd_sort_pass_kernel(const SortAr
   }
   __syncthreads();
   const uint32_t live_n = n - b0 < uint32_t(kSortTile) ? n - b0 : uint32_t(kSortTile);
-  if (a.msg && blockIdx.x == 0 && t == 0) *reinterpret_cast<int32_t*>(a.msg) = int32_t(4 + a.keep * 8);
 #pragma unroll
   for (int j = 0; j < kSortPer; j++) {
     const uint32_t p = j * kSortThreads + t;
@@ -513,12 +555,8 @@ __global__ __launch_bounds__(kSortThreads) void gd_sort_pass_kernel(const SortAr
       const uint32_t b = 255u - ((k >> a.shift) & 255u);
       const uint32_t slot = s_slot[b] + (p - s_first[b]);
       if (a.msg) {
-        // generate_S_value, gd_body.h:80-99, for the pairs that survive the cut
-        if (slot < a.keep) {
-          reinterpret_cast<int32_t*>(a.msg + 4)[slot] = i;
-          reinterpret_cast<float*>(a.msg + 4 + size_t(a.keep) * 4)[slot] = a.r[i];
-          a.r[i] = 0.0f;
-        }
+        // last pass: the indices that survive the cut go straight into the message
+        if (slot < a.keep) reinterpret_cast<int32_t*>(a.msg + 4)[slot] = i;
       } else {
         a.keys_out[slot] = k;
         a.idx_out[slot] = i;
@@ -553,8 +591,8 @@ inline uint32_t cdiv(uint64_t a, uint64_t b) { return static_cast<uint32_t>((a +
 inline size_t align256(size_t x) { return (x + 255) & ~size_t(255); }
 
 // The four passes of the cut path: (keys_a, idx_a) hold the candidates in index
-// order.  The last pass writes the `keep` largest into the message `msg` and
-// clears their residual entries.
+// order.  The last pass writes the indices of the `keep` largest into the
+// message `msg`; a gather launch adds values and header and clears the residual.
 int sort_and_cut(uint32_t* keys_a, int32_t* idx_a, uint32_t* keys_b, int32_t* idx_b, uint32_t* counts, uint32_t n,
                  uint8_t* msg, float* r, uint32_t keep, hipStream_t st) {
   static std::once_flag once;
@@ -572,7 +610,7 @@ int sort_and_cut(uint32_t* keys_a, int32_t* idx_a, uint32_t* keys_b, int32_t* id
     a.counts = counts; a.nblk = nblk;
     a.keys_out = keys_b; a.idx_out = idx_b;
     a.msg = pass == 3 ? msg : nullptr;
-    a.r = r; a.keep = keep;
+    a.keep = keep;
     HPX_LAUNCH("gd_sort_count_kernel", gd_sort_count_kernel, dim3(nblk), dim3(kSortThreads), st, keys_a, n, a.shift, counts);
     if (hpx::g_prof_on) hpx::prof_begin("gd_sort_pass_kernel", st);
     hipLaunchKernelGGL(gd_sort_pass_kernel, dim3(nblk), dim3(kSortThreads), kStageBytes, st, a);
@@ -581,6 +619,8 @@ int sort_and_cut(uint32_t* keys_a, int32_t* idx_a, uint32_t* keys_b, int32_t* id
     std::swap(keys_a, keys_b);
     std::swap(idx_a, idx_b);
   }
+  HPX_LAUNCH("gd_gather_kernel", gd_gather_kernel, dim3(cdiv(keep > 0 ? keep : 1, kThreads)), dim3(kThreads), st, msg, r, keep);
+  HPX_HIP(hipGetLastError());
   return HPX_OK;
 }
 
