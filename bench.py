@@ -314,9 +314,9 @@ def extra(torch, np, capi, L, stream, gen):
         r.copy_(r0)
         scrub.sum()
         kts = kernel_times(torch, capi, gd, all_kernels, reps=1)
-        cut = kts["gd_sort_pass_kernel"] is not None
+        cut = kts["gd_gather_kernel"] is not None
         per_seed.append({"seed": seed, "encode_ms": round(float(np.median(times[2:])) * 1e3, 4), "selected": k, "cut": cut})
-        if kt is None or (cut and kt["gd_sort_pass_kernel"] is None):
+        if kt is None or (cut and kt["gd_gather_kernel"] is None):
             kt = kts
     sec = float(np.mean([p["encode_ms"] for p in per_seed])) * 1e-3
     dout = torch.zeros(n, device="cuda")

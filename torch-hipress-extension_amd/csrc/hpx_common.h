@@ -91,6 +91,10 @@ int ensure_barrier(Workspace* ws);
 // for.  So only one stream per device may launch them: the first that asks.
 // Returns whether `ws` is (now) that stream's workspace.
 bool claim_barrier_kernels(Workspace* ws);
+// Call with ws->mu held and the workspace ensured, before queueing work: if a barrier kernel of an
+// earlier call on this stream gave up waiting, reports it once (HPX_ERR_HIP, text names `who`) and
+// turns barrier kernels off for the stream.
+int check_barrier_expired(Workspace* ws, const char* who);
 
 uint64_t clock_seed();
 
@@ -183,6 +187,92 @@ __device__ __forceinline__ int find_segment(const int32_t (&start)[CAP + 1], int
     return s;
   }
 }
+
+// ---- grid-wide exchange / barrier --------------------------------------------
+// For kernels launched with at most kBarMaxWorkgroups workgroups that are all
+// resident at once (the host guarantees it: grid <= CUs, one workgroup fits a CU,
+// and only one stream per device launches such kernels).
+constexpr int kBarGroup = 16;           // workgroups per group; also the largest number of groups
+constexpr int kBarMaxWorkgroups = kBarGroup * kBarGroup;
+constexpr int kBarRecWords = 4;         // 64-bit words per record (three used)
+constexpr int kBarAreaWords = kBarGroup * kBarRecWords;  // one area: 16 records = 64 words = 512 bytes
+// Exchange memory, in 64-bit words: group areas first (members report here), then
+// one area per workgroup (group leaders report here).
+constexpr size_t kBarGroupBase = 0;
+constexpr size_t kBarWgBase = size_t(kBarGroup) * kBarAreaWords;
+constexpr size_t kBarTotalWords = kBarWgBase + size_t(kBarMaxWorkgroups) * kBarAreaWords;
+static_assert(kBarTotalWords * 8 <= kBarWords * 4, "barrier memory too small");
+
+
+// Grid-wide exchange of (max key, min key, first-zero key) and barrier in one.
+// Every lane of wave 0 of every workgroup calls it once per launch with the
+// workgroup's three keys; on success every lane holds the grid-wide maximum of
+// key[lane & 3] (lanes with (lane & 3) == 3 hold nothing of use).
+//
+// The protocol uses only stores and polling loads, no read-modify-write and no
+// fence: a member writes its record (three self-validating words, generation in
+// the high half) into its group's area; the group's leader polls that area with
+// one wave-wide load until all records carry this generation, folds them, and
+// writes the group's record into the area of EVERY workgroup; each workgroup
+// polls its own area until all groups have reported.  A polled line has one
+// reader, a written line at most 16 writers, and the critical path is two
+// store-to-load hand-overs.  (A counter-based barrier - fence, two dependent
+// atomics, a release flag, then reading the reduction slots - took 7 us here;
+// polling one shared word from all 256 workgroups took 10.)
+__device__ __forceinline__ bool grid_exchange(uint64_t* bar, uint32_t gen, uint64_t spin_limit, uint32_t& key) {
+  const uint32_t lane = threadIdx.x;  // < 64
+  const uint32_t nwg = gridDim.x, grp = blockIdx.x / kBarGroup, mem = blockIdx.x % kBarGroup;
+  const uint32_t ngrp = (nwg + kBarGroup - 1) / kBarGroup;
+  const uint32_t left = nwg - grp * kBarGroup;
+  const uint32_t gsz = left < uint32_t(kBarGroup) ? left : uint32_t(kBarGroup);
+  const uint64_t tag = uint64_t(gen) << 32;
+  const uint64_t t0 = wall_clock64();
+  unsigned long long* garea = reinterpret_cast<unsigned long long*>(bar) + kBarGroupBase + size_t(grp) * kBarAreaWords;
+  unsigned long long* warea = reinterpret_cast<unsigned long long*>(bar) + kBarWgBase + size_t(blockIdx.x) * kBarAreaWords;
+  const uint32_t rec = lane / kBarRecWords, word = lane % kBarRecWords;
+
+  if (lane < 3) __hip_atomic_store(&garea[mem * kBarRecWords + lane], tag | key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+
+  bool ok = true;
+  if (mem == 0) {  // group leader
+    uint32_t k = 0;
+    for (;;) {
+      const unsigned long long v = __hip_atomic_load(&garea[lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const bool valid = word == 3 || rec >= gsz || uint32_t(v >> 32) == gen;
+      k = (word == 3 || rec >= gsz) ? 0u : uint32_t(v);
+      if (__ballot(valid) == ~0ull) break;
+      if (wall_clock64() - t0 > spin_limit) { ok = false; break; }
+      __builtin_amdgcn_s_sleep(1);
+    }
+    if (ok) {
+#pragma unroll
+      for (int o = kBarRecWords; o < kWave; o <<= 1) { const uint32_t t = __shfl_xor(k, o, 64); k = t > k ? t : k; }
+      // lane l now holds the group's key (l & 3); lanes 0..2 of each quad of lanes write it out
+      unsigned long long* wbase = reinterpret_cast<unsigned long long*>(bar) + kBarWgBase + size_t(grp) * kBarRecWords;
+      if (word < 3) {
+        for (uint32_t w = rec; w < nwg; w += kWave / kBarRecWords)
+          __hip_atomic_store(&wbase[size_t(w) * kBarAreaWords + word], tag | k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+  }
+  ok = __builtin_amdgcn_readfirstlane(ok ? 1 : 0) != 0;
+  if (!ok) return false;
+
+  uint32_t k = 0;
+  for (;;) {
+    const unsigned long long v = __hip_atomic_load(&warea[lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const bool valid = word == 3 || rec >= ngrp || uint32_t(v >> 32) == gen;
+    k = (word == 3 || rec >= ngrp) ? 0u : uint32_t(v);
+    if (__ballot(valid) == ~0ull) break;
+    if (wall_clock64() - t0 > spin_limit) return false;
+    __builtin_amdgcn_s_sleep(1);
+  }
+#pragma unroll
+  for (int o = kBarRecWords; o < kWave; o <<= 1) { const uint32_t t = __shfl_xor(k, o, 64); k = t > k ? t : k; }
+  key = k;
+  return true;
+}
+
 
 // The reference's 32-bit LCG (naive_random.hpp:15-33): x <- a*x + c.
 constexpr uint32_t kLcgA = 1103515245u;

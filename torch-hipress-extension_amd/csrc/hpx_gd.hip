@@ -377,7 +377,10 @@ __global__ __launch_bounds__(kThreads) void gd_gather_kernel(uint8_t* __restrict
 // Stable LSD radix sort of (key, index) pairs, 8 bits per pass, descending
 // (bin = 255 - digit).  A pass is a count launch and a scatter launch over tiles
 // of 8192 pairs (1024 lanes x 8), counts[tile * 256 + bin]; the last pass writes
-// the message's index block instead of a sorted list.  (Counting a pass's digits where its
+// the message's index block instead of a sorted list.  (All passes in one launch
+// with grid-wide barriers was tried and lost: data handed between workgroups
+// inside a launch needs device-scope accesses or whole-L2 fences, either of
+// which costs more than the launches saved.)  (Counting a pass's digits where its
 // input is written, with global atomics, saves the count launches but was five
 // times slower: some 10^5 scattered atomics cost more than the launches.)
 struct SortArgs {

@@ -123,6 +123,16 @@ bool claim_barrier_kernels(Workspace* ws) {
   return it->second == ws;
 }
 
+int check_barrier_expired(Workspace* ws, const char* who) {
+  volatile uint32_t* expired = reinterpret_cast<volatile uint32_t*>(ws->pinned + kPinnedFlagOffset);
+  if (!*expired) return HPX_OK;
+  *expired = 0;
+  ws->barrier_broken = true;
+  set_error("%s: the grid barrier of an earlier call on this stream expired; that call's output is invalid. "
+            "Kernels that use a grid barrier are now off for this stream.", who);
+  return HPX_ERR_HIP;
+}
+
 int ensure_barrier(Workspace* ws) {
   if (ws->bar) return HPX_OK;
   HPX_HIP(hipDeviceGetAttribute(&ws->num_cus, hipDeviceAttributeMultiprocessorCount, ws->device));

@@ -416,17 +416,6 @@ constexpr int kResRegGroups = 24;  // float4 per lane held in registers ...
 // ... except at 1 bit with stochastic rounding, whose eight draws per lane need the room.
 constexpr int res_reg_groups(int bits, bool random) { return (bits == 1 && random) ? 14 : kResRegGroups; }
 constexpr int kResLdsGroups = 8;   // float4 per lane held in LDS (128 KiB per workgroup)
-constexpr int kBarGroup = 16;           // workgroups per group; also the largest number of groups
-constexpr int kBarMaxWorkgroups = kBarGroup * kBarGroup;
-constexpr int kBarRecWords = 4;         // 64-bit words per record (three used)
-constexpr int kBarAreaWords = kBarGroup * kBarRecWords;  // one area: 16 records = 64 words = 512 bytes
-// Exchange memory, in 64-bit words: group areas first (members report here), then
-// one area per workgroup (group leaders report here).
-constexpr size_t kBarGroupBase = 0;
-constexpr size_t kBarWgBase = size_t(kBarGroup) * kBarAreaWords;
-constexpr size_t kBarTotalWords = kBarWgBase + size_t(kBarMaxWorkgroups) * kBarAreaWords;
-static_assert(kBarTotalWords * 8 <= hpx::kBarWords * 4, "barrier memory too small");
-
 struct ResArgs {
   EncSeg seg;
   uint32_t chunk_units;  // units per workgroup, a multiple of kResThreads
@@ -436,75 +425,6 @@ struct ResArgs {
   uint32_t* host_flag;   // pinned host word, set to 1 when the barrier wait expires
   uint64_t spin_limit;
 };
-
-// Grid-wide exchange of (max key, min key, first-zero key) and barrier in one.
-// Every lane of wave 0 of every workgroup calls it once per launch with the
-// workgroup's three keys; on success every lane holds the grid-wide maximum of
-// key[lane & 3] (lanes with (lane & 3) == 3 hold nothing of use).
-//
-// The protocol uses only stores and polling loads, no read-modify-write and no
-// fence: a member writes its record (three self-validating words, generation in
-// the high half) into its group's area; the group's leader polls that area with
-// one wave-wide load until all records carry this generation, folds them, and
-// writes the group's record into the area of EVERY workgroup; each workgroup
-// polls its own area until all groups have reported.  A polled line has one
-// reader, a written line at most 16 writers, and the critical path is two
-// store-to-load hand-overs.  (A counter-based barrier - fence, two dependent
-// atomics, a release flag, then reading the reduction slots - took 7 us here;
-// polling one shared word from all 256 workgroups took 10.)
-__device__ __forceinline__ bool grid_exchange(uint64_t* bar, uint32_t gen, uint64_t spin_limit, uint32_t& key) {
-  const uint32_t lane = threadIdx.x;  // < 64
-  const uint32_t nwg = gridDim.x, grp = blockIdx.x / kBarGroup, mem = blockIdx.x % kBarGroup;
-  const uint32_t ngrp = (nwg + kBarGroup - 1) / kBarGroup;
-  const uint32_t left = nwg - grp * kBarGroup;
-  const uint32_t gsz = left < uint32_t(kBarGroup) ? left : uint32_t(kBarGroup);
-  const uint64_t tag = uint64_t(gen) << 32;
-  const uint64_t t0 = wall_clock64();
-  unsigned long long* garea = reinterpret_cast<unsigned long long*>(bar) + kBarGroupBase + size_t(grp) * kBarAreaWords;
-  unsigned long long* warea = reinterpret_cast<unsigned long long*>(bar) + kBarWgBase + size_t(blockIdx.x) * kBarAreaWords;
-  const uint32_t rec = lane / kBarRecWords, word = lane % kBarRecWords;
-
-  if (lane < 3) __hip_atomic_store(&garea[mem * kBarRecWords + lane], tag | key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-
-  bool ok = true;
-  if (mem == 0) {  // group leader
-    uint32_t k = 0;
-    for (;;) {
-      const unsigned long long v = __hip_atomic_load(&garea[lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const bool valid = word == 3 || rec >= gsz || uint32_t(v >> 32) == gen;
-      k = (word == 3 || rec >= gsz) ? 0u : uint32_t(v);
-      if (__ballot(valid) == ~0ull) break;
-      if (wall_clock64() - t0 > spin_limit) { ok = false; break; }
-      __builtin_amdgcn_s_sleep(1);
-    }
-    if (ok) {
-#pragma unroll
-      for (int o = kBarRecWords; o < kWave; o <<= 1) { const uint32_t t = __shfl_xor(k, o, 64); k = t > k ? t : k; }
-      // lane l now holds the group's key (l & 3); lanes 0..2 of each quad of lanes write it out
-      unsigned long long* wbase = reinterpret_cast<unsigned long long*>(bar) + kBarWgBase + size_t(grp) * kBarRecWords;
-      if (word < 3) {
-        for (uint32_t w = rec; w < nwg; w += kWave / kBarRecWords)
-          __hip_atomic_store(&wbase[size_t(w) * kBarAreaWords + word], tag | k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
-    }
-  }
-  ok = __builtin_amdgcn_readfirstlane(ok ? 1 : 0) != 0;
-  if (!ok) return false;
-
-  uint32_t k = 0;
-  for (;;) {
-    const unsigned long long v = __hip_atomic_load(&warea[lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const bool valid = word == 3 || rec >= ngrp || uint32_t(v >> 32) == gen;
-    k = (word == 3 || rec >= ngrp) ? 0u : uint32_t(v);
-    if (__ballot(valid) == ~0ull) break;
-    if (wall_clock64() - t0 > spin_limit) return false;
-    __builtin_amdgcn_s_sleep(1);
-  }
-#pragma unroll
-  for (int o = kBarRecWords; o < kWave; o <<= 1) { const uint32_t t = __shfl_xor(k, o, 64); k = t > k ? t : k; }
-  key = k;
-  return true;
-}
 
 __device__ __forceinline__ void acc_zero(float v, uint32_t idx, float& mn, float& mx, uint32_t& fz) {
   mn = v < mn ? v : mn;
@@ -616,21 +536,10 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
     uint32_t key = threadIdx.x == 0 ? (has ? okey(mx) : 0u)
                  : threadIdx.x == 1 ? (has ? ~okey(mn) : 0u)
                                     : (fz != 0xFFFFFFFFu ? 0xFFFFFFFEu - fz : 0u);
-#ifndef RES_EXP
-#define RES_EXP 0
-#endif
-#if RES_EXP == 1
-    const bool ok = false;
-#elif RES_EXP == 2
-    const bool ok = grid_exchange(a.bar, a.gen, a.spin_limit, key) && mn == 12345.f;
-#elif RES_EXP == 3
-    const bool ok = true;
-#else
     const bool ok = grid_exchange(a.bar, a.gen, a.spin_limit, key);
-#endif
     if (threadIdx.x < 3) s_k[threadIdx.x] = key;
     if (threadIdx.x == 0) {
-      if (!ok && !RES_EXP) __hip_atomic_store(a.host_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      if (!ok) __hip_atomic_store(a.host_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
       s_k[3] = ok ? 1u : 0u;
     }
   }
@@ -1189,14 +1098,9 @@ HPX_API int hpx_terngrad_encode(int count, const float* const* ins, const int32_
   }
 
   // Large tensors take the single-launch resident kernel, the rest the tiled pair.
-  volatile uint32_t* expired = reinterpret_cast<volatile uint32_t*>(ws->pinned + hpx::kPinnedFlagOffset);
-  if (*expired) {
-    *expired = 0;
-    ws->barrier_broken = true;
-    hpx::set_error("hpx_terngrad_encode: the grid barrier of an earlier resident encode on this stream expired; "
-                   "that call's output is invalid. The resident path is now off for this stream.");
-    return HPX_ERR_HIP;
-  }
+  rc = hpx::check_barrier_expired(ws, "hpx_terngrad_encode");
+  if (rc != HPX_OK) return rc;
+  uint32_t* expired = reinterpret_cast<uint32_t*>(ws->pinned + hpx::kPinnedFlagOffset);
   std::vector<int> tiled;
   tiled.reserve(count);
   for (int i = 0; i < count; i++) {
@@ -1217,7 +1121,7 @@ HPX_API int hpx_terngrad_encode(int count, const float* const* ins, const int32_
     }
     ra.gen = ws->bar_gen;
     ra.bar = reinterpret_cast<uint64_t*>(ws->bar);
-    ra.host_flag = const_cast<uint32_t*>(expired);
+    ra.host_flag = expired;
     ra.spin_limit = resident_spin_limit();
     rc = launch_resident(ra, ws->num_cus, st);
     if (rc != HPX_OK) return rc;
