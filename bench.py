@@ -364,6 +364,33 @@ def extra(torch, np, capi, L, stream, gen):
         "frac_of_hbm_peak_three_phase_bytes": round(32.0 * elems / sec / 1e9 / HBM_PEAK_GBS, 4),
         "mfma_frac_of_fp32_peak": round(flops / sec / 1e12 / FP32_MFMA_PEAK_TF, 5),
         "kernel_us_per_launch": {k_: round(v * 1e6, 1) for k_, v in kt.items() if v}}
+    del G, R
+    torch.cuda.empty_cache()
+
+    # ---- the scheduler around the path: one COMP task, submit -> name in the finished queue ------------
+    # (TernGrad 2-bit, 25.56 M elements; includes the 6.4 MB device-to-host copy of the message into a
+    # pinned C buffer and both thread hand-overs; the reference's worker polls its queue every 500 us)
+    hp = importlib.import_module("torch-hipress-extension_amd").hp_cuda
+    if hp.init("terngrad", {"enable_random": 1, "bitwidth": 2, "seed": 0}, torch.cuda.current_device(), 0, 2):
+        n = N_TERNGRAD
+        x = outlier_gradient(torch, n, gen)
+        nbytes = 10 + (n + 3) // 4
+        B = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+        Cc = torch.zeros(nbytes, dtype=torch.uint8, pin_memory=True)
+        torch.cuda.synchronize()
+        lat = []
+        for it in range(30):
+            t0 = time.perf_counter()
+            hp.submit_task("g", x, B, Cc, 0, 10)
+            while not hp.getResults(10):
+                hp.wait(10, 100)
+            lat.append(time.perf_counter() - t0)
+        hp.end()
+        lat = np.array(lat[5:])
+        res["scheduler_terngrad_comp_task_25M"] = {
+            "submit_to_finished_ms_median": round(float(np.median(lat)) * 1e3, 4),
+            "submit_to_finished_ms_min": round(float(lat.min()) * 1e3, 4), "message_bytes_to_host": nbytes,
+            "errors": hp.error_count()}
     return res
 
 

@@ -1,0 +1,224 @@
+"""GPU parity of the task scheduler (hp_cuda.init / submit_task / getResults over libhpx.so) against the
+CPU oracle: what a COMP, DECOMP and ROOT_DECOMP_COMP task leaves in C, in the gradient and in the
+residual, and which finished queue its name appears in (hp_cuda.cpp:163-772, :1043-1066)."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import assert_bits_equal, dev, host
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture
+def hp(pkg):
+    assert torch.cuda.is_available()
+    yield pkg.hp_cuda
+    pkg.hp_cuda.end()
+    for q in (10, 20, 30):
+        pkg.hp_cuda.getResults(q)
+
+
+def _collect(hp, task_id, names, timeout_s=20.0):
+    got = []
+    import time
+    t0 = time.time()
+    while len(got) < len(names) and time.time() - t0 < timeout_s:
+        hp.wait(task_id, 200)
+        got += hp.getResults(task_id)
+    assert sorted(got) == sorted(names), (got, names, hp.last_error())
+    return got
+
+
+def _host_buf(nbytes, pinned):
+    return torch.zeros(nbytes, dtype=torch.uint8, pin_memory=bool(pinned))
+
+
+@pytest.mark.parametrize("pinned", [0, 1])
+def test_terngrad_comp_decomp_root(hp, oracle_cpu, pinned):
+    rng = np.random.default_rng(1)
+    n, b, seed, size, rank = 100_003, 2, 5, 3, 1
+    assert hp.init("terngrad", {"enable_random": 1, "bitwidth": b, "seed": seed}, 0, rank, size)
+    msg_bytes = oracle_cpu.terngrad_packed_size(n, b)
+
+    # COMP: tensor -> B -> C
+    x = rng.normal(0, 1e-2, n).astype(np.float32)
+    dx = dev(x)
+    B = torch.zeros(msg_bytes, dtype=torch.uint8, device="cuda")
+    Cc = _host_buf(msg_bytes, pinned)
+    torch.cuda.synchronize()
+    assert hp.submit_task("layer0.weight", dx, B, Cc, 0, 10)
+    _collect(hp, 10, ["layer0.weight"])
+    rc, ref = oracle_cpu.terngrad_encode(x, b, 1, seed)
+    assert_bits_equal(Cc.numpy(), ref, "COMP message in C")
+    assert hp.getResults(20) == [] and hp.getResults(30) == []
+
+    # DECOMP, write (is_root 0) and add (is_root 1): C -> B -> tensor
+    for is_root in (0, 1):
+        base = rng.normal(0, 1, n).astype(np.float32)
+        dt = dev(base)
+        Cd = _host_buf(msg_bytes, pinned); Cd.numpy()[:] = ref
+        Bd = torch.zeros(msg_bytes, dtype=torch.uint8, device="cuda")
+        torch.cuda.synchronize()
+        assert hp.submit_task(f"dec{is_root}", dt, Bd, Cd, is_root, 20)
+        _collect(hp, 20, [f"dec{is_root}"])
+        rc, want = oracle_cpu.terngrad_decode(ref, n, base.copy(), is_root)
+        assert_bits_equal(host(dt), want, f"DECOMP is_root={is_root}")
+
+    # ROOT: decode every gathered slot but our own rank's (add), then re-encode the sum
+    others = [rng.normal(0, 1e-2, n).astype(np.float32) for _ in range(size)]
+    slots = np.zeros(size * msg_bytes, np.uint8)
+    for i in range(size):
+        rc, m = oracle_cpu.terngrad_encode(others[i], b, 1, 100 + i)
+        slots[i * msg_bytes:(i + 1) * msg_bytes] = m
+    slots[rank * msg_bytes:(rank + 1) * msg_bytes] = 0xEE            # never read
+    mine = rng.normal(0, 1e-2, n).astype(np.float32)
+    dmine = dev(mine)
+    Cr = _host_buf(size * msg_bytes, pinned); Cr.numpy()[:] = slots
+    Br = torch.zeros(msg_bytes, dtype=torch.uint8, device="cuda")
+    torch.cuda.synchronize()
+    assert hp.submit_task("root.w", dmine, Br, Cr, 1, 30)
+    _collect(hp, 30, ["root.w"])
+    want = mine.copy()
+    for i in range(size):
+        if i != rank:
+            rc, want = oracle_cpu.terngrad_decode(slots[i * msg_bytes:(i + 1) * msg_bytes], n, want, 1)
+    assert_bits_equal(host(dmine), want, "ROOT: gradient after the gathered slots were added")
+    rc, ref2 = oracle_cpu.terngrad_encode(want, b, 1, seed)
+    assert_bits_equal(Cr.numpy()[:msg_bytes], ref2, "ROOT: re-encoded message in C")
+    assert_bits_equal(Cr.numpy()[msg_bytes:], slots[msg_bytes:], "ROOT: the other slots of C are untouched")
+    assert hp.error_count() == 0, hp.last_error()
+
+
+def test_tbq_batch_of_mixed_tasks(hp, oracle_cpu):
+    rng = np.random.default_rng(2)
+    thr, size, rank = 2e-3, 4, 0
+    assert hp.init("tbq", {"threshold": thr}, 0, rank, size)
+    keep, checks = [], []
+    sizes = [int(s) for s in rng.integers(5, 70_000, 24)]
+    for k, n in enumerate(sizes):
+        kind = (10, 20, 30)[k % 3]
+        mb = oracle_cpu.tbq_packed_size(n)
+        g = rng.normal(0, 1e-3, n).astype(np.float32)
+        r = rng.normal(0, 1e-3, n).astype(np.float32)
+        dg, dr = dev(g), dev(r)
+        B = torch.zeros(mb, dtype=torch.uint8, device="cuda")
+        if kind == 10:
+            Cc = _host_buf(mb, k & 1)
+            checks.append((kind, f"t{k}", g, r, dg, dr, Cc, None))
+        elif kind == 20:
+            src = rng.normal(0, 1e-3, n).astype(np.float32)
+            msg = oracle_cpu.tbq_encode(src, np.zeros(n, np.float32), thr)
+            Cc = _host_buf(mb, k & 1); Cc.numpy()[:] = msg
+            checks.append((kind, f"t{k}", g, r, dg, dr, Cc, msg))
+        else:
+            slots = np.zeros(size * mb, np.uint8)
+            for i in range(size):
+                slots[i * mb:(i + 1) * mb] = oracle_cpu.tbq_encode(rng.normal(0, 2e-3, n).astype(np.float32), np.zeros(n, np.float32), thr)
+            Cc = _host_buf(size * mb, k & 1); Cc.numpy()[:] = slots
+            checks.append((kind, f"t{k}", g, r, dg, dr, Cc, slots))
+        keep.append(B)
+    torch.cuda.synchronize()
+    for (kind, name, g, r, dg, dr, Cc, extra), B in zip(checks, keep):
+        assert hp.submit_task(name, dg, dr, B, Cc, 1, kind)
+    for kind in (10, 20, 30):
+        _collect(hp, kind, [c[1] for c in checks if c[0] == kind])
+    for kind, name, g, r, dg, dr, Cc, extra in checks:
+        n = g.size
+        mb = oracle_cpu.tbq_packed_size(n)
+        if kind == 10:
+            rr = r.copy()
+            msg = oracle_cpu.tbq_encode(g, rr, thr)
+            assert_bits_equal(Cc.numpy(), msg, f"{name} COMP message"); assert_bits_equal(host(dr), rr, f"{name} residual")
+            assert_bits_equal(host(dg), g, f"{name} gradient untouched")
+        elif kind == 20:
+            want = oracle_cpu.tbq_decode(extra, n, thr, g.copy(), 1)
+            assert_bits_equal(host(dg), want, f"{name} DECOMP add")
+        else:
+            want = g.copy()
+            for i in range(size):
+                if i != rank:
+                    want = oracle_cpu.tbq_decode(extra[i * mb:(i + 1) * mb], n, thr, want, 1)
+            rr = r.copy()
+            msg = oracle_cpu.tbq_encode(want, rr, thr)
+            assert_bits_equal(host(dg), want, f"{name} ROOT gradient"); assert_bits_equal(host(dr), rr, f"{name} ROOT residual")
+            assert_bits_equal(Cc.numpy()[:mb], msg, f"{name} ROOT message")
+    assert hp.error_count() == 0, hp.last_error()
+
+
+def test_graddrop_comp_and_decomp(hp, oracle_cpu):
+    rng = np.random.default_rng(3)
+    n, sr, dr_, seed = 300_007, 0.02, 0.97, 11
+    assert hp.init("graddrop", {"sample_rate": sr, "drop_ratio": dr_, "seed": seed}, 0, 0, 2)
+    fixed = 4 + int(2 * np.ceil(n * (1 - dr_))) * 4          # hp_cuda.cpp:230
+    g = rng.laplace(0, 1e-3, n).astype(np.float32)
+    r = rng.normal(0, 1e-4, n).astype(np.float32)
+    dg, dres = dev(g), dev(r)
+    B = torch.zeros(fixed, dtype=torch.uint8, device="cuda")
+    Cc = _host_buf(fixed, 0)
+    torch.cuda.synchronize()
+    assert hp.submit_task("fc.weight", dg, dres, B, Cc, 0, 10)
+    _collect(hp, 10, ["fc.weight"])
+    rr = r.copy()
+    msg, info = oracle_cpu.gd_encode(g, rr, sr, dr_, seed)
+    assert_bits_equal(Cc.numpy()[:msg.size], msg, "COMP message"); assert_bits_equal(host(dres), rr, "residual")
+    # DECOMP of that message, add mode
+    base = rng.normal(0, 1, n).astype(np.float32)
+    dt = dev(base)
+    Bd = torch.zeros(fixed, dtype=torch.uint8, device="cuda")
+    torch.cuda.synchronize()
+    assert hp.submit_task("fc.weight", dt, dres, Bd, Cc, 1, 20)
+    _collect(hp, 20, ["fc.weight"])
+    want = base.copy()
+    assert oracle_cpu.gd_decode(msg, want, 1) == 0
+    assert_bits_equal(host(dt), want, "DECOMP add")
+    assert hp.error_count() == 0, hp.last_error()
+
+
+def test_powersgd_tasks_equal_direct_calls(hp, pkg, capi):
+    rng = np.random.default_rng(4)
+    assert hp.init("powersgd", {"matrix_approximation_rank": 4}, 0, 0, 2)
+    shapes = [(256, 512), (300, 70), (64, 64)]
+    tasks, refs = [], []
+    for k, (n, m) in enumerate(shapes):
+        G = dev(rng.normal(0, 1e-2, n * m).astype(np.float32)); R = dev(rng.normal(0, 1e-3, n * m).astype(np.float32))
+        Q = dev(rng.normal(0, 1, (m, 4)).astype(np.float32)); M = torch.zeros(n, m, device="cuda"); P = torch.zeros(n, 4, device="cuda")
+        tasks.append((f"w{k}", G, R, M, P, Q))
+        refs.append(tuple(x.clone() for x in (G, R, M, P, Q)))
+    torch.cuda.synchronize()
+    for phase, tid, queue in ((1, 40, 40), (2, 50, 50), (3, 60, 60)):
+        for name, G, R, M, P, Q in tasks:
+            assert hp.submit_task(name, G, R, M, P, Q, tid)
+        _collect(hp, queue, [t[0] for t in tasks])
+        for G, R, M, P, Q in refs:
+            if phase == 1:
+                pkg.hp_cuda_powersgd_encode1([G], [R], [Q], [M], [P])
+            elif phase == 2:
+                pkg.hp_cuda_powersgd_encode2([P], [M], [Q])
+            else:
+                pkg.hp_cuda_powersgd_decode([P], [Q], [M], [R], [G])
+        torch.cuda.synchronize()
+        for (name, *ts), rs in zip(tasks, refs):
+            for a, b_, what in zip(ts, rs, "GRMPQ"):
+                assert_bits_equal(host(a), host(b_), f"{name} {what} after phase {phase}")
+    assert hp.error_count() == 0, hp.last_error()
+
+
+def test_argument_checks_and_restart(hp, capsys):
+    assert hp.init("tbq", {"threshold": 1e-3}, 0, 0, 2)
+    t = torch.zeros(16, device="cuda"); B = torch.zeros(4, dtype=torch.uint8, device="cuda"); Cc = torch.zeros(4, dtype=torch.uint8)
+    assert hp.submit_task("x", t, t.clone(), B, Cc, 2, 10) is False            # hp_cuda.cpp:947-950
+    assert "is_root should be 0 (~root) or 1 (root), find is_root is 2" in hp.last_error()
+    assert hp.submit_task("x", t, t.clone(), B, Cc, 0, 40) is False            # hp_cuda.cpp:951-954
+    assert "task_id should be 10 (comp) or 20 (decomp) or 30" in hp.last_error()
+    with pytest.raises(RuntimeError, match="CPU tensor"):
+        hp.submit_task("x", t, t.clone(), B, B, 0, 10)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        hp.submit_task("x", torch.zeros(4, 8, device="cuda").t(), t.clone(), B, Cc, 0, 10)
+    assert hp.end()
+    with pytest.raises(RuntimeError, match="not running"):                     # check_thread(), hp_cuda.cpp:892-900
+        hp.submit_task("x", t, t.clone(), B, Cc, 0, 10)
+    assert hp.init("tbq", {"threshold": 1e-3}, 0, 0, 2)                        # start again after end()
+    torch.cuda.synchronize()
+    assert hp.submit_task("y", t, t.clone(), B, Cc, 0, 10)
+    _collect(hp, 10, ["y"])

@@ -31,6 +31,30 @@ SYMBOLS = (
     "hpx_powersgd_decode",
 )
 
+# include/hpx_sched.h
+SCHED_SYMBOLS = (
+    "hpx_sched_init",
+    "hpx_sched_end",
+    "hpx_sched_submit",
+    "hpx_sched_get_results",
+    "hpx_sched_wait",
+    "hpx_sched_take_done",
+    "hpx_sched_error_count",
+    "hpx_sched_error",
+)
+
+
+class Task(C.Structure):
+    """hpx_task_t of include/hpx_sched.h."""
+    _fields_ = [("name", C.c_char_p), ("task_id", C.c_int32), ("is_root", C.c_int32),
+                ("tensor", C.c_void_p), ("tensor_numel", C.c_int64),
+                ("residual", C.c_void_p), ("residual_numel", C.c_int64),
+                ("B", C.c_void_p), ("B_bytes", C.c_int64),
+                ("C", C.c_void_p), ("C_bytes", C.c_int64),
+                ("M", C.c_void_p), ("P", C.c_void_p), ("Q", C.c_void_p),
+                ("n", C.c_int32), ("m", C.c_int32), ("r", C.c_int32)]
+
+
 _lib = None
 
 
@@ -69,7 +93,16 @@ def load():
     L.hpx_powersgd_encode1.argtypes = [i32, pp, p, pp, pp, pp, pp, p, p, p, p]
     L.hpx_powersgd_encode2.argtypes = [i32, pp, pp, pp, p, p, p, p]
     L.hpx_powersgd_decode.argtypes = [i32, pp, pp, pp, pp, pp, p, p, p, p, p]
-    for name in SYMBOLS:
+    L.hpx_sched_init.argtypes = [C.c_char_p, C.POINTER(C.c_char_p), C.POINTER(C.c_double), C.c_int, C.c_int, C.c_int, C.c_int]
+    L.hpx_sched_submit.argtypes = [C.POINTER(Task), C.POINTER(C.c_uint64)]
+    L.hpx_sched_get_results.argtypes = [C.c_int, C.c_char_p, C.c_int64]
+    L.hpx_sched_get_results.restype = C.c_int64
+    L.hpx_sched_wait.argtypes = [C.c_int, C.c_int]
+    L.hpx_sched_take_done.argtypes = [C.POINTER(C.c_uint64), C.c_int64]
+    L.hpx_sched_take_done.restype = C.c_int64
+    L.hpx_sched_error_count.restype = C.c_int64
+    L.hpx_sched_error.restype = C.c_char_p
+    for name in SYMBOLS + SCHED_SYMBOLS:
         getattr(L, name)  # AttributeError if the build lost an entry point
     _lib = L
     return L
