@@ -222,3 +222,62 @@ def test_argument_checks_and_restart(hp, capsys):
     torch.cuda.synchronize()
     assert hp.submit_task("y", t, t.clone(), B, Cc, 0, 10)
     _collect(hp, 10, ["y"])
+
+
+def test_graddrop_root_task(hp, oracle_cpu):
+    rng = np.random.default_rng(8)
+    n, sr, dr_, seed, size, rank = 120_001, 0.05, 0.98, 3, 3, 2
+    assert hp.init("graddrop", {"sample_rate": sr, "drop_ratio": dr_, "seed": seed}, 0, rank, size)
+    fixed = 4 + int(2 * np.ceil(n * (1 - dr_))) * 4
+    slots = np.zeros(size * fixed, np.uint8)
+    msgs = []
+    for i in range(size):
+        m, _ = oracle_cpu.gd_encode(rng.laplace(0, 1e-3, n).astype(np.float32), np.zeros(n, np.float32), sr, dr_, 50 + i)
+        slots[i * fixed:i * fixed + m.size] = m
+        msgs.append(m)
+    g = rng.laplace(0, 1e-3, n).astype(np.float32)
+    r = rng.normal(0, 1e-4, n).astype(np.float32)
+    dg, dres = dev(g), dev(r)
+    B = torch.zeros(fixed, dtype=torch.uint8, device="cuda")
+    Cc = _host_buf(size * fixed, 0); Cc.numpy()[:] = slots
+    torch.cuda.synchronize()
+    assert hp.submit_task("emb", dg, dres, B, Cc, 1, 30)
+    _collect(hp, 30, ["emb"])
+    want = g.copy()
+    for i in range(size):
+        if i != rank:
+            assert oracle_cpu.gd_decode(msgs[i], want, 1) == 0
+    rr = r.copy()
+    msg, info = oracle_cpu.gd_encode(want, rr, sr, dr_, seed)
+    assert_bits_equal(host(dg), want, "ROOT gradient"); assert_bits_equal(host(dres), rr, "ROOT residual")
+    assert_bits_equal(Cc.numpy()[:msg.size], msg, "ROOT message")
+    assert hp.error_count() == 0, hp.last_error()
+
+
+def test_submitters_on_several_threads(hp, oracle_cpu):
+    # tasks arrive from four host threads while the worker is busy; every name comes back once
+    import threading
+    rng = np.random.default_rng(9)
+    thr = 1e-3
+    assert hp.init("tbq", {"threshold": thr}, 0, 0, 2)
+    items = []
+    for k in range(64):
+        n = int(rng.integers(100, 200_000))
+        g = rng.normal(0, 1e-3, n).astype(np.float32)
+        items.append((f"p{k}", g, dev(g), torch.zeros(n, device="cuda"),
+                      torch.zeros(oracle_cpu.tbq_packed_size(n), dtype=torch.uint8, device="cuda"),
+                      _host_buf(oracle_cpu.tbq_packed_size(n), k & 1)))
+    torch.cuda.synchronize()
+
+    def feed(part):
+        for name, g, dg, dr, B, Cc in part:
+            assert hp.submit_task(name, dg, dr, B, Cc, 0, 10)
+    threads = [threading.Thread(target=feed, args=(items[i::4],)) for i in range(4)]
+    [t.start() for t in threads]
+    [t.join() for t in threads]
+    _collect(hp, 10, [it[0] for it in items])
+    for name, g, dg, dr, B, Cc in items:
+        rr = np.zeros(g.size, np.float32)
+        msg = oracle_cpu.tbq_encode(g, rr, thr)
+        assert_bits_equal(Cc.numpy(), msg, f"{name} message"); assert_bits_equal(host(dr), rr, f"{name} residual")
+    assert hp.error_count() == 0, hp.last_error()
