@@ -329,7 +329,26 @@ def extra(torch, np, capi, L, stream, gen):
         "algorithmic_bytes": 12.0 * n + 8 * k + 4, "frac_of_hbm_peak": round((12.0 * n + 8 * k + 4) / sec / 1e9 / HBM_PEAK_GBS, 4),
         "stream_kernel_frac_of_hbm_peak": round(12.0 * n / kt["gd_stream_kernel"] / 1e9 / HBM_PEAK_GBS, 4) if kt["gd_stream_kernel"] else None,
         "decode_add_ms": round(sec_dec * 1e3, 4), "kernel_us_per_launch": {k_: round(v * 1e6, 1) for k_, v in kt.items() if v}}
-    del g, r, r0, out, dout, scrub
+    # the same sparsifier without residual (dgc_body.h): reads the gradient once, 4 B/elt
+    del r, r0, dout
+    g0 = g.clone()
+    dgc = Call(L.hpx_dgc_encode, 1, capi.ptr_array([g.data_ptr()]), capi.i32_array([n]), capi.ptr_array([out.data_ptr()]),
+               capi.f64_array([0.01]), capi.f64_array([0.001]), capi.u64_array([3 << 24]), stream)
+    times = []
+    for it in range(7):
+        g.copy_(g0)
+        scrub.sum()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        dgc()
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+    sec_nr = float(np.median(times[2:]))
+    res["dgc_without_residual_138M"] = {
+        "encode_ms": round(sec_nr * 1e3, 4), "algorithmic_bytes": 4.0 * n,
+        "frac_of_hbm_peak": round(4.0 * n / sec_nr / 1e9 / HBM_PEAK_GBS, 4),
+        "selected": (int(out[:4].cpu().numpy().view(np.int32)[0]) - 4) // 8}
+    del g, g0, out, scrub
     torch.cuda.empty_cache()
 
     # ---- PowerSGD rank 4 over the 36-matrix layer set ------------------------------------------

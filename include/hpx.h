@@ -179,6 +179,25 @@ int hpx_gd_decode(int count, const uint8_t* const* ins, const int32_t* in_sizes,
                   float* const* outs, const int32_t* out_sizes,
                   const int32_t* is_add_tos, hpx_stream_t stream);
 
+/* ---- DGC without residual --------------------------------------------------
+ * The reference holds this sparsifier as a body without a driver
+ * (dgc_with_auxiliary_body / dgc_body, dgc_body.h:71-152 / :155-226; dgc_r_body
+ * :252-293); these two entry points are the drivers it would have.
+ * Encode is hpx_gd_encode with the gradient in the place of the residual:
+ * nothing is added, the threshold is the int(sample_cnt*s_percent)-th largest of
+ * sample_cnt = ceil(N*sample_rate) sampled |G|, entries beyond it (at most
+ * ceil(N*s_percent), the largest first if there are more) go into the message
+ * and are CLEARED IN grads[t].  Same message layout, same output size
+ * 4 + 8*ceil(N*s_percent), same one wait on the stream.
+ * Decode differs from hpx_gd_decode in write mode only: the output is not
+ * cleared first (dgc_body.h:283-289). */
+int hpx_dgc_encode(int count, float* const* grads, const int32_t* Ns, uint8_t* const* outs,
+                   const double* sample_rates, const double* s_percents,
+                   const uint64_t* seeds, hpx_stream_t stream);
+int hpx_dgc_decode(int count, const uint8_t* const* ins, const int32_t* in_sizes,
+                   float* const* outs, const int32_t* out_sizes,
+                   const int32_t* is_add_tos, hpx_stream_t stream);
+
 /* ---- PowerSGD: rank-r factorisation with error feedback ------------------- */
 /* The reference bodies operate on torch tensors (powersgd_body.h); here every
  * matrix is a row-major fp32 device array: M is n x m, Q is m x r, P is n x r,

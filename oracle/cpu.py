@@ -46,6 +46,8 @@ def lib():
         L.orc_gd_sample_index.argtypes = [C.c_uint64, C.c_int32, C.c_int32]
         L.orc_gd_encode.argtypes = [f32p, C.c_int32, f32p, u8p, C.c_double, C.c_double, C.c_uint64, i32p]
         L.orc_gd_decode.argtypes = [u8p, C.c_int32, f32p, C.c_int32, C.c_int]
+        L.orc_dgc_encode.argtypes = [f32p, C.c_int32, u8p, C.c_double, C.c_double, C.c_uint64, i32p]
+        L.orc_dgc_decode.argtypes = [u8p, C.c_int32, f32p, C.c_int]
         L.orc_max_threads.restype = C.c_int
         L.orc_set_threads.argtypes = [C.c_int]
         L.orc_set_threads.restype = None
@@ -167,3 +169,20 @@ def gd_split(msg):
 def gd_decode(msg, out, is_add_to=0, in_size=None):
     rc = lib().orc_gd_decode(_u8(msg), msg.size if in_size is None else in_size, _f32(out), out.size, int(is_add_to))
     return rc
+
+
+# ---- DGC without residual (dgc_body.h) ---------------------------------------
+def dgc_encode(g, sample_rate, s_percent, seed=0):
+    """Returns (message bytes trimmed to 4+8k, info dict). `g` is updated in place (selected entries -> 0)."""
+    n = g.size
+    out = np.zeros(4 + 8 * n, np.uint8)
+    info = (C.c_int32 * 3)()
+    rc = lib().orc_dgc_encode(_f32(g), n, _u8(out), sample_rate, s_percent, seed, info)
+    assert rc == 0
+    m = int(out[:4].view(np.int32)[0])
+    thr = np.array([info[2]], np.int32).view(np.float32)[0]
+    return out[:m].copy(), {"candidates": info[0], "kept": info[1], "threshold": thr}
+
+
+def dgc_decode(msg, out, is_add_to=0, in_size=None):
+    return lib().orc_dgc_decode(_u8(msg), msg.size if in_size is None else in_size, _f32(out), int(is_add_to))

@@ -364,14 +364,12 @@ ORC_API uint32_t orc_gd_sample_index(uint64_t seed, int32_t x, int32_t n) {
  * ties is unspecified).  info[0]=candidates before truncation, info[1]=kept,
  * info[2]=threshold bits.  Scratch is private: unlike the reference nothing
  * beyond the 4+8k message bytes of `out` is touched. */
-ORC_API int orc_gd_encode(const float *g, int32_t n, float *r, uint8_t *out,
-                          double sample_rate, double drop_ratio, uint64_t seed,
-                          int32_t *info) {
-    int32_t sample_cnt, expected, thr_index;
-    orc_gd_sizes(n, sample_rate, drop_ratio, &sample_cnt, &expected, &thr_index);
-#pragma omp parallel for schedule(static)
-    for (int32_t i = 0; i < n; i++) r[i] = g[i] + r[i];
-
+/* Everything of gd_body after R += G (gd_body.h:130-229), which is also all of
+ * dgc_with_auxiliary_body / dgc_body (dgc_body.h:71-152, :155-226) with G in the
+ * place of R. */
+static int select_and_pack(float *r, int32_t n, uint8_t *out, int32_t sample_cnt,
+                           int32_t expected, int32_t thr_index, uint64_t seed,
+                           int32_t *info) {
     float *sample = (float *)malloc(sizeof(float) * (size_t)(sample_cnt > 0 ? sample_cnt : 1) * 2);
 #pragma omp parallel for schedule(static)
     for (int32_t x = 0; x < sample_cnt; x++)
@@ -438,6 +436,51 @@ ORC_API int orc_gd_encode(const float *g, int32_t n, float *r, uint8_t *out,
         r[ix] = 0;
     }
     free(cand);
+    return 0;
+}
+
+ORC_API int orc_gd_encode(const float *g, int32_t n, float *r, uint8_t *out,
+                          double sample_rate, double drop_ratio, uint64_t seed,
+                          int32_t *info) {
+    int32_t sample_cnt, expected, thr_index;
+    orc_gd_sizes(n, sample_rate, drop_ratio, &sample_cnt, &expected, &thr_index);
+#pragma omp parallel for schedule(static)
+    for (int32_t i = 0; i < n; i++) r[i] = g[i] + r[i];
+    return select_and_pack(r, n, out, sample_cnt, expected, thr_index, seed, info);
+}
+
+/* dgc_with_auxiliary_body, dgc_body.h:71-152 (and dgc_body, :155-226, which only
+ * keeps its scratch elsewhere) for ONE tensor: the sparsifier without residual.
+ *   :79-80    sample_cnt = ceil(N*sample_rate), expected = ceil(N*s_percent)
+ *   :84-95    sample[x] = |G[idx_x]|, same index stream as GradDrop (:18-30)
+ *   :98-104   sort descending, threshold = sample[int(sample_cnt*s_percent)]
+ *   :110-117  candidates {i : G[i] > thr || G[i] < -thr}, ascending
+ *   :121-126  if more than `expected`: order by |G| descending, keep `expected`
+ *   :135-150  header int32 4+8k, index block, value block, G[idx] = 0
+ * The caller's gradient is modified: selected entries become 0.  `seed`
+ * replaces the wall-clock value of :92-95; ties as in orc_gd_encode. */
+ORC_API int orc_dgc_encode(float *g, int32_t n, uint8_t *out, double sample_rate,
+                           double s_percent, uint64_t seed, int32_t *info) {
+    int32_t sample_cnt = (int32_t)ceil(n * sample_rate);
+    int32_t expected = (int32_t)ceil(n * s_percent);
+    int32_t thr_index = (int32_t)(sample_cnt * s_percent);
+    return select_and_pack(g, n, out, sample_cnt, expected, thr_index, seed, info);
+}
+
+/* dgc_r_body, dgc_body.h:252-293 for ONE message: as gd_r_body except that write
+ * mode does NOT clear the output first (:283-289 just stores G[idx] = val). */
+ORC_API int orc_dgc_decode(const uint8_t *in, int32_t in_size, float *out, int is_add_to) {
+    int32_t M;
+    memcpy(&M, in, 4);
+    int32_t k = (M - 4) / 8;
+    if (in_size < M) return -1;
+    const int32_t *idx = (const int32_t *)(in + 4);
+    const float *val = (const float *)(in + 4 + 4 * (size_t)k);
+    if (is_add_to) {
+        for (int32_t x = 0; x < k; x++) out[idx[x]] += val[x];
+    } else {
+        for (int32_t x = 0; x < k; x++) out[idx[x]] = val[x];
+    }
     return 0;
 }
 

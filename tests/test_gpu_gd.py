@@ -225,3 +225,48 @@ def test_full_size_config3(gd):
     decoded = host(dec)
     rh2 = rh.copy(); rh2[idx] += val
     assert_bits_equal(decoded, rh2, "decode(add) restores the accumulated tensor")
+
+
+# ---- the sparsifier without residual (dgc_body.h) ---------------------------------------------------
+def _dgc_encode(gd, dg, out, sr, sp, seed, expect_rc=0):
+    c = gd.c
+    rc = gd.L.hpx_dgc_encode(1, c.ptr_array([dg.data_ptr()]), c.i32_array([dg.numel()]), c.ptr_array([out.data_ptr()]),
+                             c.f64_array([sr]), c.f64_array([sp]), c.u64_array([seed]), stream_ptr())
+    assert rc == expect_rc, (rc, c.last_error())
+
+
+@pytest.mark.parametrize("n,sr,sp", [(1000, 0.05, 0.01), (4097, 0.1, 0.1), (65536, 0.5, 0.5), (100003, 0.01, 0.001),
+                                     (1_000_003, 0.01, 0.001), (5_000_011, 0.01, 0.001)])
+def test_dgc_without_residual(gd, oracle_cpu, n, sr, sp):
+    rng = np.random.default_rng(n + 1)
+    branches = set()
+    for seed in (0, 1 << 22, 12345 << 20, 2**64 - 2):
+        g = rng.laplace(0, 1e-3, n).astype(np.float32)
+        dg = dev(g)
+        size = 4 + 8 * int(np.ceil(n * sp))
+        out = torch.full((size + 64,), 0xEE, dtype=torch.uint8, device="cuda")
+        _dgc_encode(gd, dg, out, sr, sp, seed)
+        torch.cuda.synchronize()
+        g_ref = g.copy()
+        msg, info = oracle_cpu.dgc_encode(g_ref, sr, sp, seed)
+        got = host(out)
+        m = int(got[:4].view(np.int32)[0])
+        assert m == msg.size, (m, msg.size, info)
+        assert_bits_equal(got[:m], msg, f"message n={n} seed={seed} info={info}")
+        assert np.all(got[size:] == 0xEE), "wrote past 4 + 8*expected bytes"
+        assert_bits_equal(host(dg), g_ref, "gradient after encode (selected entries cleared)")
+        branches.add(info["candidates"] > info["kept"])
+        # decode: write mode leaves the other entries alone (dgc_body.h:283-289), add mode accumulates
+        for add in (0, 1):
+            base = rng.normal(0, 1, n).astype(np.float32)
+            dout = dev(base)
+            c = gd.c
+            rc = gd.L.hpx_dgc_decode(1, c.ptr_array([out.data_ptr()]), c.i32_array([msg.size]), c.ptr_array([dout.data_ptr()]),
+                                     c.i32_array([n]), c.i32_array([add]), stream_ptr())
+            assert rc == 0, c.last_error()
+            torch.cuda.synchronize()
+            ref = base.copy()
+            assert oracle_cpu.dgc_decode(msg, ref, add) == 0
+            assert_bits_equal(host(dout), ref, f"decode add={add}")
+    if n >= 100003:
+        assert True in branches or False in branches

@@ -146,3 +146,76 @@ def test_gd_decode_against_reference(oracle_cpu, oracle_ref):
             assert oracle_cpu.gd_decode(m, a, add) == 0 and oracle_ref.gd_decode(m, b, add) == 0
             assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
         assert oracle_ref.gd_decode(m, b, 0, in_size=m.size - 1) == -1
+
+
+# ---- the sparsifier without residual (dgc_body.h) ------------------------------------------------
+def _brute_force_dgc(g0, sample_rate, s_percent, seed):
+    """Independent numpy statement of dgc_body.h:71-152."""
+    n = g0.size
+    sample_cnt = int(np.ceil(n * sample_rate))
+    expected = int(np.ceil(n * s_percent))
+    g = g0.copy()
+    x = (seed + np.arange(sample_cnt, dtype=np.uint64)) & np.uint64(0xFFFFFFFF)
+    idx = ((x * np.uint64(A2) + np.uint64(C2)) & np.uint64(0xFFFFFFFF)) % np.uint64(n)
+    sample = np.sort(np.abs(g[idx.astype(np.int64)]))[::-1]
+    thr = sample[int(sample_cnt * s_percent)]
+    cand = np.flatnonzero((g > thr) | (g < -thr))
+    total = cand.size
+    if total > expected:
+        order = np.lexsort((cand, -np.abs(g[cand]).astype(np.float64)))
+        cand = cand[order][:expected]
+    vals = g[cand].copy()
+    g[cand] = 0
+    return cand.astype(np.int32), vals, g, thr, total
+
+
+@pytest.mark.parametrize("n,sr,sp", [(1000, 0.05, 0.01), (4096, 0.01, 0.001), (10007, 0.1, 0.1), (100003, 0.01, 0.001),
+                                     (65536, 0.5, 0.5), (300007, 0.02, 0.03)])
+def test_dgc_encode_matches_brute_force(oracle_cpu, n, sr, sp):
+    rng = np.random.default_rng(n + 7)
+    cuts = set()
+    for seed in (0, 1, 12345, 2**40 + 5, 2**64 - 2):
+        g0 = rng.laplace(0, 1e-3, n).astype(np.float32)
+        g = g0.copy()
+        msg, info = oracle_cpu.dgc_encode(g, sr, sp, seed)
+        idx, val, g_ref, thr, total = _brute_force_dgc(g0, sr, sp, seed)
+        assert info["candidates"] == total and info["threshold"] == thr
+        oi, ov = oracle_cpu.gd_split(msg)
+        assert msg[:4].view(np.int32)[0] == 4 + 8 * idx.size == msg.size
+        assert np.array_equal(oi, idx) and np.array_equal(ov.view(np.uint32), val.view(np.uint32))
+        assert np.array_equal(g.view(np.uint32), g_ref.view(np.uint32))
+        cuts.add(total > idx.size)
+
+
+def test_dgc_equals_graddrop_with_zero_residual(oracle_cpu):
+    # R = 0 + G is G itself (except that -0.0 becomes +0.0), so GradDrop with a zero residual and
+    # s = 1 - drop_ratio must produce the same message and leave R as DGC leaves G.
+    rng = np.random.default_rng(5)
+    for n, sr, dr in ((50_000, 0.02, 0.99), (200_001, 0.01, 0.999), (8192, 0.3, 0.75)):
+        g0 = rng.laplace(0, 1e-3, n).astype(np.float32)
+        g0[g0 == 0] = 1e-9
+        for seed in (3, 2**33 + 1):
+            r = np.zeros(n, np.float32)
+            m_gd, i_gd = oracle_cpu.gd_encode(g0, r, sr, dr, seed)
+            g = g0.copy()
+            m_dgc, i_dgc = oracle_cpu.dgc_encode(g, sr, 1 - dr, seed)
+            assert np.array_equal(m_gd, m_dgc) and i_gd == i_dgc
+            assert np.array_equal(r.view(np.uint32), g.view(np.uint32))
+
+
+def test_dgc_decode_write_mode_keeps_other_entries(oracle_cpu):
+    rng = np.random.default_rng(6)
+    n = 10_000
+    g = rng.laplace(0, 1e-3, n).astype(np.float32)
+    msg, info = oracle_cpu.dgc_encode(g.copy(), 0.05, 0.01, 9)
+    idx, val = oracle_cpu.gd_split(msg)
+    base = rng.normal(0, 1, n).astype(np.float32)
+    out = base.copy()
+    assert oracle_cpu.dgc_decode(msg, out, 0) == 0                 # dgc_body.h:283-289: no zero fill
+    want = base.copy(); want[idx] = val
+    assert np.array_equal(out.view(np.uint32), want.view(np.uint32))
+    out = base.copy()
+    assert oracle_cpu.dgc_decode(msg, out, 1) == 0
+    want = base.copy(); want[idx] += val
+    assert np.array_equal(out.view(np.uint32), want.view(np.uint32))
+    assert oracle_cpu.dgc_decode(msg, out, 0, in_size=msg.size - 1) == -1   # dgc_body.h:268-274

@@ -26,6 +26,8 @@ SYMBOLS = (
     "hpx_terngrad_decode_status",
     "hpx_gd_encode",
     "hpx_gd_decode",
+    "hpx_dgc_encode",
+    "hpx_dgc_decode",
     "hpx_powersgd_encode1",
     "hpx_powersgd_encode2",
     "hpx_powersgd_decode",
@@ -90,6 +92,8 @@ def load():
     L.hpx_terngrad_decode_status.argtypes = [p]
     L.hpx_gd_encode.argtypes = [i32, pp, p, pp, pp, p, p, p, p]
     L.hpx_gd_decode.argtypes = [i32, pp, p, pp, p, p, p]
+    L.hpx_dgc_encode.argtypes = [i32, pp, p, pp, p, p, p, p]
+    L.hpx_dgc_decode.argtypes = [i32, pp, p, pp, p, p, p]
     L.hpx_powersgd_encode1.argtypes = [i32, pp, p, pp, pp, pp, pp, p, p, p, p]
     L.hpx_powersgd_encode2.argtypes = [i32, pp, pp, pp, p, p, p, p]
     L.hpx_powersgd_decode.argtypes = [i32, pp, pp, pp, pp, pp, p, p, p, p, p]

@@ -119,7 +119,8 @@ __global__ __launch_bounds__(kThreads) void gd_sample_kernel(const SelArgs a) {
   }
   if (x < a.sample_cnt) {
     const uint32_t i = sample_index(a.seed, x, a.n);
-    a.samples[x] = __float_as_uint(__builtin_fabsf(a.g[i] + a.r[i]));
+    // with a residual: |G[i] + R[i]|, the value the update is about to store; without (dgc_body.h:18-30): |G[i]|
+    a.samples[x] = __float_as_uint(__builtin_fabsf(a.r ? a.g[i] + a.r[i] : a.g[i]));
   }
 }
 
@@ -177,6 +178,9 @@ __global__ __launch_bounds__(kSelThreads) void gd_threshold_kernel(const SelArgs
 // The one pass over the tensor.  Lane l of wave w handles elements
 // base + w*1024 + c*64 + l for c = 0..15, so ballot number c is the mask word of
 // 64 consecutive elements in natural bit order.
+// RESIDUAL = false is the sparsifier without residual (dgc_body.h:110-117): the
+// values are G itself, nothing is added and nothing is stored (4 bytes per element).
+template <bool RESIDUAL>
 __global__ __launch_bounds__(kThreads) void gd_stream_kernel(const float* __restrict__ g, float* __restrict__ r,
                                                              uint32_t n, const GdState* __restrict__ st,
                                                              uint64_t* __restrict__ masks,
@@ -193,12 +197,12 @@ __global__ __launch_bounds__(kThreads) void gd_stream_kernel(const float* __rest
 #pragma unroll
     for (int c = 0; c < kPerLane; c++) {
       gv[c] = __builtin_nontemporal_load(g + size_t(wbase) + c * kWave + lane);
-      rv[c] = __builtin_nontemporal_load(r + size_t(wbase) + c * kWave + lane);
+      rv[c] = RESIDUAL ? __builtin_nontemporal_load(r + size_t(wbase) + c * kWave + lane) : 0.0f;
     }
 #pragma unroll
     for (int c = 0; c < kPerLane; c++) {
-      const float x = gv[c] + rv[c];  // thrust::plus<float>()(G, R), gd_body.h:121-128
-      __builtin_nontemporal_store(x, r + size_t(wbase) + c * kWave + lane);
+      const float x = RESIDUAL ? gv[c] + rv[c] : gv[c];  // thrust::plus<float>()(G, R), gd_body.h:121-128
+      if (RESIDUAL) __builtin_nontemporal_store(x, r + size_t(wbase) + c * kWave + lane);
       const uint64_t m = __ballot((x > thr) || (x < nthr));  // gd_body.h:59-67
       cnt += __popcll(m);
       lo = lane == uint32_t(c) ? uint32_t(m) : lo;  // lane c keeps mask word c
@@ -210,8 +214,8 @@ __global__ __launch_bounds__(kThreads) void gd_stream_kernel(const float* __rest
       const uint32_t e = wbase + c * kWave + lane;
       bool p = false;
       if (e < n) {
-        const float x = g[e] + r[e];
-        r[e] = x;
+        const float x = RESIDUAL ? g[e] + r[e] : g[e];
+        if (RESIDUAL) r[e] = x;
         p = (x > thr) || (x < nthr);
       }
       const uint64_t m = __ballot(p);
@@ -627,16 +631,19 @@ int sort_and_cut(uint32_t* keys_a, int32_t* idx_a, uint32_t* keys_b, int32_t* id
   return HPX_OK;
 }
 
-int gd_encode_one(const float* g, int32_t N, float* r, uint8_t* out, double sample_rate, double drop_ratio,
+// One tensor.  With a residual (`residual` non-null): gd_body, s_percent = 1 - drop_ratio.  Without:
+// dgc_with_auxiliary_body, where `grad` itself is thresholded and its selected entries cleared.
+int gd_encode_one(float* grad, int32_t N, float* residual, uint8_t* out, double sample_rate, double s_percent,
                   uint64_t seed, hpx::Workspace* ws, hipStream_t st) {
-  // size arithmetic of gd_body.h:112-115, :153
-  const double s_percent = 1 - drop_ratio;
+  // size arithmetic of gd_body.h:112-115, :153 (dgc_body.h:79-80, :103)
   const int32_t sample_cnt = static_cast<int32_t>(std::ceil(N * sample_rate));
   const int32_t expected = static_cast<int32_t>(std::ceil(N * s_percent));
   const int32_t thr_index = static_cast<int32_t>(sample_cnt * s_percent);
   HPX_ARG(sample_cnt > 0 && thr_index >= 0 && thr_index < sample_cnt && expected >= 0,
-          "hpx_gd_encode: N=%d sample_rate=%g drop_ratio=%g give sample_cnt=%d threshold index=%d", N, sample_rate,
-          drop_ratio, sample_cnt, thr_index);
+          "sparsifier encode: N=%d sample_rate=%g kept fraction=%g give sample_cnt=%d threshold index=%d", N, sample_rate,
+          s_percent, sample_cnt, thr_index);
+  const float* g = grad;
+  float* r = residual ? residual : grad;  // the array whose selected entries are read out and cleared
 
   const uint32_t n = static_cast<uint32_t>(N);
   const uint32_t ntiles = cdiv(n, kTile);
@@ -681,7 +688,7 @@ int gd_encode_one(const float* g, int32_t N, float* r, uint8_t* out, double samp
   uint32_t* chunk_off = reinterpret_cast<uint32_t*>(base + o_coff);
   const uint32_t nchunks = cdiv(ntiles, kScanChunk);
 
-  SelArgs sa{g, r, n, static_cast<uint32_t>(sample_cnt), static_cast<uint32_t>(seed), static_cast<uint32_t>(thr_index),
+  SelArgs sa{g, residual, n, static_cast<uint32_t>(sample_cnt), static_cast<uint32_t>(seed), static_cast<uint32_t>(thr_index),
              samples, hist, state};
   uint32_t sel_blocks = cdiv(sample_cnt, kSelThreads * 8);
   if (sel_blocks > kSelBlocksMax) sel_blocks = kSelBlocksMax;
@@ -692,7 +699,10 @@ int gd_encode_one(const float* g, int32_t N, float* r, uint8_t* out, double samp
   HPX_LAUNCH("gd_select_kernel", gd_select_kernel<2>, dim3(sel_blocks), dim3(kSelThreads), st, sa);
   HPX_LAUNCH("gd_select_kernel", gd_select_kernel<3>, dim3(sel_blocks), dim3(kSelThreads), st, sa);
   HPX_LAUNCH("gd_threshold_kernel", gd_threshold_kernel, dim3(1), dim3(kSelThreads), st, sa);
-  HPX_LAUNCH("gd_stream_kernel", gd_stream_kernel, dim3(ntiles), dim3(kThreads), st, g, r, n, state, masks, blk_cnt);
+  if (residual)
+    HPX_LAUNCH("gd_stream_kernel", gd_stream_kernel<true>, dim3(ntiles), dim3(kThreads), st, g, r, n, state, masks, blk_cnt);
+  else
+    HPX_LAUNCH("gd_stream_kernel", gd_stream_kernel<false>, dim3(ntiles), dim3(kThreads), st, g, r, n, state, masks, blk_cnt);
   uint32_t* h_total = reinterpret_cast<uint32_t*>(ws->pinned);
   HPX_LAUNCH("gd_scan_kernel", gd_scan_kernel, dim3(nchunks), dim3(kSelThreads), st, blk_cnt, blk_off, ntiles, chunk_tot,
              chunk_off, state, h_total);
@@ -763,14 +773,18 @@ HPX_API int hpx_gd_encode(int count, const float* const* grads, const int32_t* N
   int worst = HPX_OK;
   for (int i = 0; i < count; i++) {
     const uint64_t seed = seeds ? seeds[i] : hpx::clock_seed();
-    const int rc = gd_encode_one(grads[i], Ns[i], residuals[i], outs[i], sample_rates[i], drop_ratios[i], seed, ws, st);
+    const int rc = gd_encode_one(const_cast<float*>(grads[i]), Ns[i], residuals[i], outs[i], sample_rates[i],
+                                 1 - drop_ratios[i], seed, ws, st);
     if (rc != HPX_OK && worst == HPX_OK) worst = rc;  // like the reference driver: report, go on
   }
   return worst;
 }
 
-HPX_API int hpx_gd_decode(int count, const uint8_t* const* ins, const int32_t* in_sizes, float* const* outs,
-                          const int32_t* out_sizes, const int32_t* is_add_tos, hpx_stream_t stream) {
+namespace {
+// gd_r_body (zero_fill: write mode clears the whole output first, gd_body.h:335-347)
+// and dgc_r_body (no clearing, dgc_body.h:283-289).
+int decode_messages(int count, const uint8_t* const* ins, const int32_t* in_sizes, float* const* outs,
+                    const int32_t* out_sizes, const int32_t* is_add_tos, bool zero_fill, hpx_stream_t stream) {
   hpx::clear_error();
   HPX_ARG(count >= 0, "hpx_gd_decode: negative count");
   if (count == 0) return HPX_OK;
@@ -805,7 +819,7 @@ HPX_API int hpx_gd_decode(int count, const uint8_t* const* ins, const int32_t* i
     const float* val = reinterpret_cast<const float*>(ins[i] + 4 + size_t(k) * 4);
     if (!is_add_tos[i]) {
       const uint32_t n = static_cast<uint32_t>(out_sizes[i]);
-      if (n) {
+      if (n && zero_fill) {
         uint32_t blocks = cdiv(n, kThreads * 4);
         HPX_LAUNCH("gd_zero_kernel", gd_zero_kernel, dim3(blocks), dim3(kThreads), st, outs[i], n);
       }
@@ -817,3 +831,40 @@ HPX_API int hpx_gd_decode(int count, const uint8_t* const* ins, const int32_t* i
   }
   return HPX_OK;
 }
+}  // namespace
+
+HPX_API int hpx_gd_decode(int count, const uint8_t* const* ins, const int32_t* in_sizes, float* const* outs,
+                          const int32_t* out_sizes, const int32_t* is_add_tos, hpx_stream_t stream) {
+  return decode_messages(count, ins, in_sizes, outs, out_sizes, is_add_tos, true, stream);
+}
+
+HPX_API int hpx_dgc_decode(int count, const uint8_t* const* ins, const int32_t* in_sizes, float* const* outs,
+                           const int32_t* out_sizes, const int32_t* is_add_tos, hpx_stream_t stream) {
+  return decode_messages(count, ins, in_sizes, outs, out_sizes, is_add_tos, false, stream);
+}
+
+HPX_API int hpx_dgc_encode(int count, float* const* grads, const int32_t* Ns, uint8_t* const* outs,
+                           const double* sample_rates, const double* s_percents, const uint64_t* seeds,
+                           hpx_stream_t stream) {
+  hpx::clear_error();
+  HPX_ARG(count >= 0, "hpx_dgc_encode: negative count");
+  if (count == 0) return HPX_OK;
+  HPX_ARG(grads && Ns && outs && sample_rates && s_percents, "hpx_dgc_encode: null argument array");
+  for (int i = 0; i < count; i++) {
+    HPX_ARG(Ns[i] > 0, "hpx_dgc_encode: tensor %d has size %d (must be positive)", i, Ns[i]);
+    HPX_ARG(grads[i] && outs[i], "hpx_dgc_encode: tensor %d has a null pointer", i);
+    HPX_ARG((reinterpret_cast<uintptr_t>(outs[i]) & 3) == 0, "hpx_dgc_encode: output %d is not 4-byte aligned", i);
+  }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  hpx::Workspace* ws = hpx::workspace_record(st);
+  if (!ws) return HPX_ERR_HIP;
+  std::lock_guard<std::mutex> lock(ws->mu);
+  int worst = HPX_OK;
+  for (int i = 0; i < count; i++) {
+    const uint64_t seed = seeds ? seeds[i] : hpx::clock_seed();
+    const int rc = gd_encode_one(grads[i], Ns[i], nullptr, outs[i], sample_rates[i], s_percents[i], seed, ws, st);
+    if (rc != HPX_OK && worst == HPX_OK) worst = rc;
+  }
+  return worst;
+}
+
