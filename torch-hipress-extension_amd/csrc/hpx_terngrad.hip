@@ -414,12 +414,16 @@ __global__ __launch_bounds__(kThreads) void terngrad_quant_kernel(const EncArgs<
 constexpr int kResThreads = 1024;
 constexpr int kResRegGroups = 24;  // float4 per lane held in registers ...
 // ... except at 1 bit with stochastic rounding, whose eight draws per lane need the room.
+// Rows of prepared random addends when the LDS has room for them (8 float4 per lane).
+constexpr int res_pre_rows(int bits) { return bits == 1 ? 4 : 8; }
 constexpr int res_reg_groups(int bits, bool random) { return (bits == 1 && random) ? 14 : kResRegGroups; }
-constexpr int kResLdsGroups = 8;   // float4 per lane held in LDS (128 KiB per workgroup)
+constexpr int kResLdsGroups = 8;   // float4 per lane of the tensor held in LDS (128 KiB per workgroup)
+constexpr int kResLdsTotalGroups = 9;  // ... and what the workgroup may use altogether (144 KiB): the rest holds prepared draws
 struct ResArgs {
   EncSeg seg;
   uint32_t chunk_units;  // units per workgroup, a multiple of kResThreads
   uint32_t lds_rows;     // rows of kResThreads units kept in LDS
+  uint32_t pre_rows;     // register rows whose random addends are prepared during pass 1: 0 or res_pre_rows(bits)
   uint32_t gen;          // generation of this launch, counted from 1: the tag of its records
   uint64_t* bar;         // exchange memory (kBarTotalWords); only ever holds (gen << 32 | key) words
   uint32_t* host_flag;   // pinned host word, set to 1 when the barrier wait expires
@@ -436,7 +440,30 @@ __device__ __forceinline__ void acc_zero4(float4 v, uint32_t idx, float& mn, flo
   acc_zero(v.z, idx + 2, mn, mx, fz); acc_zero(v.w, idx + 3, mn, mx, fz);
 }
 
-template <int B, bool RANDOM>
+// quant_unit for a unit whose random addends (2^32 * u per element) were prepared earlier.
+template <int B, int UNIT = (8 / B > 4 ? 8 / B : 4)>
+__device__ __forceinline__ uint32_t quant_unit_prepared(const float4 (&v)[UNIT / 4], const float4 (&s)[UNIT / 4], float mn,
+                                                        float gi) {
+  constexpr int DPB = 8 / B;
+  uint32_t packed = 0;
+#pragma unroll
+  for (int q = 0; q < UNIT; q++) {
+    const float4 f = v[q / 4], g = s[q / 4];
+    const float x = (q & 3) == 0 ? f.x : (q & 3) == 1 ? f.y : (q & 3) == 2 ? f.z : f.w;
+    const float sc = (q & 3) == 0 ? g.x : (q & 3) == 1 ? g.y : (q & 3) == 2 ? g.z : g.w;
+    float th = (x - mn) * gi;
+    th = __builtin_fmaf(sc, 0x1p-32f, th);
+    const uint32_t t = static_cast<uint32_t>(static_cast<int32_t>(th)) & 0xFFu;
+    const int jb = q / DPB, j = q % DPB;
+    packed |= ((t << (B * j)) & 0xFFu) << (8 * jb);
+  }
+  return packed;
+}
+
+// PRE: register rows whose random addends are prepared during pass 1 (a compile-time count, so that pass 2
+// stays one straight block the scheduler can interleave across rows; a per-row branch cost as much as the
+// prepared rows saved).
+template <int B, bool RANDOM, int PRE>
 __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const ResArgs a) {
   constexpr int DPB = 8 / B;
   constexpr int UNIT = DPB > 4 ? DPB : 4;
@@ -478,6 +505,28 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
 #pragma unroll
       for (int h = 0; h < H; h++)
         v[k][h] = u < wg_end ? ld4_stream(xp + size_t(u) * UNIT + h * 4) : make_float4(qnan, qnan, qnan, qnan);
+    }
+  }
+  // While the loads are in flight and the ALUs idle: the random addends of the first pre_rows
+  // register rows, which depend on position and seed only, go into the LDS the tensor does not
+  // need; pass 2 (ALU-bound: nothing left to overlap with) then skips 6 of its 11 operations
+  // per element for those rows.
+  float4* s_pre = s_rows + size_t(a.lds_rows) * H * kResThreads;
+  if (RANDOM && PRE > 0) {
+    uint32_t d[UNIT];
+    const uint32_t x0 = a.seg.seed + u0 * BPU;
+#pragma unroll
+    for (int q = 0; q < UNIT; q++) {
+      const int jb = q / DPB, j = q % DPB;
+      d[q] = lcg_mul(j + 2) * (x0 + jb) + lcg_add(j + 2);
+    }
+    for (uint32_t k = 0; k < uint32_t(PRE); k++) {
+#pragma unroll
+      for (int h = 0; h < H; h++)
+        s_pre[(k * H + h) * kResThreads + threadIdx.x] =
+            make_float4(u01_scaled(d[4 * h]), u01_scaled(d[4 * h + 1]), u01_scaled(d[4 * h + 2]), u01_scaled(d[4 * h + 3]));
+#pragma unroll
+      for (int q = 0; q < UNIT; q++) d[q] += lcg_mul(q % DPB + 2) * stride_bytes;
     }
   }
   float mn = __builtin_inff(), mx = -__builtin_inff();
@@ -562,7 +611,7 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
   uint8_t* __restrict__ pay = a.seg.out + 10;
   uint32_t draw[UNIT];
   if (RANDOM) {
-    const uint32_t x0 = a.seg.seed + u0 * BPU;
+    const uint32_t x0 = a.seg.seed + u0 * BPU + uint32_t(PRE) * stride_bytes;  // first row that draws for itself
 #pragma unroll
     for (int q = 0; q < UNIT; q++) {
       const int jb = q / DPB, j = q % DPB;
@@ -572,7 +621,15 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
 #pragma unroll
   for (int k = 0; k < KU; k++) {
     const uint32_t u = u0 + k * rs;
-    const uint32_t packed = quant_unit<B, RANDOM>(v[k], mn, gi, draw, stride_bytes);
+    uint32_t packed;
+    if (RANDOM && k < PRE) {
+      float4 sc[H];
+#pragma unroll
+      for (int h = 0; h < H; h++) sc[h] = s_pre[(k * H + h) * kResThreads + threadIdx.x];
+      packed = quant_unit_prepared<B>(v[k], sc, mn, gi);
+    } else {
+      packed = quant_unit<B, RANDOM>(v[k], mn, gi, draw, stride_bytes);
+    }
     if (u < wg_end) {
 #pragma unroll
       for (int jb = 0; jb < BPU; jb++) pay[size_t(u) * BPU + jb] = uint8_t(packed >> (8 * jb));
@@ -882,35 +939,43 @@ bool resident_plan(int32_t n, int bits, bool random, const hpx::Workspace* ws, R
   if (rows > reg_rows + lds_rows_max) return false;
   ra.chunk_units = static_cast<uint32_t>(rows * kResThreads);
   ra.lds_rows = rows > reg_rows ? static_cast<uint32_t>(rows - reg_rows) : 0u;
+  const int spare_rows = (kResLdsTotalGroups - int(ra.lds_rows) * h) / h;
+  ra.pre_rows = (random && spare_rows >= res_pre_rows(bits)) ? static_cast<uint32_t>(res_pre_rows(bits)) : 0u;
   return true;
 }
 
-template <int B, bool RANDOM>
+template <int B, bool RANDOM, int PRE>
 int launch_resident_as(const ResArgs& ra, int num_cus, hipStream_t st) {
   constexpr int H = ((8 / B) > 4 ? (8 / B) : 4) / 4;
   static std::once_flag once;  // per instantiation
   static hipError_t attr_rc = hipSuccess;
   std::call_once(once, [] {
-    attr_rc = hipFuncSetAttribute(reinterpret_cast<const void*>(&terngrad_resident_kernel<B, RANDOM>),
+    attr_rc = hipFuncSetAttribute(reinterpret_cast<const void*>(&terngrad_resident_kernel<B, RANDOM, PRE>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  kResLdsGroups * kResThreads * int(sizeof(float4)));
+                                  kResLdsTotalGroups * kResThreads * int(sizeof(float4)));
   });
   HPX_HIP(attr_rc);
-  const size_t lds = size_t(ra.lds_rows) * H * kResThreads * sizeof(float4);
+  const size_t lds = size_t(ra.lds_rows + PRE) * H * kResThreads * sizeof(float4);
   if (hpx::g_prof_on) hpx::prof_begin("terngrad_resident_kernel", st);
-  hipLaunchKernelGGL((terngrad_resident_kernel<B, RANDOM>), dim3(num_cus), dim3(kResThreads), lds, st, ra);
+  hipLaunchKernelGGL((terngrad_resident_kernel<B, RANDOM, PRE>), dim3(num_cus), dim3(kResThreads), lds, st, ra);
   if (hpx::g_prof_on) hpx::prof_end(st);
   HPX_HIP(hipGetLastError());
   return HPX_OK;
 }
 
+template <int B>
+int launch_resident_bits(const ResArgs& ra, int num_cus, hipStream_t st) {
+  if (!ra.seg.random) return launch_resident_as<B, false, 0>(ra, num_cus, st);
+  if (ra.pre_rows) return launch_resident_as<B, true, res_pre_rows(B)>(ra, num_cus, st);
+  return launch_resident_as<B, true, 0>(ra, num_cus, st);
+}
+
 int launch_resident(const ResArgs& ra, int num_cus, hipStream_t st) {
-  const bool r = ra.seg.random != 0;
   switch (ra.seg.bits) {
-    case 1: return r ? launch_resident_as<1, true>(ra, num_cus, st) : launch_resident_as<1, false>(ra, num_cus, st);
-    case 2: return r ? launch_resident_as<2, true>(ra, num_cus, st) : launch_resident_as<2, false>(ra, num_cus, st);
-    case 4: return r ? launch_resident_as<4, true>(ra, num_cus, st) : launch_resident_as<4, false>(ra, num_cus, st);
-    default: return r ? launch_resident_as<8, true>(ra, num_cus, st) : launch_resident_as<8, false>(ra, num_cus, st);
+    case 1: return launch_resident_bits<1>(ra, num_cus, st);
+    case 2: return launch_resident_bits<2>(ra, num_cus, st);
+    case 4: return launch_resident_bits<4>(ra, num_cus, st);
+    default: return launch_resident_bits<8>(ra, num_cus, st);
   }
 }
 
