@@ -602,14 +602,20 @@ inline size_t align256(size_t x) { return (x + 255) & ~size_t(255); }
 // message `msg`; a gather launch adds values and header and clears the residual.
 int sort_and_cut(uint32_t* keys_a, int32_t* idx_a, uint32_t* keys_b, int32_t* idx_b, uint32_t* counts, uint32_t n,
                  uint8_t* msg, float* r, uint32_t keep, hipStream_t st) {
-  static std::once_flag once;
-  static hipError_t attr_rc = hipSuccess;
   constexpr int kStageBytes = 2 * kSortTile * int(sizeof(uint32_t));
-  std::call_once(once, [] {
-    attr_rc = hipFuncSetAttribute(reinterpret_cast<const void*>(&gd_sort_pass_kernel),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, kStageBytes);
-  });
-  HPX_HIP(attr_rc);
+  // The dynamic-LDS limit is a property of the function on one device: raise it once per device.
+  static std::mutex attr_mu;
+  static uint64_t attr_done = 0;  // bit d: done on device d (devices beyond 63 set it on every call)
+  {
+    int dev = 0;
+    HPX_HIP(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> g(attr_mu);
+    if (dev >= 64 || !(attr_done >> dev & 1)) {
+      HPX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gd_sort_pass_kernel),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, kStageBytes));
+      if (dev < 64) attr_done |= uint64_t(1) << dev;
+    }
+  }
   const uint32_t nblk = cdiv(n, kSortTile);
   for (int pass = 0; pass < 4; pass++) {
     SortArgs a;

@@ -947,14 +947,20 @@ bool resident_plan(int32_t n, int bits, bool random, const hpx::Workspace* ws, R
 template <int B, bool RANDOM, int PRE>
 int launch_resident_as(const ResArgs& ra, int num_cus, hipStream_t st) {
   constexpr int H = ((8 / B) > 4 ? (8 / B) : 4) / 4;
-  static std::once_flag once;  // per instantiation
-  static hipError_t attr_rc = hipSuccess;
-  std::call_once(once, [] {
-    attr_rc = hipFuncSetAttribute(reinterpret_cast<const void*>(&terngrad_resident_kernel<B, RANDOM, PRE>),
+  // The dynamic-LDS limit is a property of the function on one device: raise it once per device.
+  static std::mutex attr_mu;
+  static uint64_t attr_done = 0;  // bit d: done on device d (devices beyond 63 set it on every launch)
+  {
+    int dev = 0;
+    HPX_HIP(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> g(attr_mu);
+    if (dev >= 64 || !(attr_done >> dev & 1)) {
+      HPX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&terngrad_resident_kernel<B, RANDOM, PRE>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  kResLdsTotalGroups * kResThreads * int(sizeof(float4)));
-  });
-  HPX_HIP(attr_rc);
+                                  kResLdsTotalGroups * kResThreads * int(sizeof(float4))));
+      if (dev < 64) attr_done |= uint64_t(1) << dev;
+    }
+  }
   const size_t lds = size_t(ra.lds_rows + PRE) * H * kResThreads * sizeof(float4);
   if (hpx::g_prof_on) hpx::prof_begin("terngrad_resident_kernel", st);
   hipLaunchKernelGGL((terngrad_resident_kernel<B, RANDOM, PRE>), dim3(num_cus), dim3(kResThreads), lds, st, ra);
