@@ -410,6 +410,36 @@ def extra(torch, np, capi, L, stream, gen):
             "submit_to_finished_ms_median": round(float(np.median(lat)) * 1e3, 4),
             "submit_to_finished_ms_min": round(float(lat.min()) * 1e3, 4), "message_bytes_to_host": nbytes,
             "errors": hp.error_count()}
+
+    # 200 COMP tasks at once (the TBQ bucket, 110 M elements): the worker batches what is queued into
+    # multi-tensor encodes; 27.5 MB of messages go to pinned C buffers on the data stream
+    if hp.init("tbq", {"threshold": 1e-2}, torch.cuda.current_device(), 0, 2):
+        rng = np.random.default_rng(0)
+        sizes = np.exp(rng.uniform(np.log(768), np.log(3e7), 200))
+        sizes = np.clip(np.floor(sizes * (110e6 / sizes.sum())), 768, 3e7).astype(np.int64)
+        gs = [torch.randn(int(n_), device="cuda", generator=gen) * 5e-3 for n_ in sizes]
+        rs = [torch.zeros(int(n_), device="cuda") for n_ in sizes]
+        Bs = [torch.zeros((int(n_) + 3) // 4, dtype=torch.uint8, device="cuda") for n_ in sizes]
+        Cs = [torch.zeros((int(n_) + 3) // 4, dtype=torch.uint8, pin_memory=True) for n_ in sizes]
+        names = [f"t{i}" for i in range(200)]
+        torch.cuda.synchronize()
+        lat = []
+        for it in range(8):
+            t0 = time.perf_counter()
+            for nm, g_, r_, B_, C_ in zip(names, gs, rs, Bs, Cs):
+                hp.submit_task(nm, g_, r_, B_, C_, 0, 10)
+            got = 0
+            while got < 200:
+                hp.wait(10, 100)
+                got += len(hp.getResults(10))
+            lat.append(time.perf_counter() - t0)
+        hp.end()
+        lat = np.array(lat[2:])
+        msg_bytes = int(sum((int(n_) + 3) // 4 for n_ in sizes))
+        res["scheduler_tbq_bucket_200_comp_tasks"] = {
+            "submit_all_to_all_finished_ms_median": round(float(np.median(lat)) * 1e3, 4),
+            "elements": int(sizes.sum()), "message_bytes_to_host": msg_bytes,
+            "GBps_of_gradient": round(4.0 * float(sizes.sum()) / float(np.median(lat)) / 1e9, 1), "errors": hp.error_count()}
     return res
 
 

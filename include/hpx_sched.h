@@ -16,8 +16,10 @@
  * gathered slot but their own rank's and then re-encoding.
  * What is different: one worker thread that sleeps on a condition variable
  * (the reference polls five queues every 500 us, one for TBQ); staging copies
- * run on a data stream ordered against the compute stream by events, through
- * pinned bounce buffers when the caller's host tensor is pageable; a name is
+ * run on a data stream ordered against the compute stream by events, all
+ * messages of a phase in ONE kernel launch that reads or writes the pinned host
+ * buffers directly (through a pinned bounce buffer when the caller's host tensor
+ * is pageable) instead of one copy call per message; a name is
  * published once its own copy has landed rather than at fixed points of the
  * batch; HIP errors are counted and kept (hpx_sched_error) instead of ignored.
  */

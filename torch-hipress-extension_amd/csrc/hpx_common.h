@@ -98,6 +98,12 @@ int check_barrier_expired(Workspace* ws, const char* who);
 
 uint64_t clock_seed();
 
+// Copies `count` byte ranges in as few launches as their number allows (one kernel, a table of ranges in
+// its arguments).  Either side may be device memory or pinned host memory: the scheduler moves all
+// messages of a batch between the device buffers and the host buffers with it instead of one
+// hipMemcpyAsync per message (200 of those cost the host more than the copies take).
+int copy_ranges(int count, uint8_t* const* dst, const uint8_t* const* src, const int64_t* bytes, hipStream_t st);
+
 // How the outputs of a decode call relate: 0 = pairwise disjoint, 1 = some are
 // named more than once but every overlap is an exact duplicate (same pointer,
 // same size: several messages accumulate into one tensor), 2 = partial overlaps.

@@ -200,6 +200,79 @@ int classify_outputs(int count, float* const* outs, const int32_t* sizes) {
   return cls;
 }
 
+// ---- range copies ---------------------------------------------------------------
+namespace {
+constexpr int kCopyThreads = 256;
+constexpr int kCopySegs = 224;
+constexpr uint32_t kCopyTileBytes = kCopyThreads * 4 * 16;  // 16 KiB per workgroup
+struct CopySeg {
+  uint8_t* dst;
+  const uint8_t* src;
+  uint32_t bytes;
+  uint32_t pad;
+};
+struct CopyArgs {
+  int32_t nseg;
+  int32_t tile_start[kCopySegs + 1];
+  CopySeg seg[kCopySegs];
+};
+static_assert(sizeof(CopyArgs) <= 9600, "kernel-argument budget");
+
+struct __attribute__((packed, aligned(1))) u32x4u {
+  uint32_t x, y, z, w;
+};
+
+__global__ __launch_bounds__(kCopyThreads) void copy_ranges_kernel(const CopyArgs a) {
+  const int tile = blockIdx.x;
+  const int s = find_segment<kCopySegs>(a.tile_start, a.nseg, tile);
+  const uint8_t* __restrict__ src = a.seg[s].src;
+  uint8_t* __restrict__ dst = a.seg[s].dst;
+  const uint32_t bytes = a.seg[s].bytes;
+  const uint32_t b0 = uint32_t(tile - a.tile_start[s]) * kCopyTileBytes;
+  const uint32_t b1 = bytes - b0 < kCopyTileBytes ? bytes : b0 + kCopyTileBytes;
+  // 16-byte pieces (no alignment assumed: gfx950 global memory takes unaligned 128-bit accesses)
+  u32x4u v[4];
+  uint32_t at[4];
+#pragma unroll
+  for (int k = 0; k < 4; k++) {
+    at[k] = b0 + (k * kCopyThreads + threadIdx.x) * 16u;
+    if (at[k] + 16u <= b1) v[k] = *reinterpret_cast<const u32x4u*>(src + at[k]);
+  }
+#pragma unroll
+  for (int k = 0; k < 4; k++)
+    if (at[k] + 16u <= b1) *reinterpret_cast<u32x4u*>(dst + at[k]) = v[k];
+  // the last, partial piece of the range
+  const uint32_t whole = b0 + ((b1 - b0) & ~15u);
+  if (threadIdx.x < (b1 - whole)) dst[whole + threadIdx.x] = src[whole + threadIdx.x];
+}
+}  // namespace
+
+int copy_ranges(int count, uint8_t* const* dst, const uint8_t* const* src, const int64_t* bytes, hipStream_t st) {
+  CopyArgs a;
+  int i = 0;
+  while (i < count) {
+    a.nseg = 0;
+    a.tile_start[0] = 0;
+    while (i < count && a.nseg < kCopySegs) {
+      if (bytes[i] <= 0) { i++; continue; }
+      if (bytes[i] > int64_t(0xFFFFFFFFu) - kCopyTileBytes || !dst[i] || !src[i]) {
+        set_error("copy_ranges: range %d has %lld bytes or a null pointer", i, static_cast<long long>(bytes[i]));
+        return HPX_ERR_ARG;
+      }
+      const int64_t tiles = (bytes[i] + kCopyTileBytes - 1) / kCopyTileBytes;
+      if (int64_t(a.tile_start[a.nseg]) + tiles > INT32_MAX) break;
+      a.seg[a.nseg] = CopySeg{dst[i], src[i], static_cast<uint32_t>(bytes[i]), 0};
+      a.tile_start[a.nseg + 1] = a.tile_start[a.nseg] + static_cast<int32_t>(tiles);
+      a.nseg++;
+      i++;
+    }
+    if (a.nseg == 0) continue;
+    HPX_LAUNCH("copy_ranges_kernel", copy_ranges_kernel, dim3(a.tile_start[a.nseg]), dim3(kCopyThreads), st, a);
+    HPX_HIP(hipGetLastError());
+  }
+  return HPX_OK;
+}
+
 uint64_t clock_seed() {
   return static_cast<uint64_t>(
       std::chrono::high_resolution_clock::now().time_since_epoch().count());
