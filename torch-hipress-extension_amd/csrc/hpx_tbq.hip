@@ -206,6 +206,9 @@ __global__ __launch_bounds__(kThreads) void tbq_decode_kernel(const DecArgs<CAP>
 constexpr int kMultiSegs = 64;
 constexpr int kMultiSlots = 448;
 constexpr int kMultiSlotsPerSeg = 32;  // a tensor's messages are staged in LDS; more of them go to a later launch
+struct __attribute__((packed, aligned(1))) u32u {
+  uint32_t v;
+};
 struct MSeg {
   float* out;
   int32_t n;
@@ -245,18 +248,34 @@ __global__ __launch_bounds__(kThreads) void tbq_decode_multi_kernel(const MArgs 
   const uint32_t full = n >> 2;
   const uint32_t g0 = static_cast<uint32_t>(tile - a.tile_start[s]) * kTileGroups + threadIdx.x;
   if (g0 - threadIdx.x + kTileGroups <= full) {
-    // whole tile inside the tensor: the old values and the bytes of up to 8 messages x 4 groups are requested
-    // together, then folded in message order
+    // Whole tile inside the tensor.  A wave owns kIters * 64 consecutive groups, i.e. that many
+    // consecutive bytes of every message: each message costs the wave ONE load (a dword per lane)
+    // and the lanes pick their bytes out of it with cross-lane reads, instead of one byte load per
+    // group and message (28 loads per lane for 7 messages; the address pipeline, not memory,
+    // was the limit).  The old values and up to 8 messages are requested together, then folded in
+    // message order.
+    static_assert(kIters * 4 <= kWave, "a wave's bytes of one message must fit one dword per lane");
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    const uint32_t gw = g0 - threadIdx.x + (threadIdx.x / kWave) * uint32_t(kIters * kWave);  // the wave's first group
     float4 acc[kIters];
 #pragma unroll
     for (int k = 0; k < kIters; k++)
-      acc[k] = need_old ? ld4_stream(op + size_t(g0 + k * kThreads) * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+      acc[k] = need_old ? ld4_stream(op + size_t(gw + k * kWave + lane) * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
     for (int j0 = 0; j0 < ns; j0 += 8) {
+      uint32_t dw[8];
+#pragma unroll
+      for (int jj = 0; jj < 8; jj++) {
+        dw[jj] = 0u;
+        if (j0 + jj < ns && lane < uint32_t(kIters * kWave / 4)) {
+          dw[jj] = reinterpret_cast<const u32u*>(s_in[j0 + jj] + gw + lane * 4)->v;  // messages start at any byte
+        }
+      }
       uint32_t q[8][kIters];
 #pragma unroll
       for (int jj = 0; jj < 8; jj++)
 #pragma unroll
-        for (int k = 0; k < kIters; k++) q[jj][k] = (j0 + jj < ns) ? s_in[j0 + jj][g0 + k * kThreads] : 0u;
+        for (int k = 0; k < kIters; k++)
+          q[jj][k] = (__shfl(dw[jj], k * (kWave / 4) + lane / 4, kWave) >> (8 * (lane & 3))) & 0xFFu;
 #pragma unroll
       for (int jj = 0; jj < 8; jj++) {
         if (j0 + jj < ns) {
@@ -276,7 +295,7 @@ __global__ __launch_bounds__(kThreads) void tbq_decode_multi_kernel(const MArgs 
     }
 #pragma unroll
     for (int k = 0; k < kIters; k++) {
-      st4_stream(op + size_t(g0 + k * kThreads) * 4, acc[k]);
+      st4_stream(op + size_t(gw + k * kWave + lane) * 4, acc[k]);
       __asm__ volatile("" ::: "memory");
     }
     return;
