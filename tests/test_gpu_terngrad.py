@@ -333,3 +333,32 @@ def test_resident_kernel_belongs_to_one_stream(tg, oracle_cpu, capi):
         L.hpx_profile_enable(0); L.hpx_profile_reset()
     assert_bits_equal(host(out0), ref, "owning stream")
     assert_bits_equal(host(out1), ref, "second stream")
+
+
+def test_random_sweep_of_calls(tg, oracle_cpu, capi):
+    # seeded sweep over sizes, widths, rounding modes, seeds and call shapes; the threshold for the resident
+    # encode is lowered so that about half of the tensors take it
+    rng = np.random.default_rng(2024)
+    old = capi.set_option("terngrad_resident_min", 300_000)
+    try:
+        for call in range(12):
+            count = int(rng.integers(1, 7))
+            sizes = [int(np.exp(rng.uniform(np.log(1), np.log(3_000_000)))) for _ in range(count)]
+            xs = []
+            for n in sizes:
+                kind = int(rng.integers(0, 4))
+                x = rng.normal(0, 10.0 ** rng.uniform(-6, 2), n).astype(np.float32)
+                if kind == 1:
+                    x = np.abs(x)                       # minimum may be a zero
+                    x[rng.integers(0, n, max(1, n // 50))] = 0.0
+                elif kind == 2:
+                    x[rng.integers(0, n, max(1, n // 3))] = -0.0
+                elif kind == 3:
+                    x = np.round(x / x.std() * 2).astype(np.float32) if n > 1 and x.std() > 0 else x
+                xs.append(x)
+            bws = [int(b) for b in rng.choice([1, 2, 4, 8], count)]
+            rnds = [int(r) for r in rng.integers(0, 2, count)]
+            seeds = [int(s) for s in rng.integers(0, 2**64 - 1, count, dtype=np.uint64)]
+            _check(tg, oracle_cpu, xs, bws, rnds, seeds, [int(a) for a in rng.integers(0, 2, count)], rng)
+    finally:
+        capi.set_option("terngrad_resident_min", old)
