@@ -282,6 +282,26 @@ def extra(torch, np, capi, L, stream, gen):
     del gs, rs, ps, os_, msgs7, outs7, ins7
     torch.cuda.empty_cache()
 
+    # the same for TernGrad: 7 gathered 2-bit messages of the 25.56 M-element gradient accumulate into it
+    n = N_TERNGRAD
+    x = outlier_gradient(torch, n, gen)
+    nbytes = 10 + (n + 3) // 4
+    msgs = [torch.zeros(nbytes, dtype=torch.uint8, device="cuda") for _ in range(slots)]
+    for k in range(slots):
+        rc = L.hpx_terngrad_encode(1, capi.ptr_array([x.data_ptr()]), capi.i32_array([n]), capi.ptr_array([msgs[k].data_ptr()]),
+                                   capi.i32_array([nbytes]), capi.u8_array([2]), capi.i32_array([1]), capi.u64_array([k + 1]), stream)
+        assert rc == 0, capi.last_error()
+    acc = torch.zeros(n, device="cuda")
+    troot = Call(L.hpx_terngrad_decode, slots, capi.ptr_array([acc.data_ptr()] * slots), capi.i32_array([n] * slots),
+                 capi.ptr_array([m_.data_ptr() for m_ in msgs]), capi.i32_array([nbytes] * slots), capi.i32_array([1] * slots), stream)
+    sec = timed(torch, troot, 30, 5)
+    alg = (8.0 + 0.25 * slots) * n
+    res["terngrad_root_decode_add_7_messages_25M"] = {
+        "ms": round(sec * 1e3, 4), "algorithmic_bytes": alg, "frac_of_hbm_peak": round(alg / sec / 1e9 / HBM_PEAK_GBS, 4),
+        "bytes_if_applied_one_message_at_a_time": 8.25 * slots * n}
+    del x, msgs, acc
+    torch.cuda.empty_cache()
+
     # ---- DGC / GradDrop top-0.1 %: 138,357,544 elements --------------------------------------
     n = N_DGC
     u = torch.rand(n, device="cuda", generator=gen) - 0.5

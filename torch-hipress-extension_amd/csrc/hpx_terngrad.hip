@@ -70,6 +70,9 @@ struct EncArgs {
   uint64_t* slots;      // kSlotsPerTensor words per segment of this launch
   uint32_t epoch;       // tag of this call; slots carrying an older tag are stale
 };
+struct __attribute__((packed, aligned(1))) u32u {
+  uint32_t v;
+};
 struct DecSeg {
   float* out;
   const uint8_t* in;
@@ -846,9 +849,56 @@ __global__ __launch_bounds__(kThreads) void terngrad_decode_multi_kernel(const M
   const uint32_t g0 = static_cast<uint32_t>(tile - a.tile_start[s]) * uint32_t(kThreads * kDIters) + threadIdx.x;
   bool all_cover = true;  // every message covers the whole tensor (the normal case)
   for (int j = 0; j < ns; j++) all_cover = all_cover && s_cnt[j] == n;
+  bool all_two_bit = true;  // ... and is a 2-bit message (the configuration the reference ships with)
+  for (int j = 0; j < ns; j++) all_two_bit = all_two_bit && s_bits[j] == 2u;
+  if (all_cover && all_two_bit && uint64_t(g0 - threadIdx.x + kThreads * kDIters) * 4 <= n) {
+    // Whole tile of complete 2-bit messages.  A wave owns kDIters * 64 consecutive groups, i.e. that many
+    // consecutive payload bytes of every message: each message costs the wave ONE load (a dword per lane)
+    // and the lanes pick their bytes out of it with cross-lane reads, instead of one byte load per group
+    // and message (28 loads per lane for 7 messages: the address pipeline, not memory, was the limit).
+    static_assert(kDIters * 4 <= kWave, "a wave's bytes of one message must fit one dword per lane");
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    const uint32_t gw = g0 - threadIdx.x + (threadIdx.x / kWave) * uint32_t(kDIters * kWave);  // the wave's first group
+    float4 acc[kDIters];
+#pragma unroll
+    for (int k = 0; k < kDIters; k++)
+      acc[k] = need_old ? ld4_stream(op + size_t(gw + k * kWave + lane) * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int j0 = 0; j0 < ns; j0 += 8) {
+      uint32_t dw[8];
+#pragma unroll
+      for (int jj = 0; jj < 8; jj++) {
+        dw[jj] = 0u;
+        if (j0 + jj < ns && lane < uint32_t(kDIters * kWave / 4))
+          dw[jj] = reinterpret_cast<const u32u*>(s_pay[j0 + jj] + gw + lane * 4)->v;  // the payload starts at byte 10
+      }
+#pragma unroll
+      for (int jj = 0; jj < 8; jj++) {
+        if (j0 + jj < ns) {
+          const float gap = s_gap[j0 + jj], mn = s_mn[j0 + jj];
+          const bool add = s_add[j0 + jj] != 0;
+#pragma unroll
+          for (int k = 0; k < kDIters; k++) {
+            const uint32_t byte = (__shfl(dw[jj], k * (kWave / 4) + lane / 4, kWave) >> (8 * (lane & 3))) & 0xFFu;
+            const float4 v = group_values<2>(byte, gap, mn);
+            if (add) {
+              acc[k].x = v.x + acc[k].x; acc[k].y = v.y + acc[k].y; acc[k].z = v.z + acc[k].z; acc[k].w = v.w + acc[k].w;
+            } else {
+              acc[k] = v;
+            }
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < kDIters; k++) {
+      st4_stream(op + size_t(gw + k * kWave + lane) * 4, acc[k]);
+      __asm__ volatile("" ::: "memory");
+    }
+    return;
+  }
   if (all_cover && uint64_t(g0 - threadIdx.x + kThreads * kDIters) * 4 <= n) {
-    // Whole tile, every message complete: old values and the code bytes of up to 8 messages x 4 groups are
-    // requested together, then folded in message order.
+    // Whole tile, every message complete, other widths: old values and the code bytes of up to 8 messages x 4
+    // groups are requested together, then folded in message order.
     float4 acc[kDIters];
 #pragma unroll
     for (int k = 0; k < kDIters; k++)
