@@ -281,3 +281,17 @@ def test_submitters_on_several_threads(hp, oracle_cpu):
         msg = oracle_cpu.tbq_encode(g, rr, thr)
         assert_bits_equal(Cc.numpy(), msg, f"{name} message"); assert_bits_equal(host(dr), rr, f"{name} residual")
     assert hp.error_count() == 0, hp.last_error()
+
+
+def test_codec_failure_is_counted_and_the_task_still_finishes(hp):
+    # A body failure (here: bitwidth 3, terngrad_body.h:207-212) is printed and the loop carries on in the
+    # reference (hp_cuda_kernel.cu:63); the task's name is still pushed to its finished queue.
+    assert hp.init("terngrad", {"enable_random": 0, "bitwidth": 3}, 0, 0, 2)
+    x = torch.randn(1000, device="cuda")
+    B = torch.zeros(10 + 1000, dtype=torch.uint8, device="cuda")
+    Cc = torch.full((10 + 1000,), 7, dtype=torch.uint8)
+    torch.cuda.synchronize()
+    assert hp.submit_task("bad", x, B, Cc, 0, 10)
+    _collect(hp, 10, ["bad"])
+    assert hp.error_count() >= 1 and "bitwidth" in hp.last_error()
+    assert int(B.sum()) == 0            # nothing was encoded
