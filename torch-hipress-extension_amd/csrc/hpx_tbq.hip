@@ -52,6 +52,10 @@ struct DecArgs {
 };
 static_assert(sizeof(EncArgs<kCapLarge>) <= 9600 && sizeof(DecArgs<kCapLarge>) <= 9600, "kernel-argument budget");
 
+struct __attribute__((packed, aligned(1))) u32u {
+  uint32_t v;
+};
+
 // One element of the reference rule; returns the 2-bit code.
 __device__ __forceinline__ uint32_t tbq_code(float g, float& r, float thr) {
   r += g;
@@ -87,20 +91,33 @@ __global__ __launch_bounds__(kThreads) void tbq_encode_kernel(const EncArgs<CAP>
   const uint32_t g0 = static_cast<uint32_t>(tile - a.tile_start[s]) * kTileGroups + threadIdx.x;
 
   if (g0 - threadIdx.x + kTileGroups <= full) {
+    // Whole tile inside the tensor.  A wave owns kIters * 64 consecutive groups, i.e. 256 consecutive
+    // bytes of codes, and writes them as ONE dword per lane (a 256-byte store per wave) instead of four
+    // single-byte stores per lane.
+    static_assert(kIters == 4, "the code gather below pairs the four steps with the four lanes of a quad");
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    const uint32_t gw = g0 - threadIdx.x + (threadIdx.x / kWave) * uint32_t(kIters * kWave);  // the wave's first group
     float4 gv[kIters], rv[kIters];
 #pragma unroll
     for (int k = 0; k < kIters; k++) {
-      const size_t e = size_t(g0 + k * kThreads) * 4;
+      const size_t e = size_t(gw + k * kWave + lane) * 4;
       gv[k] = ld4_stream(gp + e);
       rv[k] = ld4_stream(rp + e);
     }
+    uint32_t d[kIters];
 #pragma unroll
     for (int k = 0; k < kIters; k++) {
-      const uint32_t grp = g0 + k * kThreads;
-      const uint32_t q = tbq_code4(gv[k], rv[k], thr);
-      st4_stream(rp + size_t(grp) * 4, rv[k]);
-      op[grp] = static_cast<uint8_t>(q);
+      uint32_t b = tbq_code4(gv[k], rv[k], thr) << (8 * (lane & 3));
+      st4_stream(rp + size_t(gw + k * kWave + lane) * 4, rv[k]);
+      b |= __shfl_xor(b, 1, kWave);
+      b |= __shfl_xor(b, 2, kWave);
+      d[k] = b;  // every lane of quad m: the four bytes of groups gw + 64k + 4m .. +3, i.e. dword 16k + m of the wave
     }
+    // Lane 4m + k of a quad offers dword 16k + m; lane l fetches dword l from lane 4 (l % 16) + l / 16.
+    const uint32_t i = lane & 3;
+    const uint32_t offer = i == 0 ? d[0] : i == 1 ? d[1] : i == 2 ? d[2] : d[3];
+    const uint32_t dw = __shfl(offer, int(4 * (lane & 15) + (lane >> 4)), kWave);
+    reinterpret_cast<u32u*>(op + gw + 4 * lane)->v = dw;  // messages start at any byte
     return;
   }
   // Last tile of the tensor: bounds-checked, and the lane owning the partial
@@ -206,9 +223,6 @@ __global__ __launch_bounds__(kThreads) void tbq_decode_kernel(const DecArgs<CAP>
 constexpr int kMultiSegs = 64;
 constexpr int kMultiSlots = 448;
 constexpr int kMultiSlotsPerSeg = 32;  // a tensor's messages are staged in LDS; more of them go to a later launch
-struct __attribute__((packed, aligned(1))) u32u {
-  uint32_t v;
-};
 struct MSeg {
   float* out;
   int32_t n;
