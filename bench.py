@@ -409,7 +409,10 @@ def extra(torch, np, capi, L, stream, gen):
     # ---- the scheduler around the path: one COMP task, submit -> name in the finished queue ------------
     # (TernGrad 2-bit, 25.56 M elements; includes the 6.4 MB device-to-host copy of the message into a
     # pinned C buffer and both thread hand-overs; the reference's worker polls its queue every 500 us)
-    hp = importlib.import_module("torch-hipress-extension_amd").hp_cuda
+    ext_dir = os.path.join(ROOT, "torch-hipress-extension_amd", "ext")   # the compiled `hp_cuda` extension module
+    if ext_dir not in sys.path:
+        sys.path.insert(0, ext_dir)
+    hp = importlib.import_module("hp_cuda")
     if hp.init("terngrad", {"enable_random": 1, "bitwidth": 2, "seed": 0}, torch.cuda.current_device(), 0, 2):
         n = N_TERNGRAD
         x = outlier_gradient(torch, n, gen)

@@ -26,6 +26,17 @@ def capi(pkg):
 
 
 @pytest.fixture(scope="session")
+def hp_cuda_compiled(pkg):
+    """The compiled torch extension `hp_cuda` (csrc/hp_cuda_module.cpp), imported by its top-level name as
+    a caller of the reference's extension would; it must have been built (make -C csrc)."""
+    import torch  # noqa: F401  (the extension links libtorch)
+    ext_dir = os.path.join(os.path.dirname(pkg.__file__), "ext")
+    if ext_dir not in sys.path:
+        sys.path.insert(0, ext_dir)
+    return importlib.import_module("hp_cuda")
+
+
+@pytest.fixture(scope="session")
 def oracle_cpu():
     from oracle import cpu
     cpu.lib()

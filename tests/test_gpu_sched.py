@@ -1,6 +1,8 @@
 """GPU parity of the task scheduler (hp_cuda.init / submit_task / getResults over libhpx.so) against the
 CPU oracle: what a COMP, DECOMP and ROOT_DECOMP_COMP task leaves in C, in the gradient and in the
-residual, and which finished queue its name appears in (hp_cuda.cpp:163-772, :1043-1066)."""
+residual, and which finished queue its name appears in (hp_cuda.cpp:163-772, :1043-1066).  Every test
+runs through both front ends of the scheduler: the compiled `hp_cuda` extension module and the ctypes
+module of the package."""
 import numpy as np
 import pytest
 import torch
@@ -10,13 +12,14 @@ from gpu_util import assert_bits_equal, dev, host
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture
-def hp(pkg):
+@pytest.fixture(params=["compiled", "ctypes"])
+def hp(request, pkg, hp_cuda_compiled):
     assert torch.cuda.is_available()
-    yield pkg.hp_cuda
-    pkg.hp_cuda.end()
+    mod = hp_cuda_compiled if request.param == "compiled" else pkg.hp_cuda
+    yield mod
+    mod.end()
     for q in (10, 20, 30):
-        pkg.hp_cuda.getResults(q)
+        mod.getResults(q)
 
 
 def _collect(hp, task_id, names, timeout_s=20.0):
