@@ -56,7 +56,7 @@ __device__ __forceinline__ f32x4 mfma4(float a, float b, f32x4 c) {
 }
 
 // ---- encode1: M = G + R (flat prefix), P = M Q -------------------------------
-// One workgroup per group of 4 rows; its 4 waves split the columns and meet in
+// One workgroup per group of 4 rows; its 4 waves share out the columns and meet in
 // LDS.  Lane 4b+i of a wave owns row i and the 4 columns k0+4b..k0+4b+3 of each
 // 64-column step, which is one 128-bit load of G and of R and one store of M.
 template <int CG>
@@ -74,23 +74,22 @@ __global__ __launch_bounds__(kThreads) void psgd_encode1_kernel(const Args a) {
   const int row0 = (tile - a.tile_start[s]) * 4;
   const int i = lane & 3, b = lane >> 2;
   const int row = row0 + i;
-  // columns of this wave: a contiguous quarter, in whole 64-column steps
-  const int steps = (m + 63) / 64;
-  const int per = (steps + kWaves - 1) / kWaves;
-  const int kbeg = wave * per * 64;
-  int kend = kbeg + per * 64;
-  if (kend > m) kend = m;
+  // Columns: the workgroup walks the rows in chunks of kWaves * 256 columns, wave w taking the w-th 256 of each
+  // chunk, so that at any time the four waves read neighbouring pieces of the same four rows (a contiguous
+  // quarter of the row per wave ran 9 % slower); what is left past the last whole 256 goes round the waves in
+  // 64-column steps.
+  constexpr int kUnroll = 4;
+  constexpr int kChunk = 64 * kUnroll;
+  const int mfull = m / kChunk * kChunk;
 
   f32x4 acc[CG];
 #pragma unroll
   for (int c = 0; c < CG; c++) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   const bool rows_full = (row0 + 3 < n) && (int64_t(row0 + 4) * m <= N);
-  int k0 = kbeg;
   if (rows_full) {
     // Main loop: kUnroll 64-column steps at a time, every load issued before the first use.
-    constexpr int kUnroll = 4;
-    for (; k0 + 64 * kUnroll <= kend; k0 += 64 * kUnroll) {
+    for (int k0 = wave * kChunk; k0 < mfull; k0 += kWaves * kChunk) {
       float4 g4[kUnroll], r4[kUnroll];
       float q[kUnroll][4][CG];
 #pragma unroll
@@ -121,7 +120,7 @@ __global__ __launch_bounds__(kThreads) void psgd_encode1_kernel(const Args a) {
       }
     }
   }
-  for (; k0 < kend; k0 += 64) {
+  for (int k0 = (rows_full ? mfull : 0) + wave * 64; k0 < m; k0 += kWaves * 64) {
     const int kk = k0 + 4 * b;
     float v[4];
     if (rows_full && k0 + 64 <= m) {
