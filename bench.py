@@ -119,6 +119,8 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
     torch.cuda.set_device(0)
+    import __graft_entry__
+    __graft_entry__.ensure_built()     # loads what is built; builds only if nothing is
     pkg = importlib.import_module("torch-hipress-extension_amd")
     capi = pkg._capi
     L = capi.load()

@@ -15,7 +15,10 @@ def pytest_configure(config):
 
 @pytest.fixture(scope="session")
 def pkg():
-    """The product package (its directory name is not a Python identifier)."""
+    """The product package (its directory name is not a Python identifier).  The tests load what is built;
+    only when nothing is built do they run the build first."""
+    import __graft_entry__
+    __graft_entry__.ensure_built()
     return importlib.import_module("torch-hipress-extension_amd")
 
 
