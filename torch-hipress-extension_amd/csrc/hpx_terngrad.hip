@@ -782,6 +782,7 @@ __global__ __launch_bounds__(kThreads) void terngrad_decode_kernel(const DecArgs
 constexpr int kMultiSegs = 64;
 constexpr int kMultiSlots = 448;
 constexpr int kMultiSlotsPerSeg = 32;  // header fields of one tensor's messages are staged in LDS
+constexpr int kMultiRep = 4;            // sub-tiles of kDecTile elements per workgroup of the multi-message decode
 struct MSeg {
   float* out;
   int32_t out_size;
@@ -846,11 +847,14 @@ __global__ __launch_bounds__(kThreads) void terngrad_decode_multi_kernel(const M
   __syncthreads();
   const uint32_t n = static_cast<uint32_t>(a.seg[s].out_size);
   const bool need_old = s_add[0] != 0;
-  const uint32_t g0 = static_cast<uint32_t>(tile - a.tile_start[s]) * uint32_t(kThreads * kDIters) + threadIdx.x;
   bool all_cover = true;  // every message covers the whole tensor (the normal case)
   for (int j = 0; j < ns; j++) all_cover = all_cover && s_cnt[j] == n;
   bool all_two_bit = true;  // ... and is a 2-bit message (the configuration the reference ships with)
   for (int j = 0; j < ns; j++) all_two_bit = all_two_bit && s_bits[j] == 2u;
+  // The headers are parsed once per workgroup and serve kMultiRep consecutive sub-tiles.
+  for (uint32_t rep = 0; rep < uint32_t(kMultiRep); rep++) {
+  const uint32_t g0 = (static_cast<uint32_t>(tile - a.tile_start[s]) * kMultiRep + rep) * uint32_t(kThreads * kDIters) + threadIdx.x;
+  if (uint64_t(g0 - threadIdx.x) * 4 >= n) break;
   if (all_cover && all_two_bit && uint64_t(g0 - threadIdx.x + kThreads * kDIters) * 4 <= n) {
     // Whole tile of complete 2-bit messages.  A wave owns kDIters * 64 consecutive groups, i.e. that many
     // consecutive payload bytes of every message: each message costs the wave ONE load (a dword per lane)
@@ -894,7 +898,7 @@ __global__ __launch_bounds__(kThreads) void terngrad_decode_multi_kernel(const M
       st4_stream(op + size_t(gw + k * kWave + lane) * 4, acc[k]);
       __asm__ volatile("" ::: "memory");
     }
-    return;
+    continue;
   }
   if (all_cover && uint64_t(g0 - threadIdx.x + kThreads * kDIters) * 4 <= n) {
     // Whole tile, every message complete, other widths: old values and the code bytes of up to 8 messages x 4
@@ -947,7 +951,7 @@ __global__ __launch_bounds__(kThreads) void terngrad_decode_multi_kernel(const M
       st4_stream(op + size_t(g0 + k * kThreads) * 4, acc[k]);
       __asm__ volatile("" ::: "memory");
     }
-    return;
+    continue;
   }
   for (int k = 0; k < kDIters; k++) {
     const size_t e = size_t(g0 + k * kThreads) * 4;
@@ -965,6 +969,7 @@ __global__ __launch_bounds__(kThreads) void terngrad_decode_multi_kernel(const M
       }
       if (touched) op[e + i] = acc;
     }
+  }
   }
 }
 
@@ -1158,7 +1163,7 @@ int launch_decode_multi(int count, float* const* outs, const int32_t* out_sizes,
   }
   MArgs a;
   a.status = status;
-  auto tiles_of = [](int32_t n) { return ceil_div(n, kDecTile); };
+  auto tiles_of = [](int32_t n) { return ceil_div(n, kDecTile * kMultiRep); };
   while (left > 0) {
     const std::vector<MultiGroup> groups = plan_multi_launch(count, outs, out_sizes, done, tiles_of);
     a.nseg = 0;
