@@ -229,9 +229,40 @@ def cpu_baseline(np, n, budget_s):
         one()
         reps += 1
     sec = (time.perf_counter() - t0) / reps
-    return {"value": round(4.0 * n / sec / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
-            "sample": f"{reps} full encode+decode passes of the same {n}-element workload, OpenMP over {threads} threads "
-                      f"(os.cpu_count()={os.cpu_count()})", "ms_per_step": round(sec * 1e3, 2)}
+    res = {"value": round(4.0 * n / sec / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+           "sample": f"{reps} full encode+decode passes of the same {n}-element workload, OpenMP over {threads} threads "
+                     f"(os.cpu_count()={os.cpu_count()})", "ms_per_step": round(sec * 1e3, 2)}
+    # the same port on one thread
+    cpu.set_threads(1)
+    t0 = time.perf_counter()
+    for _ in range(2):
+        one()
+    sec1 = (time.perf_counter() - t0) / 2
+    cpu.set_threads(threads)
+    res["one_thread"] = {"value": round(4.0 * n / sec1 / 1e9, 3), "ms_per_step": round(sec1 * 1e3, 2)}
+    # The reference's own header bodies (terngrad_body / terngrad_r_body under thrust::omp::par), where the
+    # host build of them exists: it is made from a reference checkout and travels as a built library.
+    from oracle import ref
+    if ref.available():
+        msg = np.zeros(10 + (n + 3) // 4, np.uint8)
+
+        def ref_one():
+            rc = ref.lib().ref_terngrad_encode(ref._f32(x), n, ref._u8(msg), msg.size, 2, 1, 1)
+            rc2, _ = ref.terngrad_decode(msg, n, out, 0, 1)
+            assert rc == 0 and rc2 == 0
+
+        ref_one()
+        t0 = time.perf_counter()
+        r_reps = 0
+        while r_reps < 3 or (time.perf_counter() - t0 < budget_s / 2 and r_reps < 100):
+            ref_one()
+            r_reps += 1
+        rsec = (time.perf_counter() - t0) / r_reps
+        res["reference_bodies"] = {"value": round(4.0 * n / rsec / 1e9, 3), "unit": "GB/s", "ms_per_step": round(rsec * 1e3, 2),
+                                   "policy": "thrust::omp::par", "threads": threads,
+                                   "sample": f"{r_reps} encode+decode passes of the same workload through the reference's "
+                                             "terngrad_body / terngrad_r_body compiled for the host (clock-seeded)"}
+    return res
 
 
 def extra(torch, np, capi, L, stream, gen):
