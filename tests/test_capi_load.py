@@ -37,3 +37,11 @@ def test_ops_mirror_reference_names(pkg):
     for name in ("hp_cuda_terngrad", "hp_cuda_terngradr", "hp_cuda_tbq", "hp_cuda_tbqr", "hp_cuda_gd", "hp_cuda_gdr",
                  "hp_cuda_powersgd_encode1", "hp_cuda_powersgd_encode2", "hp_cuda_powersgd_decode"):
         assert callable(getattr(pkg, name))
+
+
+def test_driver_module_exposes_the_nine_reference_drivers(hp_cuda_compiled):
+    import importlib
+    drv = importlib.import_module("hp_cuda_drivers")
+    for name in ("hp_cuda_terngrad", "hp_cuda_terngradr", "hp_cuda_tbq", "hp_cuda_tbqr", "hp_cuda_gd", "hp_cuda_gdr",
+                 "hp_cuda_powersgd_encode1", "hp_cuda_powersgd_encode2", "hp_cuda_powersgd_decode"):
+        assert callable(getattr(drv, name))
