@@ -4,10 +4,11 @@
  * drivers: Task / TaskQueue / FinishQueue / ThreadManager (hp_cuda.h:28-148),
  * the four RunLoopOnceFor* batch builders (hp_cuda.cpp:163-772), the B <-> C
  * staging copies they issue, and init / end / submit_task / getResults
- * (hp_cuda.cpp:824-1066).  Signatures use plain pointers and sizes; the Python
- * module torch-hipress-extension_amd/hp_cuda.py puts the reference's
- * torch-tensor interface (hp_cuda.cpp:1073-1080) on top and keeps the tensors
- * alive while a task is in flight.
+ * (hp_cuda.cpp:824-1066).  Signatures use plain pointers and sizes; the torch
+ * extension csrc/hp_cuda_module.cpp (and torch-hipress-extension_amd/hp_cuda.py
+ * over ctypes) puts the reference's torch-tensor interface
+ * (hp_cuda.cpp:1073-1080) on top and keeps the tensors alive while a task is in
+ * flight.
  *
  * What is kept: task ids, the grouping of one batch's tasks into multi-tensor
  * codec calls and their order (per algorithm, see hpx_sched.cpp), which
@@ -21,7 +22,9 @@
  * buffers directly (through a pinned bounce buffer when the caller's host tensor
  * is pageable) instead of one copy call per message; a name is
  * published once its own copy has landed rather than at fixed points of the
- * batch; HIP errors are counted and kept (hpx_sched_error) instead of ignored.
+ * batch; HIP errors are counted and kept (hpx_sched_error) instead of ignored;
+ * a task whose buffers are too small for its message is skipped and counted as
+ * a failure (the reference overruns them), and its name is still published.
  */
 #ifndef HPX_SCHED_H_
 #define HPX_SCHED_H_

@@ -298,3 +298,18 @@ def test_codec_failure_is_counted_and_the_task_still_finishes(hp):
     _collect(hp, 10, ["bad"])
     assert hp.error_count() >= 1 and "bitwidth" in hp.last_error()
     assert int(B.sum()) == 0            # nothing was encoded
+
+
+def test_task_with_too_small_buffers_is_skipped_counted_and_still_named(hp):
+    n, sr, dr_ = 100_003, 0.05, 0.99
+    assert hp.init("graddrop", {"sample_rate": sr, "drop_ratio": dr_, "seed": 1}, 0, 0, 2)
+    g = torch.randn(n, device="cuda") * 1e-3
+    res = torch.zeros(n, device="cuda")
+    before = hp.error_count()
+    B = torch.zeros(64, dtype=torch.uint8, device="cuda")            # far less than 4 + 8*ceil(n*(1-drop))
+    Cc = torch.zeros(64, dtype=torch.uint8, pin_memory=True)
+    torch.cuda.synchronize()
+    assert hp.submit_task("tiny", g, res, B, Cc, 0, 20)
+    _collect(hp, 20, ["tiny"])
+    assert hp.error_count() == before + 1 and "does not fit" in hp.last_error()
+    assert float(g.abs().max()) > 0 and int(Cc.sum()) == 0           # nothing was decoded, nothing written

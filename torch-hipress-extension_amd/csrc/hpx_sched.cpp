@@ -475,13 +475,21 @@ void worker_main() {
     }
     for (Task& t : batch) t.t.name = t.name.c_str();
     if (p.alg == kPowersgd) run_powersgd_batch(w, p, batch); else run_codec_batch(w, p, batch);
-    // a task that failed its checks is not published, but its buffers are released
+    // A task that failed its checks was skipped (the failure is counted and kept for hpx_sched_error); its
+    // name is published all the same, once the batch has drained, so that a caller polling for it does not
+    // wait for ever: the reference publishes every task of a batch (hp_cuda.cpp:626-636).
     SCHED_HIP(hipStreamSynchronize(w.compute));
     SCHED_HIP(hipStreamSynchronize(w.data));
     {
+      bool any = false;
       std::lock_guard<std::mutex> l(g.fmu);
-      for (const Task& t : batch)
-        if (!t.published) g.done.push_back(t.serial);
+      for (const Task& t : batch) {
+        if (t.published) continue;
+        const int q = queue_of(t.t.task_id);
+        if (q >= 0) { g.finished[q].push_back(t.name); any = true; }
+        g.done.push_back(t.serial);
+      }
+      if (any) g.fcv.notify_all();
     }
   }
   (void)hipStreamSynchronize(w.compute);
