@@ -264,7 +264,8 @@ def cpu_baseline(np, n, budget_s):
         res = {"value": round(4.0 * n / rsec / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "reference",
                "sample": f"{r_reps} full encode+decode passes of the same {n}-element workload through the reference's "
                          f"terngrad_body / terngrad_r_body compiled for the host, thrust::omp::par over {threads} threads "
-                         f"(clock-seeded; os.cpu_count()={os.cpu_count()})",
+                         f"(clock-seeded; os.cpu_count()={os.cpu_count()}); the bodies' memcpy/sync policy shim is the "
+                         "harness's own, all arithmetic and Thrust calls are the reference's",
                "ms_per_step": round(rsec * 1e3, 2), "port": port}
     return res
 
