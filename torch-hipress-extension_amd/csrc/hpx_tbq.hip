@@ -78,6 +78,32 @@ __device__ __forceinline__ uint32_t tbq_code4(const float4& g, float4& r, float 
   return q;
 }
 
+// Tiles are laid on absolute addresses: a workgroup's 16 KiB of residual (encode) or output (decode)
+// starts on a 16 KiB boundary whatever the tensor's base address is, because a tile that straddles such a
+// boundary streams measurably slower (7 % at an offset of 8 KiB).  The groups before the first boundary,
+// `head` of them, form a short first tile.  Host and kernels use the same two functions.
+__host__ __device__ inline uint32_t tbq_head_groups(const void* p, uint32_t total_groups) {
+  const uint32_t to_boundary = (16384u - (static_cast<uint32_t>(reinterpret_cast<uintptr_t>(p)) & 16383u)) & 16383u;
+  const uint32_t h = (to_boundary + 15u) >> 4;  // groups of 16 bytes
+  return h >= total_groups ? 0u : h;
+}
+__host__ __device__ inline uint32_t tbq_tiles(const void* p, uint32_t n) {
+  const uint32_t total = (n + 3u) >> 2;
+  const uint32_t head = tbq_head_groups(p, total);
+  return (head ? 1u : 0u) + (total - head + uint32_t(kTileGroups) - 1u) / uint32_t(kTileGroups);
+}
+// Groups [gbeg, glim) of tile t (glim may lie past the end of the tensor for its last tile).
+__device__ __forceinline__ void tbq_tile_range(const void* p, uint32_t n, uint32_t t, uint32_t& gbeg, uint32_t& glim) {
+  const uint32_t head = tbq_head_groups(p, (n + 3u) >> 2);
+  if (head && t == 0) {
+    gbeg = 0;
+    glim = head;
+  } else {
+    gbeg = head + (t - (head ? 1u : 0u)) * uint32_t(kTileGroups);
+    glim = gbeg + uint32_t(kTileGroups);
+  }
+}
+
 template <int CAP>
 __global__ __launch_bounds__(kThreads) void tbq_encode_kernel(const EncArgs<CAP> a) {
   const int tile = blockIdx.x;
@@ -88,9 +114,11 @@ __global__ __launch_bounds__(kThreads) void tbq_encode_kernel(const EncArgs<CAP>
   const uint32_t n = static_cast<uint32_t>(a.seg[s].n);
   const float thr = a.seg[s].thr;
   const uint32_t full = n >> 2;  // complete groups
-  const uint32_t g0 = static_cast<uint32_t>(tile - a.tile_start[s]) * kTileGroups + threadIdx.x;
+  uint32_t gbeg, glim;
+  tbq_tile_range(rp, n, static_cast<uint32_t>(tile - a.tile_start[s]), gbeg, glim);
+  const uint32_t g0 = gbeg + threadIdx.x;
 
-  if (g0 - threadIdx.x + kTileGroups <= full) {
+  if (glim - gbeg == uint32_t(kTileGroups) && glim <= full) {
     // Whole tile inside the tensor.  A wave owns kIters * 64 consecutive groups, i.e. 256 consecutive
     // bytes of codes, and writes them as ONE dword per lane (a 256-byte store per wave) instead of four
     // single-byte stores per lane.
@@ -120,18 +148,29 @@ __global__ __launch_bounds__(kThreads) void tbq_encode_kernel(const EncArgs<CAP>
     reinterpret_cast<u32u*>(op + gw + 4 * lane)->v = dw;  // messages start at any byte
     return;
   }
-  // Last tile of the tensor: bounds-checked, and the lane owning the partial
-  // group leaves the fields past the end at code 1.
+  // First (short) or last tile of the tensor: bounds-checked, and the lane owning the
+  // partial group leaves the fields past the end at code 1.  All loads first: the last
+  // tile of the last tensor is the tail of the launch.
+  const uint32_t lim = glim < full ? glim : full;  // complete groups of this tile end here
+  float4 gt[kIters], rt[kIters];
+#pragma unroll
+  for (int k = 0; k < kIters; k++) {
+    const uint32_t grp = g0 + k * kThreads;
+    if (grp < lim) {
+      gt[k] = ld4(gp + size_t(grp) * 4);
+      rt[k] = ld4(rp + size_t(grp) * 4);
+    }
+  }
 #pragma unroll
   for (int k = 0; k < kIters; k++) {
     const uint32_t grp = g0 + k * kThreads;
     const size_t e = size_t(grp) * 4;
-    if (grp < full) {
-      float4 gv = ld4(gp + e), rv = ld4(rp + e);
+    if (grp < lim) {
+      float4 gv = gt[k], rv = rt[k];
       const uint32_t q = tbq_code4(gv, rv, thr);
       st4(rp + e, rv);
       op[grp] = static_cast<uint8_t>(q);
-    } else if (grp == full && (n & 3)) {
+    } else if (grp == full && grp < glim && (n & 3)) {
       uint32_t q = 85;
       for (uint32_t j = 0; j < (n & 3); j++) {
         float r = rp[e + j];
@@ -151,13 +190,16 @@ __device__ __forceinline__ float4 tbq_values(uint32_t q, float thr) {
 }
 
 template <bool ADD>
-__device__ __forceinline__ void tbq_decode_tile(const DecSeg& sg, uint32_t g0, bool stream_store) {
+__device__ __forceinline__ void tbq_decode_tile(const DecSeg& sg, uint32_t t, bool stream_store) {
   float* __restrict__ op = sg.out;
   const uint8_t* __restrict__ ip = sg.in;
   const uint32_t n = static_cast<uint32_t>(sg.n);
   const float thr = sg.thr;
   const uint32_t full = n >> 2;
-  if (g0 - threadIdx.x + kTileGroups <= full) {
+  uint32_t gbeg, glim;
+  tbq_tile_range(op, n, t, gbeg, glim);
+  const uint32_t g0 = gbeg + threadIdx.x;
+  if (glim - gbeg == uint32_t(kTileGroups) && glim <= full) {
     uint32_t q[kIters];
     float4 acc[kIters];
 #pragma unroll
@@ -181,18 +223,29 @@ __device__ __forceinline__ void tbq_decode_tile(const DecSeg& sg, uint32_t g0, b
     }
     return;
   }
+  const uint32_t lim = glim < full ? glim : full;  // complete groups of this (first or last) tile end here
+  uint32_t qt[kIters];
+  float4 ot[kIters];
+#pragma unroll
+  for (int k = 0; k < kIters; k++) {  // all loads first: the last tile of the last tensor is the tail of the launch
+    const uint32_t grp = g0 + k * kThreads;
+    if (grp < lim) {
+      qt[k] = ip[grp];
+      if (ADD) ot[k] = ld4(op + size_t(grp) * 4);
+    }
+  }
 #pragma unroll
   for (int k = 0; k < kIters; k++) {
     const uint32_t grp = g0 + k * kThreads;
     const size_t e = size_t(grp) * 4;
-    if (grp < full) {
-      float4 v = tbq_values(ip[grp], thr);
+    if (grp < lim) {
+      float4 v = tbq_values(qt[k], thr);
       if (ADD) {
-        const float4 o = ld4(op + e);
+        const float4 o = ot[k];
         v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w;
       }
       st4(op + e, v);
-    } else if (grp == full && (n & 3)) {
+    } else if (grp == full && grp < glim && (n & 3)) {
       const uint32_t q = ip[grp];
       for (uint32_t j = 0; j < (n & 3); j++) {
         const float v = (static_cast<float>((q >> (2 * j)) & 3) - 1) * thr;
@@ -206,11 +259,11 @@ template <int CAP>
 __global__ __launch_bounds__(kThreads) void tbq_decode_kernel(const DecArgs<CAP> a) {
   const int tile = blockIdx.x;
   const int s = find_segment<CAP>(a.tile_start, a.nseg, tile);
-  const uint32_t g0 = static_cast<uint32_t>(tile - a.tile_start[s]) * kTileGroups + threadIdx.x;
+  const uint32_t t = static_cast<uint32_t>(tile - a.tile_start[s]);
   if (a.seg[s].add)
-    tbq_decode_tile<true>(a.seg[s], g0, true);
+    tbq_decode_tile<true>(a.seg[s], t, true);
   else
-    tbq_decode_tile<false>(a.seg[s], g0, a.stream_store != 0);
+    tbq_decode_tile<false>(a.seg[s], t, a.stream_store != 0);
 }
 
 // ---- several messages into one tensor ---------------------------------------
@@ -348,7 +401,7 @@ int launch_encode(int count, const float* const* grads, const int32_t* sizes, fl
       HPX_ARG(n >= 0, "hpx_tbq_encode: tensor %d has negative size %d", i, n);
       if (n > 0) {
         HPX_ARG(grads[i] && residuals[i] && outs[i], "hpx_tbq_encode: tensor %d has a null pointer", i);
-        const int32_t t = tiles_for(n);
+        const int32_t t = static_cast<int32_t>(tbq_tiles(residuals[i], static_cast<uint32_t>(n)));
         if (int64_t(a.tile_start[a.nseg]) + t > INT32_MAX) break;  // next launch
         a.seg[a.nseg] = EncSeg{grads[i], residuals[i], outs[i], n, thresholds[i]};
         a.tile_start[a.nseg + 1] = a.tile_start[a.nseg] + t;
@@ -379,7 +432,7 @@ int launch_decode(int count, float* const* outs, const int32_t* sizes, const uin
       HPX_ARG(n >= 0, "hpx_tbq_decode: tensor %d has negative size %d", i, n);
       if (n > 0) {
         HPX_ARG(outs[i] && ins[i], "hpx_tbq_decode: tensor %d has a null pointer", i);
-        const int32_t t = tiles_for(n);
+        const int32_t t = static_cast<int32_t>(tbq_tiles(outs[i], static_cast<uint32_t>(n)));
         if (int64_t(a.tile_start[a.nseg]) + t > INT32_MAX) break;
         a.seg[a.nseg] = DecSeg{outs[i], ins[i], n, thresholds[i], is_add_tos[i] != 0, 0};
         a.tile_start[a.nseg + 1] = a.tile_start[a.nseg] + t;
