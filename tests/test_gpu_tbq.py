@@ -96,6 +96,49 @@ def test_unaligned_views(tbq, oracle_cpu):
     assert float(out[0]) == 0.0
 
 
+def test_tiles_on_address_boundaries(tbq, oracle_cpu):
+    # Workgroup tiles start on 16 KiB address boundaries; the groups before the first boundary form a short
+    # first tile.  Tensors that start at chosen distances from a boundary, with sizes around the first
+    # tile's length, must encode and decode as anywhere else; all of them go out in one call.
+    rng = np.random.default_rng(21)
+    thr = 2e-3
+    span = 3 * 4096 + 64
+    gs, rs, views_g, views_r, views_o, views_d, bases = [], [], [], [], [], [], []
+    for off in (0, 4, 2048, 4092, 4095, 1, 3073):          # elements past a 16 KiB boundary
+        to_boundary = (-(off * 4)) % 16384
+        head = (to_boundary + 15) // 16                     # groups before the first boundary
+        for n in sorted({1, 3, 4, 5, max(1, 4 * head - 1), 4 * head, 4 * head + 1, 4 * head + 3, 4 * head + 4,
+                         4 * head + 4096, 4 * head + 4097, 4 * head + 2 * 4096 + 2}):
+            if n > span - 8 or n < 1:
+                continue
+            gbuf = torch.zeros(4096 * 2 + span, device="cuda")
+            rbuf = torch.zeros(4096 * 2 + span, device="cuda")
+            dbuf = torch.zeros(4096 * 2 + span, device="cuda")
+            obuf = torch.full(((span + 3) // 4 + 8,), 0xAA, dtype=torch.uint8, device="cuda")
+            # first element of the view sits `off` elements past a 16 KiB boundary of ITS buffer's address
+            def view(buf, n_):
+                skip = ((-buf.data_ptr()) % 16384) // 4 + off
+                return buf[skip:skip + n_]
+            g = rng.normal(0, 2e-3, n).astype(np.float32)
+            r = rng.normal(0, 1e-3, n).astype(np.float32)
+            b = rng.normal(0, 1, n).astype(np.float32)
+            vg, vr, vd = view(gbuf, n), view(rbuf, n), view(dbuf, n)
+            vg.copy_(dev(g)); vr.copy_(dev(r)); vd.copy_(dev(b))
+            gs.append(g); rs.append(r); bases.append(b)
+            views_g.append(vg); views_r.append(vr); views_d.append(vd); views_o.append(obuf[5:5 + (n + 3) // 4])
+    tbq.encode(views_g, views_r, [thr] * len(gs), outs=views_o)
+    adds = [i % 2 for i in range(len(gs))]
+    tbq.decode(views_o, views_d, [thr] * len(gs), adds)
+    torch.cuda.synchronize()
+    for i, (g, r) in enumerate(zip(gs, rs)):
+        r_ref = r.copy()
+        p_ref = oracle_cpu.tbq_encode(g, r_ref, thr)
+        assert_bits_equal(host(views_o[i]), p_ref, f"packed, case {i} n={g.size}")
+        assert_bits_equal(host(views_r[i]), r_ref, f"residual, case {i} n={g.size}")
+        assert_bits_equal(host(views_d[i]), oracle_cpu.tbq_decode(p_ref, g.size, thr, bases[i].copy(), adds[i]),
+                          f"decoded, case {i} n={g.size} add={adds[i]}")
+
+
 def test_bucket_of_many_tensors(tbq, oracle_cpu):
     # More tensors than one launch table holds, ragged sizes, per-tensor thresholds,
     # an empty tensor in the middle; two consecutive steps exercise residual feedback.
