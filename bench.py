@@ -340,6 +340,38 @@ def extra(torch, np, capi, L, stream, gen):
     del x, msgs, acc
     torch.cuda.empty_cache()
 
+    # ---- TernGrad over ResNet-50's own 161 parameter tensors (the same 25,557,032 elements, one call each way) ----
+    r50 = [64 * 3 * 7 * 7, 64, 64]
+    inp = 64
+    for planes, blocks in ((64, 3), (128, 4), (256, 6), (512, 3)):
+        for b in range(blocks):
+            r50 += [planes * inp, planes, planes, planes * planes * 9, planes, planes, planes * 4 * planes, planes * 4, planes * 4]
+            if b == 0:
+                r50 += [planes * 4 * inp, planes * 4, planes * 4]
+            inp = planes * 4
+    r50 += [1000 * 2048, 1000]
+    assert sum(r50) == N_TERNGRAD
+    xs = [torch.randn(m_, device="cuda", generator=gen) * 1e-2 for m_ in r50]
+    ms_ = [torch.zeros(10 + (m_ + 3) // 4, dtype=torch.uint8, device="cuda") for m_ in r50]
+    ds_ = [torch.empty(m_, device="cuda") for m_ in r50]
+    k_ = len(r50)
+    enc = Call(L.hpx_terngrad_encode, k_, capi.ptr_array([t_.data_ptr() for t_ in xs]), capi.i32_array(r50),
+               capi.ptr_array([t_.data_ptr() for t_ in ms_]), capi.i32_array([t_.numel() for t_ in ms_]), capi.u8_array([2] * k_),
+               capi.i32_array([1] * k_), capi.u64_array(list(range(k_))), stream)
+    dec = Call(L.hpx_terngrad_decode, k_, capi.ptr_array([t_.data_ptr() for t_ in ds_]), capi.i32_array(r50),
+               capi.ptr_array([t_.data_ptr() for t_ in ms_]), capi.i32_array([t_.numel() for t_ in ms_]), capi.i32_array([0] * k_), stream)
+
+    def r50_step():
+        enc()
+        dec()
+
+    sec = timed(torch, r50_step, 50, 10)
+    res["terngrad_resnet50_161_tensors"] = {
+        "ms_per_step": round(sec * 1e3, 4), "tensors": k_, "launches_per_step": 3,
+        "algorithmic_bytes": 8.5 * N_TERNGRAD, "frac_of_hbm_peak": round(8.5 * N_TERNGRAD / sec / 1e9 / HBM_PEAK_GBS, 4)}
+    del xs, ms_, ds_
+    torch.cuda.empty_cache()
+
     # ---- DGC / GradDrop top-0.1 %: 138,357,544 elements --------------------------------------
     n = N_DGC
     u = torch.rand(n, device="cuda", generator=gen) - 0.5

@@ -215,6 +215,14 @@ def test_many_tensors_each_with_several_messages(tg, oracle_cpu):
 
 # ---- the single-launch resident encode (tensor kept on chip between the two passes) ----
 @pytest.fixture
+def resident_from_2m(capi):
+    """By default only tensors of 2^23 elements and more take the resident encode; these tests want it at 2^21."""
+    old = capi.set_option("terngrad_resident_min", 1 << 21)
+    yield
+    capi.set_option("terngrad_resident_min", old)
+
+
+@pytest.fixture
 def resident_forced(capi):
     old = capi.set_option("terngrad_resident_min", 1)
     yield
@@ -275,14 +283,14 @@ def test_resident_capacity_edge(tg, oracle_cpu, b, n):
     assert_bits_equal(host(out), ref, f"message n={n} b={b}")
 
 
-def test_resident_and_tiled_tensors_in_one_call(tg, oracle_cpu):
+def test_resident_and_tiled_tensors_in_one_call(tg, oracle_cpu, resident_from_2m):
     rng = np.random.default_rng(77)
     sizes = [3_000_001, 1000, 2_500_000, 70001, 2_097_152, 2_097_151]
     xs = [rng.normal(0, 1e-2, n).astype(np.float32) for n in sizes]
     _check(tg, oracle_cpu, xs, [2, 4, 1, 8, 2, 2], [1, 0, 1, 1, 0, 1], [5, 6, 7, 8, 9, 10], [0] * len(sizes), rng)
 
 
-def test_resident_barrier_expiry_is_reported(tg, oracle_cpu, capi):
+def test_resident_barrier_expiry_is_reported(tg, oracle_cpu, capi, resident_from_2m):
     # A zero bound makes the barrier wait give up at once: every workgroup still leaves normally, the
     # next encode on that stream reports it, and the stream then uses the two-launch path.
     rng = np.random.default_rng(5)
@@ -312,7 +320,7 @@ def test_resident_barrier_expiry_is_reported(tg, oracle_cpu, capi):
         assert capi.load().hpx_release_workspaces() == 0
 
 
-def test_resident_kernel_belongs_to_one_stream(tg, oracle_cpu, capi):
+def test_resident_kernel_belongs_to_one_stream(tg, oracle_cpu, capi, resident_from_2m):
     # A second stream encoding a large tensor takes the two-launch path (same bytes out).
     rng = np.random.default_rng(6)
     x = rng.normal(0, 1e-2, 3_000_000).astype(np.float32)
