@@ -200,12 +200,49 @@ def main():
 
     del sets
     torch.cuda.empty_cache()
+    result["plain_streams"] = plain_streams(torch, capi, L, stream, n)
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(np, n, args.cpu_seconds)
     if not args.no_extra:
         result["extra"] = extra(torch, np, capi, L, stream, gen)
     print(json.dumps(result), flush=True)
+
+
+def plain_streams(torch, capi, L, stream, n):
+    """What the memory system gives the simplest kernels of the codecs' shapes (hpx_probe_stream), measured the way
+    the headline is: buffers rotate over distinct sets, HIP events on the launch stream around each kernel.  The
+    TernGrad step reads 4*n bytes once and writes 4*n bytes once, so read + write of 4*n bytes is the time below
+    which no encode+decode of this tensor can go on this part."""
+    names = {0: "read", 1: "write_streaming", 2: "write_plain", 3: "read_read_write"}
+    out = {}
+    for label, elems, nsets in (("headline_tensor", n, 6), ("440MB", 110_000_000, 3)):
+        nbytes = elems * 4 // 16384 * 16384
+        a = [torch.zeros(elems, device="cuda") for _ in range(nsets)]
+        b = torch.zeros(elems, device="cuda")
+        res = {"bytes": nbytes}
+        for kind, name in names.items():
+            i = [0]
+
+            def f():
+                i[0] += 1
+                rc = L.hpx_probe_stream(kind, a[i[0] % nsets].data_ptr(), b.data_ptr(), nbytes, stream)
+                assert rc == 0, capi.last_error()
+
+            for _ in range(2 * nsets):   # untimed: clocks up, the zero fill's dirty lines out of the caches
+                f()
+            kt = kernel_times(torch, capi, f, ["probe_stream_kernel"], reps=24)["probe_stream_kernel"]
+            traffic = nbytes * (3 if kind == 3 else 1)
+            res[name] = {"us": round(kt * 1e6, 2), "GBps": round(traffic / kt / 1e9, 1),
+                         "frac_of_hbm_peak": round(traffic / kt / 1e9 / HBM_PEAK_GBS, 4)}
+        out[label] = res
+        del a, b
+        torch.cuda.empty_cache()
+    h = out["headline_tensor"]
+    floor_us = h["read"]["us"] + min(h["write_streaming"]["us"], h["write_plain"]["us"])
+    out["headline_floor"] = {"read_plus_write_us": round(floor_us, 2),
+                             "frac_of_hbm_peak_at_that_floor": round(8.5 * n / (floor_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)}
+    return out
 
 
 def cpu_baseline(np, n, budget_s):
