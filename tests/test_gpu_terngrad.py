@@ -216,7 +216,7 @@ def test_many_tensors_each_with_several_messages(tg, oracle_cpu):
 # ---- the single-launch resident encode (tensor kept on chip between the two passes) ----
 @pytest.fixture
 def resident_from_2m(capi):
-    """By default only tensors of 2^23 elements and more take the resident encode; these tests want it at 2^21."""
+    """By default only tensors of 10 * 2^20 elements and more take the resident encode; these tests want it at 2^21."""
     old = capi.set_option("terngrad_resident_min", 1 << 21)
     yield
     capi.set_option("terngrad_resident_min", old)

@@ -161,8 +161,8 @@ size_t stream_store_max_bytes();
 enum Option {
   kOptStreamStoreMaxBytes = 0,  // "stream_store_max_bytes", default kStreamStoreMaxBytes
   kOptTerngradResidentMin,      // "terngrad_resident_min": smallest tensor (elements) that takes the
-                                // single-launch resident encode; negative = never.  Default 2^23:
-                                // below about 8 M elements the two-launch encode is faster (2.2 M: 8.6 against 15.1 us).
+                                // single-launch resident encode; negative = never.  Default 10 * 2^20:
+                                // below about 10 M elements the two-launch encode is faster (2.2 M: 8.7 against 14.9 us).
   kOptTerngradBarrierMs,        // "terngrad_barrier_ms": bound on the resident kernel's barrier wait.  Default 2000.
   kOptCount
 };

@@ -150,7 +150,7 @@ struct OptionDef {
 };
 const OptionDef kOptions[kOptCount] = {
     {"stream_store_max_bytes", "HPX_STREAM_STORE_MAX_BYTES", int64_t(kStreamStoreMaxBytes)},
-    {"terngrad_resident_min", "HPX_TERNGRAD_RESIDENT_MIN", int64_t(1) << 23},
+    {"terngrad_resident_min", "HPX_TERNGRAD_RESIDENT_MIN", int64_t(10) << 20},
     {"terngrad_barrier_ms", "HPX_TERNGRAD_BARRIER_MS", 2000},
 };
 std::atomic<int64_t> g_opt[kOptCount];
