@@ -170,10 +170,13 @@ int64_t option(Option o);
 
 // Index of the segment owning `tile`: the largest s < nseg with start[s] <= tile,
 // where start[] is the strictly increasing exclusive prefix of tiles per
-// segment.  `tile` is wave-uniform, so this runs on the scalar unit; it is
-// written as two rounds of independent loads (16 pivots, then the 16 entries
-// under the chosen pivot) so a workgroup pays two scalar-load latencies before
-// its first vector load instead of log2(CAP) dependent ones.
+// segment.  `tile` is wave-uniform and every lane of the wave must be active.
+// Each round of dependent loads from the argument table, cold at the start of
+// a launch, delays the first data load of every workgroup of the first wave
+// of workgroups by about a microsecond, so the search is ONE round: tables of
+// up to 16 entries are read whole on the scalar unit; larger ones are read by
+// the lanes (entry k by lane k % 64), and the answer is the number of entries
+// that do not exceed `tile`, counted with ballots.
 template <int CAP>
 __device__ __forceinline__ int find_segment(const int32_t (&start)[CAP + 1], int nseg, int tile) {
   if constexpr (CAP <= 16) {
@@ -182,15 +185,14 @@ __device__ __forceinline__ int find_segment(const int32_t (&start)[CAP + 1], int
     for (int k = 1; k < CAP; k++) s += (k < nseg && start[k] <= tile) ? 1 : 0;
     return s;
   } else {
-    constexpr int kStride = 16;
-    constexpr int kPivots = (CAP + kStride - 1) / kStride;
-    int blk = 0;
+    const int lane = threadIdx.x & (kWave - 1);
+    int s = 0;
 #pragma unroll
-    for (int j = 1; j < kPivots; j++) blk += (j * kStride < nseg && start[j * kStride] <= tile) ? 1 : 0;
-    const int base = blk * kStride;
-    int s = base;
-#pragma unroll
-    for (int k = 1; k < kStride; k++) s += (base + k < nseg && base + k <= CAP && start[base + k] <= tile) ? 1 : 0;
+    for (int j = 0; j < CAP; j += kWave) {
+      const int k = j + lane;
+      const int v = start[k < CAP ? k : CAP];
+      s += __popcll(__ballot(k >= 1 && k < nseg && v <= tile));
+    }
     return s;
   }
 }
