@@ -93,12 +93,14 @@ def test_terngrad_comp_decomp_root(hp, oracle_cpu, pinned):
     assert hp.error_count() == 0, hp.last_error()
 
 
-def test_tbq_batch_of_mixed_tasks(hp, oracle_cpu):
+@pytest.mark.parametrize("lo,hi,count", [(5, 70_000, 24), (2 << 20, 5 << 20, 18)])
+def test_tbq_batch_of_mixed_tasks(hp, oracle_cpu, lo, hi, count):
+    # the large case: messages of 0.5 to 1.25 MB, so the batch's transfers and codec calls are cut into several runs
     rng = np.random.default_rng(2)
     thr, size, rank = 2e-3, 4, 0
     assert hp.init("tbq", {"threshold": thr}, 0, rank, size)
     keep, checks = [], []
-    sizes = [int(s) for s in rng.integers(5, 70_000, 24)]
+    sizes = [int(s) for s in rng.integers(lo, hi, count)]
     for k, n in enumerate(sizes):
         kind = (10, 20, 30)[k % 3]
         mb = oracle_cpu.tbq_packed_size(n)
@@ -146,6 +148,37 @@ def test_tbq_batch_of_mixed_tasks(hp, oracle_cpu):
             msg = oracle_cpu.tbq_encode(want, rr, thr)
             assert_bits_equal(host(dg), want, f"{name} ROOT gradient"); assert_bits_equal(host(dr), rr, f"{name} ROOT residual")
             assert_bits_equal(Cc.numpy()[:mb], msg, f"{name} ROOT message")
+    assert hp.error_count() == 0, hp.last_error()
+
+
+def test_terngrad_batch_spanning_several_runs(hp, oracle_cpu):
+    # 10 COMP and 10 DECOMP tasks with messages of about 1 MB each, submitted in one go
+    rng = np.random.default_rng(21)
+    b, seed = 2, 9
+    assert hp.init("terngrad", {"enable_random": 1, "bitwidth": b, "seed": seed}, 0, 0, 2)
+    comp, dec, keep = [], [], []
+    for k in range(10):
+        n = int(rng.integers(3 << 20, 5 << 20))
+        mb = oracle_cpu.terngrad_packed_size(n, b)
+        x = rng.normal(0, 1e-2, n).astype(np.float32)
+        comp.append((f"c{k}", x, dev(x), torch.zeros(mb, dtype=torch.uint8, device="cuda"), _host_buf(mb, k & 1)))
+        src = rng.normal(0, 1e-2, n).astype(np.float32)
+        rc, msg = oracle_cpu.terngrad_encode(src, b, 1, 100 + k)
+        base = rng.normal(0, 1, n).astype(np.float32)
+        C = _host_buf(mb, (k + 1) & 1); C.numpy()[:] = msg
+        dec.append((f"d{k}", msg, base, dev(base), torch.zeros(mb, dtype=torch.uint8, device="cuda"), C, k % 2))
+    torch.cuda.synchronize()
+    for (cn, x, dx, B, C), (dn, msg, base, dt, Bd, Cd, add) in zip(comp, dec):
+        assert hp.submit_task(cn, dx, B, C, 0, 10)
+        assert hp.submit_task(dn, dt, Bd, Cd, add, 20)
+    _collect(hp, 10, [c[0] for c in comp])
+    _collect(hp, 20, [d[0] for d in dec])
+    for cn, x, dx, B, C in comp:
+        rc, ref = oracle_cpu.terngrad_encode(x, b, 1, seed)
+        assert_bits_equal(C.numpy(), ref, f"{cn} message in C")
+    for dn, msg, base, dt, Bd, Cd, add in dec:
+        rc, want = oracle_cpu.terngrad_decode(msg, base.size, base.copy(), add)
+        assert_bits_equal(host(dt), want, f"{dn} decoded")
     assert hp.error_count() == 0, hp.last_error()
 
 

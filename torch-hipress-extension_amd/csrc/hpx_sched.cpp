@@ -187,6 +187,12 @@ int64_t message_bytes(const Params& p, const hpx_task_t& t) {
   return t.B_bytes;        // compressed_size = t.B->numel(), hp_cuda.cpp:411, :558
 }
 
+// Message bytes per run of a batch (see run_codec_batch).  The first run is short so that the link starts
+// early (1 MB is 4 Mi elements of 2-bit codes: about 10 us of encode, 20 us on the link); each run is twice
+// as long as the one before, up to 16 MB, because every run costs its own launches and event hand-overs.
+constexpr int64_t kPipeFirstBytes = int64_t(1) << 20;
+constexpr int64_t kPipeMaxBytes = int64_t(16) << 20;
+
 struct Group {  // tasks published together once `landed` has passed
   std::vector<const Task*> tasks;
   int queue = 0;
@@ -282,35 +288,81 @@ void run_codec_batch(Worker& w, const Params& p, const std::vector<Task>& batch)
   if (!w.pinned_arena.reserve(pinned_need) || !w.device_arena.reserve(device_need)) return;
   w.next_event = 0;
 
-  // ---- messages in (data stream) ----
-  std::vector<float*> d_out;           // decode argument lists (hp_cuda.cpp:420-461)
-  std::vector<int32_t> d_out_size, d_in_size, d_add;
-  std::vector<const uint8_t*> d_in;
-  std::vector<const Task*> decomp_ok, root_ok;
-  CopyList cl_in;
-  for (const Task* t : decomp) {
-    const int64_t bytes = message_bytes(p, t->t);
-    if (bytes > t->t.C_bytes || bytes > t->t.B_bytes) { fail("scheduler: decode task '%s': message of %lld bytes does not fit B (%lld) / C (%lld)", t->name.c_str(), (long long)bytes, (long long)t->t.B_bytes, (long long)t->t.C_bytes); continue; }
-    copy_in(w, cl_in, t->t.B, t->t.C, bytes);  // t.B->copy_(t.C->slice(0,0,compressed_size,1), true)
-    d_out.push_back(t->t.tensor); d_out_size.push_back(int32_t(t->t.tensor_numel));
-    d_in.push_back(t->t.B); d_in_size.push_back(int32_t(bytes)); d_add.push_back(t->t.is_root);
-    decomp_ok.push_back(t);
-  }
-  for (const Task* t : root) {
-    const int64_t bytes = message_bytes(p, t->t);
-    const int64_t slots = int64_t(p.size) * bytes;
-    if (slots > t->t.C_bytes) { fail("scheduler: root task '%s': C holds %lld bytes, %d slots of %lld needed", t->name.c_str(), (long long)t->t.C_bytes, p.size, (long long)bytes); continue; }
-    uint8_t* tmp = w.device_arena.take(size_t(slots));  // temp_cuda_tensors_for_c, hp_cuda.cpp:149-158
-    copy_in(w, cl_in, tmp, t->t.C, slots);
-    for (int i = 0; i < p.size; i++) {
-      if (i == p.rank) continue;
-      d_out.push_back(t->t.tensor); d_out_size.push_back(int32_t(t->t.tensor_numel));
-      d_in.push_back(tmp + int64_t(i) * bytes); d_in_size.push_back(int32_t(bytes)); d_add.push_back(t->t.is_root);
+  // Transfers and codec calls are cut into runs so that the PCIe transfer of one run overlaps the kernels of
+  // the next (a 200-tensor TBQ bucket spends 2.5 times as long on the link as in its encode kernel).
+  // GradDrop messages are tiny and its encode has a large fixed cost per call, so a GradDrop batch stays
+  // one run.
+  const bool one_run = p.alg == kGraddrop;
+  auto next_run_bytes = [one_run](int64_t b) {
+    if (one_run) return INT64_MAX;
+    return b == 0 ? kPipeFirstBytes : (b * 2 < kPipeMaxBytes ? b * 2 : kPipeMaxBytes);
+  };
+
+  // ---- messages in (data stream): every run's copy is queued now, its decode later ----
+  struct DecodeRun {
+    std::vector<float*> out;           // decode argument lists (hp_cuda.cpp:420-461)
+    std::vector<int32_t> out_size, in_size, add;
+    std::vector<const uint8_t*> in;
+    std::vector<const Task*> decomp;   // the DECOMP tasks among them: published once the decode has run
+    hipEvent_t arrived = nullptr;
+    int64_t bytes = 0;
+  };
+  std::vector<DecodeRun> dec_runs;
+  std::vector<const Task*> root_ok;
+  {
+    CopyList cl_in;
+    DecodeRun run;
+    int64_t pipe_bytes = next_run_bytes(0);
+    auto close_run = [&]() {
+      if (run.out.empty()) return;
+      cl_in.issue(w);
+      run.arrived = chain(w, w.data, nullptr);
+      dec_runs.push_back(std::move(run));
+      run = DecodeRun();
+      pipe_bytes = next_run_bytes(pipe_bytes);
+    };
+    for (const Task* t : decomp) {
+      const int64_t bytes = message_bytes(p, t->t);
+      if (bytes > t->t.C_bytes || bytes > t->t.B_bytes) { fail("scheduler: decode task '%s': message of %lld bytes does not fit B (%lld) / C (%lld)", t->name.c_str(), (long long)bytes, (long long)t->t.B_bytes, (long long)t->t.C_bytes); continue; }
+      copy_in(w, cl_in, t->t.B, t->t.C, bytes);  // t.B->copy_(t.C->slice(0,0,compressed_size,1), true)
+      run.out.push_back(t->t.tensor); run.out_size.push_back(int32_t(t->t.tensor_numel));
+      run.in.push_back(t->t.B); run.in_size.push_back(int32_t(bytes)); run.add.push_back(t->t.is_root);
+      run.decomp.push_back(t);
+      run.bytes += bytes;
+      if (run.bytes >= pipe_bytes) close_run();
     }
-    root_ok.push_back(t);
+    for (const Task* t : root) {
+      const int64_t bytes = message_bytes(p, t->t);
+      const int64_t slots = int64_t(p.size) * bytes;
+      if (slots > t->t.C_bytes) { fail("scheduler: root task '%s': C holds %lld bytes, %d slots of %lld needed", t->name.c_str(), (long long)t->t.C_bytes, p.size, (long long)bytes); continue; }
+      uint8_t* tmp = w.device_arena.take(size_t(slots));  // temp_cuda_tensors_for_c, hp_cuda.cpp:149-158
+      copy_in(w, cl_in, tmp, t->t.C, slots);
+      for (int i = 0; i < p.size; i++) {
+        if (i == p.rank) continue;
+        run.out.push_back(t->t.tensor); run.out_size.push_back(int32_t(t->t.tensor_numel));
+        run.in.push_back(tmp + int64_t(i) * bytes); run.in_size.push_back(int32_t(bytes)); run.add.push_back(t->t.is_root);
+      }
+      root_ok.push_back(t);
+      run.bytes += slots;
+      if (run.bytes >= pipe_bytes) close_run();  // all slots of a tensor stay in one run: one fused pass over it
+    }
+    close_run();
   }
-  cl_in.issue(w);
-  chain(w, w.data, w.compute);
+  root = root_ok;
+
+  // Groups in the order they were queued; names go out as their events pass.
+  std::deque<Group> sent;
+  size_t next_pub = 0;
+  auto publish_landed = [&](bool wait) {
+    for (; next_pub < sent.size(); next_pub++) {
+      Group& grp = sent[next_pub];
+      if (!wait && grp.landed && hipEventQuery(grp.landed) != hipSuccess) {
+        (void)hipGetLastError();  // "not ready" must not be taken for a failed launch later on
+        return;
+      }
+      publish(grp);
+    }
+  };
 
   // ---- compute ----
   auto encode = [&](const std::vector<const Task*>& ts, const char* what) {
@@ -340,52 +392,71 @@ void run_codec_batch(Worker& w, const Params& p, const std::vector<Task>& batch)
     }
   };
   auto decode = [&]() {
-    if (d_out.empty()) return;
-    const int n = int(d_out.size());
-    if (p.alg == kTerngrad) {
-      codec(hpx_terngrad_decode(n, d_out.data(), d_out_size.data(), d_in.data(), d_in_size.data(), d_add.data(), w.compute), "hp_cuda_terngradr");
-    } else if (p.alg == kTbq) {
-      std::vector<float> thr(n, p.threshold);
-      codec(hpx_tbq_decode(n, d_out.data(), d_out_size.data(), d_in.data(), thr.data(), d_add.data(), w.compute), "hp_cuda_tbqr");
-    } else {
-      codec(hpx_gd_decode(n, d_in.data(), d_in_size.data(), d_out.data(), d_out_size.data(), d_add.data(), w.compute), "hp_cuda_gdr");
+    for (DecodeRun& r : dec_runs) {
+      if (r.arrived) SCHED_HIP(hipStreamWaitEvent(w.compute, r.arrived, 0));
+      const int n = int(r.out.size());
+      if (p.alg == kTerngrad) {
+        codec(hpx_terngrad_decode(n, r.out.data(), r.out_size.data(), r.in.data(), r.in_size.data(), r.add.data(), w.compute), "hp_cuda_terngradr");
+      } else if (p.alg == kTbq) {
+        std::vector<float> thr(n, p.threshold);
+        codec(hpx_tbq_decode(n, r.out.data(), r.out_size.data(), r.in.data(), thr.data(), r.add.data(), w.compute), "hp_cuda_tbqr");
+      } else {
+        codec(hpx_gd_decode(n, r.in.data(), r.in_size.data(), r.out.data(), r.out_size.data(), r.add.data(), w.compute), "hp_cuda_gdr");
+      }
+      if (!r.decomp.empty()) {
+        sent.emplace_back();
+        Group& grp = sent.back();
+        grp.queue = 1;
+        grp.tasks = std::move(r.decomp);
+        grp.landed = chain(w, w.compute, nullptr);
+      }
+      publish_landed(false);
     }
   };
-  auto messages_out = [&](Group& grp) {  // t.C->slice(0,0,compressed_size,1).copy_(*(t.B))
-    if (grp.tasks.empty()) return;
-    chain(w, w.compute, w.data);
-    CopyList cl;
-    for (const Task* t : grp.tasks) copy_out(w, cl, grp, t->t, message_bytes(p, t->t));
-    cl.issue(w);
-    grp.landed = chain(w, w.data, nullptr);
+  // Encodes `ts` run by run; each run's messages go out behind it:
+  // t.C->slice(0,0,compressed_size,1).copy_(*(t.B)).
+  auto encode_and_send = [&](const std::vector<const Task*>& ts, const char* what) {
+    size_t i = 0;
+    int64_t pipe_bytes = 0;
+    while (i < ts.size()) {
+      std::vector<const Task*> run;
+      int64_t bytes = 0;
+      pipe_bytes = next_run_bytes(pipe_bytes);
+      while (i < ts.size() && bytes < pipe_bytes) {
+        bytes += message_bytes(p, ts[i]->t);
+        run.push_back(ts[i++]);
+      }
+      encode(run, what);
+      chain(w, w.compute, w.data);
+      CopyList cl;
+      const size_t first_group = sent.size();
+      for (const Task* t : run) {
+        const int q = queue_of(t->t.task_id);
+        if (sent.size() == first_group || sent.back().queue != q) {
+          sent.emplace_back();
+          sent.back().queue = q;
+        }
+        sent.back().tasks.push_back(t);
+        copy_out(w, cl, sent.back(), t->t, message_bytes(p, t->t));
+      }
+      cl.issue(w);
+      hipEvent_t landed = chain(w, w.data, nullptr);
+      for (size_t k = first_group; k < sent.size(); k++) sent[k].landed = landed;
+      publish_landed(false);
+    }
   };
 
-  Group g_comp, g_root, g_dec;
-  g_comp.queue = 0; g_dec.queue = 1; g_root.queue = 2;
-  g_comp.tasks = comp; g_root.tasks = root_ok; g_dec.tasks = decomp_ok;
-  root = root_ok;
   if (p.alg == kTerngrad) {
-    encode(comp, "hp_cuda_terngrad");
-    messages_out(g_comp);
+    encode_and_send(comp, "hp_cuda_terngrad");
     decode();
-    encode(root, "hp_cuda_terngrad");
-    messages_out(g_root);
-    g_dec.landed = chain(w, w.compute, nullptr);
-    publish(g_comp);
-    publish(g_root);
-    publish(g_dec);
+    encode_and_send(root, "hp_cuda_terngrad");
   } else {
     decode();
-    g_dec.landed = chain(w, w.compute, nullptr);
-    std::vector<const Task*> both = comp;
-    both.insert(both.end(), root.begin(), root.end());
-    encode(both, p.alg == kTbq ? "hp_cuda_tbq" : "hp_cuda_gd");
-    messages_out(g_root);   // root first, then comp (hp_cuda.cpp:304-314, :614-622)
-    messages_out(g_comp);
-    publish(g_dec);
-    publish(g_root);
-    publish(g_comp);
+    std::vector<const Task*> both = root;  // root first, then comp (hp_cuda.cpp:304-314, :614-622)
+    both.insert(both.end(), comp.begin(), comp.end());
+    encode_and_send(both, p.alg == kTbq ? "hp_cuda_tbq" : "hp_cuda_gd");
   }
+  publish_landed(true);
 }
 
 // ---- PowerSGD --------------------------------------------------------------------
