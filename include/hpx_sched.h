@@ -17,12 +17,14 @@
  * gathered slot but their own rank's and then re-encoding.
  * What is different: one worker thread that sleeps on a condition variable
  * (the reference polls five queues every 500 us, one for TBQ); staging copies
- * run on a data stream ordered against the compute stream by events, all
- * messages of a phase in ONE kernel launch that reads or writes the pinned host
- * buffers directly (through a pinned bounce buffer when the caller's host tensor
- * is pageable) instead of one copy call per message; a name is
- * published once its own copy has landed rather than at fixed points of the
- * batch; HIP errors are counted and kept (hpx_sched_error) instead of ignored;
+ * run on a data stream ordered against the compute stream by events; a batch's
+ * transfers and codec calls are cut into runs (1 MB of messages, then 2, 4 ...
+ * 16 MB; GradDrop: one run) so that one run's transfer overlaps the next run's
+ * kernels, all messages of a run in ONE kernel launch that reads or writes the
+ * pinned host buffers directly (through a pinned bounce buffer when the caller's
+ * host tensor is pageable) instead of one copy call per message; a name is
+ * published once its own run's copy has landed rather than at fixed points of
+ * the batch; HIP errors are counted and kept (hpx_sched_error) instead of ignored;
  * a task whose buffers are too small for its message is skipped and counted as
  * a failure (the reference overruns them), and its name is still published.
  */

@@ -4,14 +4,16 @@
 // One worker thread owns a compute stream and a data stream.  It sleeps on a
 // condition variable, takes everything that is queued as one batch (like
 // TaskQueue::GetTasksFromQueue, hp_cuda.cpp:122-133) and turns the batch into a
-// few multi-tensor codec calls:
+// few multi-tensor codec calls.  Transfers and codec calls are cut into runs of
+// growing size (1 MB of messages, then 2, 4 ... 16 MB) so that the link and the
+// kernels work at the same time:
 //
-//   data stream     H2D of every message to decode  ── e_in ─┐
-//   compute stream  (waits e_in) group 1 ── e_1 ── group 2 ── e_2 ── ...
-//   data stream     (waits e_k) D2H of group k's messages ── d_k
-//   worker          waits d_k, finishes pageable copies, publishes group k
+//   data stream     H2D run 1 ── a_1 ── H2D run 2 ── a_2 ...      D2H run 1 ── d_1 ── D2H run 2 ── d_2 ...
+//   compute stream  (waits a_1) decode run 1, (waits a_2) decode run 2 ... encode run 1 ── e_1 ── encode run 2 ── e_2 ...
+//                                                                  (D2H run k waits e_k)
+//   worker          between runs, and at the end: publishes every run whose event has passed
 //
-// A transfer phase is one launch of the range-copy kernel over all its messages (the GPU reads or
+// A transfer run is one launch of the range-copy kernel over all its messages (the GPU reads or
 // writes the pinned host buffers itself): with a copy call per message the host spent longer
 // issuing 200 copies than the copies and the encode take together.
 //
