@@ -262,13 +262,15 @@ def cpu_baseline(np, n, budget_s):
     one()
     one()
     t0 = time.perf_counter()
-    reps = 0
+    reps, laps = 0, []
     while reps < 3 or (time.perf_counter() - t0 < budget_s and reps < 200):
+        t1 = time.perf_counter()
         one()
+        laps.append(time.perf_counter() - t1)
         reps += 1
-    sec = (time.perf_counter() - t0) / reps
+    sec = float(np.median(laps))
     res = {"value": round(4.0 * n / sec / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
-           "sample": f"{reps} full encode+decode passes of the same {n}-element workload, OpenMP over {threads} threads "
+           "sample": f"median of {reps} full encode+decode passes of the same {n}-element workload, OpenMP over {threads} threads "
                      f"(os.cpu_count()={os.cpu_count()})", "ms_per_step": round(sec * 1e3, 2)}
     # the same port on one thread
     cpu.set_threads(1)
@@ -291,15 +293,17 @@ def cpu_baseline(np, n, budget_s):
 
         ref_one()
         t0 = time.perf_counter()
-        r_reps = 0
-        while r_reps < 3 or (time.perf_counter() - t0 < budget_s / 2 and r_reps < 100):
+        r_reps, laps = 0, []
+        while r_reps < 3 or (time.perf_counter() - t0 < budget_s / 2 and r_reps < 200):
+            t1 = time.perf_counter()
             ref_one()
+            laps.append(time.perf_counter() - t1)
             r_reps += 1
-        rsec = (time.perf_counter() - t0) / r_reps
+        rsec = float(np.median(laps))
         # the reference's own code is the baseline proper; the port's figures stay beside it
         port = {k: res[k] for k in ("value", "ms_per_step", "one_thread", "sample")}
         res = {"value": round(4.0 * n / rsec / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "reference",
-               "sample": f"{r_reps} full encode+decode passes of the same {n}-element workload through the reference's "
+               "sample": f"median of {r_reps} full encode+decode passes of the same {n}-element workload through the reference's "
                          f"terngrad_body / terngrad_r_body compiled for the host, thrust::omp::par over {threads} threads "
                          f"(clock-seeded; os.cpu_count()={os.cpu_count()}); the bodies' memcpy/sync policy shim is the "
                          "harness's own, all arithmetic and Thrust calls are the reference's",
