@@ -407,9 +407,13 @@ def extra(torch, np, capi, L, stream, gen):
         dec()
 
     sec = timed(torch, r50_step, 50, 10)
+    L.hpx_set_option(b"terngrad_resident_bucket", 0)          # the same call as a min/max launch and a quantise launch
+    sec_tiled = timed(torch, r50_step, 50, 10)
+    L.hpx_set_option(b"terngrad_resident_bucket", 1)
     res["terngrad_resnet50_161_tensors"] = {
-        "ms_per_step": round(sec * 1e3, 4), "tensors": k_, "launches_per_step": 3,
-        "algorithmic_bytes": 8.5 * N_TERNGRAD, "frac_of_hbm_peak": round(8.5 * N_TERNGRAD / sec / 1e9 / HBM_PEAK_GBS, 4)}
+        "ms_per_step": round(sec * 1e3, 4), "tensors": k_, "launches_per_step": 2,
+        "algorithmic_bytes": 8.5 * N_TERNGRAD, "frac_of_hbm_peak": round(8.5 * N_TERNGRAD / sec / 1e9 / HBM_PEAK_GBS, 4),
+        "ms_per_step_with_the_two_launch_encode": round(sec_tiled * 1e3, 4)}
     del xs, ms_, ds_
     torch.cuda.empty_cache()
 

@@ -64,6 +64,11 @@ int hpx_release_workspaces(void);
  *                             negative: never)
  *   "terngrad_barrier_ms"     bound on that kernel's grid-barrier wait
  *                             (default 2000)
+ *   "terngrad_resident_bucket" 1 (default): a call with 2 to 192 tensors of one
+ *                             bit width and rounding mode that add up to at
+ *                             least terngrad_resident_min elements and fit the
+ *                             chip together takes ONE resident launch for all of
+ *                             them; 0: each tensor is looked at on its own
  * Unknown names return HPX_ERR_ARG. */
 int hpx_set_option(const char* name, int64_t value);
 int hpx_get_option(const char* name, int64_t* value);

@@ -216,17 +216,22 @@ def test_many_tensors_each_with_several_messages(tg, oracle_cpu):
 # ---- the single-launch resident encode (tensor kept on chip between the two passes) ----
 @pytest.fixture
 def resident_from_2m(capi):
-    """By default only tensors of 10 * 2^20 elements and more take the resident encode; these tests want it at 2^21."""
+    """By default only tensors of 10 * 2^20 elements and more take the resident encode; these tests want it at 2^21
+    (and every tensor looked at on its own: the one-launch encode of a whole call has its own tests below)."""
     old = capi.set_option("terngrad_resident_min", 1 << 21)
+    old_b = capi.set_option("terngrad_resident_bucket", 0)
     yield
     capi.set_option("terngrad_resident_min", old)
+    capi.set_option("terngrad_resident_bucket", old_b)
 
 
 @pytest.fixture
 def resident_forced(capi):
     old = capi.set_option("terngrad_resident_min", 1)
+    old_b = capi.set_option("terngrad_resident_bucket", 0)
     yield
     capi.set_option("terngrad_resident_min", old)
+    capi.set_option("terngrad_resident_bucket", old_b)
 
 
 @pytest.mark.parametrize("b", [1, 2, 4, 8])
@@ -341,6 +346,89 @@ def test_resident_kernel_belongs_to_one_stream(tg, oracle_cpu, capi, resident_fr
         L.hpx_profile_enable(0); L.hpx_profile_reset()
     assert_bits_equal(host(out0), ref, "owning stream")
     assert_bits_equal(host(out1), ref, "second stream")
+
+
+# ---- the resident encode of a whole call (several tensors in one launch) ----
+@pytest.fixture
+def bucket_forced(capi):
+    """Every call with two or more tensors of one width and rounding mode takes the one-launch encode."""
+    old = capi.set_option("terngrad_resident_min", 1)
+    old_b = capi.set_option("terngrad_resident_bucket", 1)
+    L = capi.load()
+    L.hpx_profile_reset(); L.hpx_profile_enable(1)
+    yield
+    L.hpx_profile_enable(0); L.hpx_profile_reset()
+    capi.set_option("terngrad_resident_min", old)
+    capi.set_option("terngrad_resident_bucket", old_b)
+
+
+def _bucket_launches(capi):
+    return capi.profile_query("terngrad_resident_multi_kernel")[1]
+
+
+@pytest.mark.parametrize("b", [1, 2, 4, 8])
+@pytest.mark.parametrize("rnd", [0, 1])
+def test_resident_bucket_sizes_and_tails(tg, oracle_cpu, capi, bucket_forced, b, rnd):
+    rng = np.random.default_rng(1900 + 10 * b + rnd)
+    unit = max(4, 8 // b)
+    sizes = [1, 2, 3, 5, 7, 8, 9, 17, unit * 64 - 1, unit * 64, unit * 64 + 1, 4097, 300007, 64, 256, 2048, 70001, 1_000_003]
+    xs = [rng.normal(0, 1e-2, n).astype(np.float32) for n in sizes]
+    seeds = [int(s) for s in rng.integers(0, 2**63, len(sizes))]
+    before = _bucket_launches(capi)
+    _check(tg, oracle_cpu, xs, [b] * len(sizes), [rnd] * len(sizes), seeds, [i & 1 for i in range(len(sizes))], rng)
+    assert _bucket_launches(capi) == before + 1
+
+
+def test_resident_bucket_zero_extremes_and_constants(tg, oracle_cpu, capi, bucket_forced):
+    rng = np.random.default_rng(31)
+    far = np.full(1_300_000, 0.5, np.float32); far[1_200_001] = -0.0; far[1_250_000] = 0.0   # first zero many pieces in
+    neg = np.full(2_100_001, -0.25, np.float32); neg[5] = 0.0; neg[2_000_000] = -0.0
+    xs = [np.zeros(1000, np.float32), np.full(1003, -0.0, np.float32), np.full(4097, 0.125, np.float32),
+          np.array([0.5, -0.0, 0.0, 0.25, 0.0], np.float32), np.array([-0.5, 0.0, -0.0, -0.25], np.float32),
+          np.array([1e-45, 0, 3e-45, 2e-45] * 50, np.float32), far, neg]
+    for b in (1, 2, 8):
+        for rnd in (0, 1):
+            before = _bucket_launches(capi)
+            _check(tg, oracle_cpu, xs, [b] * len(xs), [rnd] * len(xs), [77] * len(xs), [0] * len(xs), rng)
+            assert _bucket_launches(capi) == before + 1
+
+
+def test_resident_bucket_many_rows_and_full_table(tg, oracle_cpu, capi, bucket_forced):
+    # 192 tensors (a full table) that need LDS rows as well: about 27 M elements
+    rng = np.random.default_rng(32)
+    sizes = [int(s) for s in rng.integers(1, 2000, 150)] + [int(s) for s in rng.integers(500_000, 800_000, 41)] + [27_000_000 - 41 * 650_000]
+    assert len(sizes) == 192
+    xs = [rng.normal(0, 1e-2, n).astype(np.float32) for n in sizes]
+    dx = [dev(x) for x in xs]
+    seeds = [int(s) for s in rng.integers(0, 2**64 - 1, len(sizes), dtype=np.uint64)]
+    before = _bucket_launches(capi)
+    outs = tg.encode(dx, [2] * len(xs), [1] * len(xs), seeds)
+    torch.cuda.synchronize()
+    assert _bucket_launches(capi) == before + 1
+    for i, x in enumerate(xs):
+        rc, ref = oracle_cpu.terngrad_encode(x, 2, 1, seeds[i])
+        assert rc == 0
+        assert_bits_equal(host(outs[i]), ref, f"message[{i}] n={x.size}")
+
+
+def test_resident_bucket_falls_back(tg, oracle_cpu, capi, bucket_forced):
+    rng = np.random.default_rng(33)
+    xs = [rng.normal(0, 1e-2, n).astype(np.float32) for n in (5000, 70001, 1234)]
+    before = _bucket_launches(capi)
+    # mixed widths or rounding modes: every tensor on its own
+    _check(tg, oracle_cpu, xs, [2, 4, 2], [1, 1, 1], [1, 2, 3], [0, 0, 0], rng)
+    _check(tg, oracle_cpu, xs, [2, 2, 2], [1, 0, 1], [1, 2, 3], [0, 0, 0], rng)
+    # more tensors than one table holds
+    many = [rng.normal(0, 1e-2, 300).astype(np.float32) for _ in range(193)]
+    _check(tg, oracle_cpu, many, [2] * 193, [1] * 193, list(range(193)), [0] * 193, rng)
+    assert _bucket_launches(capi) == before
+    # below the threshold
+    capi.set_option("terngrad_resident_min", 1 << 20)
+    _check(tg, oracle_cpu, xs, [2, 2, 2], [1, 1, 1], [1, 2, 3], [0, 0, 0], rng)
+    assert _bucket_launches(capi) == before
+    capi.set_option("terngrad_resident_min", 1)
+    _check(tg, oracle_cpu, xs, [2, 2, 2], [1, 1, 1], [1, 2, 3], [0, 0, 0], rng)
+    assert _bucket_launches(capi) == before + 1
 
 
 def test_random_sweep_of_calls(tg, oracle_cpu, capi):

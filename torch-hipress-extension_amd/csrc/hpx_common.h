@@ -164,6 +164,8 @@ enum Option {
                                 // single-launch resident encode; negative = never.  Default 10 * 2^20:
                                 // below about 10 M elements the two-launch encode is faster (2.2 M: 8.7 against 14.9 us).
   kOptTerngradBarrierMs,        // "terngrad_barrier_ms": bound on the resident kernel's barrier wait.  Default 2000.
+  kOptTerngradResidentBucket,   // "terngrad_resident_bucket": 1 = a call with several tensors that fit the chip together
+                                // and add up to terngrad_resident_min elements takes ONE resident launch.  Default 1.
   kOptCount
 };
 int64_t option(Option o);

@@ -680,6 +680,238 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
   }
 }
 
+// ---- resident encode of a bucket -------------------------------------------------
+// The same idea for a call with several tensors whose sum fits the chip: ONE launch
+// reads every tensor once.  The unit of work is a piece: `rows` rows of 64 units of
+// one tensor, held by one wave (register rows first, LDS rows after them), so the
+// tensor, its extremes and its seed are wave-uniform and the inner loops are those
+// of the single-tensor kernel.  Piece p belongs to wave p % 16 of workgroup p / 16;
+// the host picks the smallest `rows` for which all pieces fit (every tensor has at
+// least one piece; the piece that ends a tensor also takes the 1..UNIT-1 elements
+// behind its last whole unit).
+//
+// The extremes travel through the epoch-tagged slots of the tiled kernels: a wave
+// folds its piece into way (piece index % kSlotWays) of its tensor's three slots with
+// atomic max operations whose results it waits for, the grid meets at the barrier of
+// grid_exchange (its payload unused), and every wave then folds the ways of its
+// tensor.
+struct ResMultiArgs {
+  int32_t nseg;
+  int32_t piece_start[kCapLarge + 1];
+  EncSeg seg[kCapLarge];
+  uint64_t* slots;
+  uint32_t epoch;
+  uint32_t rows;       // rows of 64 units per piece
+  uint32_t lds_rows;   // rows beyond the register rows, kept in LDS
+  uint32_t gen;
+  uint64_t* bar;
+  uint32_t* host_flag;
+  uint64_t spin_limit;
+};
+static_assert(sizeof(ResMultiArgs) <= 9600, "kernel-argument budget");
+
+template <int B, bool RANDOM, int PRE>
+__global__ __launch_bounds__(kResThreads) void terngrad_resident_multi_kernel(const ResMultiArgs a) {
+  constexpr int DPB = 8 / B;
+  constexpr int UNIT = DPB > 4 ? DPB : 4;
+  constexpr int H = UNIT / 4;
+  constexpr int BPU = UNIT / DPB;
+  constexpr int KU = res_reg_groups(B, RANDOM) / H;  // unit rows held in registers
+  constexpr int kWaves = kResThreads / kWave;
+  constexpr uint32_t stride_bytes = uint32_t(kWave) * BPU;
+  extern __shared__ float4 s_rows[];  // [wave][lds_rows][H][64], then the prepared draws [wave][PRE][H][64]
+  __shared__ uint32_t s_ok;
+
+  const uint32_t wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  const int total = a.piece_start[a.nseg];
+  const int my_piece = int(blockIdx.x) * kWaves + int(wave);
+  const bool active = my_piece < total;           // wave-uniform
+  const int piece = active ? my_piece : total - 1;  // an idle wave looks at the last piece and touches nothing
+  const int s = __builtin_amdgcn_readfirstlane(find_segment<kCapLarge>(a.piece_start, a.nseg, piece));
+  const EncSeg& sg = a.seg[s];
+  const float* __restrict__ xp = sg.x;
+  const uint32_t n = static_cast<uint32_t>(sg.n);
+  const uint32_t full_units = n / UNIT;
+  const uint32_t pl = uint32_t(piece - a.piece_start[s]);
+  const uint32_t npieces = uint32_t(a.piece_start[s + 1] - a.piece_start[s]);
+  const uint32_t u_beg = pl * a.rows * kWave;
+  const uint32_t u_lim = u_beg + a.rows * kWave;
+  const uint32_t u_end = !active ? 0u : (u_lim < full_units ? u_lim : full_units);
+  const bool ends_tensor = active && pl == npieces - 1;
+  const uint32_t u0 = u_beg + lane;
+  const float qnan = __builtin_nanf("");  // compares false both ways: ignored by min and max
+  float4* s_mine = s_rows + size_t(wave) * a.lds_rows * H * kWave;
+  float4* s_pre = s_rows + size_t(kWaves) * a.lds_rows * H * kWave + size_t(wave) * PRE * H * kWave;
+
+  // ---- pass 1: load the piece, reduce ---------------------------------------------
+  float4 v[KU][H];
+  if (u_beg + uint32_t(KU * kWave) <= u_end) {
+#pragma unroll
+    for (int k = 0; k < KU; k++)
+#pragma unroll
+      for (int h = 0; h < H; h++) v[k][h] = ld4_stream(xp + size_t(u0 + k * kWave) * UNIT + h * 4);
+  } else {
+#pragma unroll
+    for (int k = 0; k < KU; k++) {
+      const uint32_t u = u0 + k * kWave;
+#pragma unroll
+      for (int h = 0; h < H; h++)
+        v[k][h] = u < u_end ? ld4_stream(xp + size_t(u) * UNIT + h * 4) : make_float4(qnan, qnan, qnan, qnan);
+    }
+  }
+  if (RANDOM && PRE > 0) {  // random addends of the first PRE rows, while the loads are in flight
+    uint32_t d[UNIT];
+    const uint32_t x0 = sg.seed + u0 * BPU;
+#pragma unroll
+    for (int q = 0; q < UNIT; q++) {
+      const int jb = q / DPB, j = q % DPB;
+      d[q] = lcg_mul(j + 2) * (x0 + jb) + lcg_add(j + 2);
+    }
+    for (uint32_t k = 0; k < uint32_t(PRE); k++) {
+#pragma unroll
+      for (int h = 0; h < H; h++)
+        s_pre[(k * H + h) * kWave + lane] =
+            make_float4(u01_scaled(d[4 * h]), u01_scaled(d[4 * h + 1]), u01_scaled(d[4 * h + 2]), u01_scaled(d[4 * h + 3]));
+#pragma unroll
+      for (int q = 0; q < UNIT; q++) d[q] += lcg_mul(q % DPB + 2) * stride_bytes;
+    }
+  }
+  float mn = __builtin_inff(), mx = -__builtin_inff();
+  uint32_t fz = 0xFFFFFFFFu;
+  for (uint32_t r = 0; r < a.lds_rows; r++) {
+    const uint32_t u = u0 + (uint32_t(KU) + r) * kWave;
+#pragma unroll
+    for (int h = 0; h < H; h++) {
+      const float4 f = u < u_end ? ld4_stream(xp + size_t(u) * UNIT + h * 4) : make_float4(qnan, qnan, qnan, qnan);
+      s_mine[(r * H + h) * kWave + lane] = f;
+      acc_zero4(f, u * UNIT + h * 4, mn, mx, fz);
+    }
+  }
+  float am = __builtin_inff();
+#pragma unroll
+  for (int k = 0; k < KU; k++)
+#pragma unroll
+    for (int h = 0; h < H; h++) {
+      acc3(v[k][h].x, mn, mx, am); acc3(v[k][h].y, mn, mx, am);
+      acc3(v[k][h].z, mn, mx, am); acc3(v[k][h].w, mn, mx, am);
+    }
+  if (am == 0.0f) {
+    float d0 = 0.f, d1 = 0.f;
+#pragma unroll
+    for (int k = 0; k < KU; k++)
+#pragma unroll
+      for (int h = 0; h < H; h++) acc_zero4(v[k][h], (u0 + k * kWave) * UNIT + h * 4, d0, d1, fz);
+  }
+  if (ends_tensor && lane == 0)
+    for (uint32_t e = full_units * UNIT; e < n; e++) acc_zero(xp[e], e, mn, mx, fz);
+  mn = wave_min(mn);
+  mx = wave_max(mx);
+  fz = wave_min_u32(fz);
+  const uint32_t ways = npieces < uint32_t(kSlotWays) ? npieces : uint32_t(kSlotWays);
+  unsigned long long* sl = reinterpret_cast<unsigned long long*>(a.slots) + size_t(s) * kSlotsPerTensor;
+  if (active && lane < 3) {
+    // lane 0: key of the maximum; lane 1: complemented key of the minimum; lane 2: complemented index
+    // of the first zero, 0 for none.  An active piece is never empty.
+    const uint32_t key = lane == 0 ? okey(mx) : lane == 1 ? ~okey(mn) : (fz != 0xFFFFFFFFu ? 0xFFFFFFFEu - fz : 0u);
+    const unsigned long long word = (static_cast<unsigned long long>(a.epoch) << 32) | key;
+    const unsigned long long old =
+        __hip_atomic_fetch_max(sl + lane * kSlotWays + (pl % kSlotWays), word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // The barrier below must not be entered before the slot holds this piece: wait for the result.
+    __asm__ volatile("" ::"v"(old));
+  }
+  __syncthreads();
+  if (threadIdx.x < kWave) {
+    uint32_t key = 0u;
+    const bool ok = grid_exchange(a.bar, a.gen, a.spin_limit, key);
+    if (threadIdx.x == 0) {
+      if (!ok) __hip_atomic_store(a.host_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      s_ok = ok ? 1u : 0u;
+    }
+  }
+  __syncthreads();
+  if (s_ok == 0u || !active) return;
+
+  // ---- pass 2: the tensor's extremes, then quantise from registers ----------------
+  {
+    uint32_t kx = 0u, kn = 0u, kz = 0u;
+    for (uint32_t w = lane; w < ways; w += kWave) {
+      const unsigned long long vx = __hip_atomic_load(sl + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const unsigned long long vn = __hip_atomic_load(sl + kSlotWays + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const unsigned long long vz = __hip_atomic_load(sl + 2 * kSlotWays + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const uint32_t x1 = (uint32_t(vx >> 32) == a.epoch) ? uint32_t(vx) : 0u;
+      const uint32_t n1 = (uint32_t(vn >> 32) == a.epoch) ? uint32_t(vn) : 0u;
+      const uint32_t z1 = (uint32_t(vz >> 32) == a.epoch) ? uint32_t(vz) : 0u;
+      kx = x1 > kx ? x1 : kx;
+      kn = n1 > kn ? n1 : kn;
+      kz = z1 > kz ? z1 : kz;
+    }
+    kx = wave_max_u32(kx);
+    kn = wave_max_u32(kn);
+    kz = wave_max_u32(kz);
+    mx = from_okey(kx);
+    mn = from_okey(~kn);
+    if ((mn == 0.0f || mx == 0.0f) && kz != 0u) {
+      // thrust::minmax_element returns the first extreme: a zero extreme carries the
+      // sign of the first zero of the tensor.
+      const float zv = xp[0xFFFFFFFEu - kz];
+      if (mn == 0.0f) mn = zv;
+      if (mx == 0.0f) mx = zv;
+    }
+  }
+  const float gi = inverse_gap(mn, mx, B);
+  if (pl == 0 && lane == 0) write_header(sg.out, B, n, mn, mx);
+
+  uint8_t* __restrict__ pay = sg.out + 10;
+  uint32_t draw[UNIT];
+  if (RANDOM) {
+    const uint32_t x0 = sg.seed + u0 * BPU + uint32_t(PRE) * stride_bytes;  // first row that draws for itself
+#pragma unroll
+    for (int q = 0; q < UNIT; q++) {
+      const int jb = q / DPB, j = q % DPB;
+      draw[q] = lcg_mul(j + 2) * (x0 + jb) + lcg_add(j + 2);
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < KU; k++) {
+    const uint32_t u = u0 + k * kWave;
+    uint32_t packed;
+    if (RANDOM && k < PRE) {
+      float4 sc[H];
+#pragma unroll
+      for (int h = 0; h < H; h++) sc[h] = s_pre[(k * H + h) * kWave + lane];
+      packed = quant_unit_prepared<B>(v[k], sc, mn, gi);
+    } else {
+      packed = quant_unit<B, RANDOM>(v[k], mn, gi, draw, stride_bytes);
+    }
+    if (u < u_end) {
+#pragma unroll
+      for (int jb = 0; jb < BPU; jb++) pay[size_t(u) * BPU + jb] = uint8_t(packed >> (8 * jb));
+    }
+  }
+  // The LDS rows follow the register rows of the same wave, so the draws simply go on.
+  for (uint32_t r = 0; r < a.lds_rows; r++) {
+    const uint32_t u = u0 + (uint32_t(KU) + r) * kWave;
+    float4 f[H];
+#pragma unroll
+    for (int h = 0; h < H; h++) f[h] = s_mine[(r * H + h) * kWave + lane];
+    const uint32_t packed = quant_unit<B, RANDOM>(f, mn, gi, draw, stride_bytes);
+    if (u < u_end) {
+#pragma unroll
+      for (int jb = 0; jb < BPU; jb++) pay[size_t(u) * BPU + jb] = uint8_t(packed >> (8 * jb));
+    }
+  }
+  // The unit that holds the end of the tensor, if its length is not a whole number of units.
+  if (ends_tensor && lane == 0 && full_units * UNIT < n) {
+    uint32_t d[UNIT];
+#pragma unroll
+    for (int q = 0; q < UNIT; q++) {
+      const int jb = q / DPB, j = q % DPB;
+      d[q] = lcg_mul(j + 2) * (sg.seed + full_units * BPU + jb) + lcg_add(j + 2);
+    }
+    quant_unit_ragged<B, RANDOM>(sg, mn, gi, full_units, d);
+  }
+}
+
 // The 4*B bits holding the codes of the 4-element group that starts at element e.
 template <int B>
 __device__ __forceinline__ uint32_t group_bits(const uint8_t* __restrict__ pay, size_t e) {
@@ -1039,6 +1271,91 @@ int launch_resident_bits(const ResArgs& ra, int num_cus, hipStream_t st) {
   return launch_resident_as<B, true, 0>(ra, num_cus, st);
 }
 
+// Rows per piece for a call with several tensors, or false when the call does not qualify: one bit
+// width and rounding mode, a total of at least the resident threshold, and all pieces on the chip at once.
+bool resident_multi_plan(int count, const int32_t* in_sizes, const uint8_t* bitwidths, const int32_t* enable_randoms,
+                         const hpx::Workspace* ws, ResMultiArgs& ma, uint32_t& pre_rows) {
+  const int64_t min_elems = hpx::option(hpx::kOptTerngradResidentMin);
+  if (min_elems < 0 || hpx::option(hpx::kOptTerngradResidentBucket) == 0) return false;
+  if (count < 2 || count > kCapLarge || ws->num_cus <= 0 || ws->num_cus > kBarMaxWorkgroups) return false;
+  const int bits = bitwidths[0];
+  const bool random = enable_randoms[0] != 0;
+  int64_t total = 0;
+  for (int i = 0; i < count; i++) {
+    if (bitwidths[i] != bits || (enable_randoms[i] != 0) != random) return false;
+    total += in_sizes[i];
+  }
+  if (total < min_elems) return false;
+  const int unit = (8 / bits) > 4 ? (8 / bits) : 4;
+  const int h = unit / 4;
+  const int reg_rows = res_reg_groups(bits, random) / h, lds_rows_max = kResLdsGroups / h;
+  const int64_t waves = int64_t(ws->num_cus) * (kResThreads / kWave);
+  int64_t total_units = 0;
+  for (int i = 0; i < count; i++) total_units += in_sizes[i] / unit;
+  int64_t rows = (total_units + waves * kWave - 1) / (waves * kWave);
+  if (rows < 1) rows = 1;
+  for (; rows <= reg_rows + lds_rows_max; rows++) {
+    int64_t pieces = 0;
+    for (int i = 0; i < count; i++) {
+      const int64_t p = (in_sizes[i] / unit + rows * kWave - 1) / (rows * kWave);
+      pieces += p < 1 ? 1 : p;
+    }
+    if (pieces <= waves) break;
+  }
+  if (rows > reg_rows + lds_rows_max) return false;
+  ma.rows = static_cast<uint32_t>(rows);
+  ma.lds_rows = rows > reg_rows ? static_cast<uint32_t>(rows - reg_rows) : 0u;
+  const int spare_rows = (kResLdsTotalGroups - int(ma.lds_rows) * h) / h;
+  pre_rows = (random && spare_rows >= res_pre_rows(bits)) ? static_cast<uint32_t>(res_pre_rows(bits)) : 0u;
+  ma.nseg = count;
+  ma.piece_start[0] = 0;
+  for (int i = 0; i < count; i++) {
+    const int64_t p = (in_sizes[i] / unit + rows * kWave - 1) / (rows * kWave);
+    ma.piece_start[i + 1] = ma.piece_start[i] + static_cast<int32_t>(p < 1 ? 1 : p);
+  }
+  return true;
+}
+
+template <int B, bool RANDOM, int PRE>
+int launch_resident_multi_as(const ResMultiArgs& ma, int num_cus, hipStream_t st) {
+  constexpr int H = ((8 / B) > 4 ? (8 / B) : 4) / 4;
+  static std::mutex attr_mu;
+  static uint64_t attr_done = 0;  // bit d: done on device d (devices beyond 63 set it on every launch)
+  {
+    int dev = 0;
+    HPX_HIP(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> g(attr_mu);
+    if (dev >= 64 || !(attr_done >> dev & 1)) {
+      HPX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&terngrad_resident_multi_kernel<B, RANDOM, PRE>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  kResLdsTotalGroups * kResThreads * int(sizeof(float4))));
+      if (dev < 64) attr_done |= uint64_t(1) << dev;
+    }
+  }
+  const size_t lds = size_t(ma.lds_rows + PRE) * H * kResThreads * sizeof(float4);
+  if (hpx::g_prof_on) hpx::prof_begin("terngrad_resident_multi_kernel", st);
+  hipLaunchKernelGGL((terngrad_resident_multi_kernel<B, RANDOM, PRE>), dim3(num_cus), dim3(kResThreads), lds, st, ma);
+  if (hpx::g_prof_on) hpx::prof_end(st);
+  HPX_HIP(hipGetLastError());
+  return HPX_OK;
+}
+
+template <int B>
+int launch_resident_multi_bits(const ResMultiArgs& ma, bool random, uint32_t pre_rows, int num_cus, hipStream_t st) {
+  if (!random) return launch_resident_multi_as<B, false, 0>(ma, num_cus, st);
+  if (pre_rows) return launch_resident_multi_as<B, true, res_pre_rows(B)>(ma, num_cus, st);
+  return launch_resident_multi_as<B, true, 0>(ma, num_cus, st);
+}
+
+int launch_resident_multi(const ResMultiArgs& ma, int bits, bool random, uint32_t pre_rows, int num_cus, hipStream_t st) {
+  switch (bits) {
+    case 1: return launch_resident_multi_bits<1>(ma, random, pre_rows, num_cus, st);
+    case 2: return launch_resident_multi_bits<2>(ma, random, pre_rows, num_cus, st);
+    case 4: return launch_resident_multi_bits<4>(ma, random, pre_rows, num_cus, st);
+    default: return launch_resident_multi_bits<8>(ma, random, pre_rows, num_cus, st);
+  }
+}
+
 int launch_resident(const ResArgs& ra, int num_cus, hipStream_t st) {
   switch (ra.seg.bits) {
     case 1: return launch_resident_bits<1>(ra, num_cus, st);
@@ -1235,6 +1552,30 @@ HPX_API int hpx_terngrad_encode(int count, const float* const* ins, const int32_
   rc = hpx::check_barrier_expired(ws, "hpx_terngrad_encode");
   if (rc != HPX_OK) return rc;
   uint32_t* expired = reinterpret_cast<uint32_t*>(ws->pinned + hpx::kPinnedFlagOffset);
+  // A call with several tensors that fit the chip together: one resident launch for all of them.
+  if (count >= 2 && !ws->barrier_broken) {
+    ResMultiArgs ma;
+    uint32_t pre_rows = 0;
+    if (resident_multi_plan(count, in_sizes, bitwidths, enable_randoms, ws, ma, pre_rows) && hpx::claim_barrier_kernels(ws)) {
+      for (int i = 0; i < count; i++) {
+        const uint64_t seed = seeds ? seeds[i] : hpx::clock_seed();
+        ma.seg[i] = EncSeg{ins[i], outs[i], in_sizes[i], out_sizes[i], static_cast<uint32_t>(seed), bitwidths[i],
+                           static_cast<uint8_t>(enable_randoms[i] != 0), 0};
+      }
+      if (++ws->bar_gen == 0) {
+        HPX_HIP(hipStreamSynchronize(st));
+        HPX_HIP(hipMemset(ws->bar, 0, hpx::kBarWords * sizeof(uint32_t)));
+        ws->bar_gen = 1;
+      }
+      ma.slots = ws->slots;
+      ma.epoch = ws->epoch;
+      ma.gen = ws->bar_gen;
+      ma.bar = reinterpret_cast<uint64_t*>(ws->bar);
+      ma.host_flag = expired;
+      ma.spin_limit = resident_spin_limit();
+      return launch_resident_multi(ma, bitwidths[0], enable_randoms[0] != 0, pre_rows, ws->num_cus, st);
+    }
+  }
   std::vector<int> tiled;
   tiled.reserve(count);
   for (int i = 0; i < count; i++) {
