@@ -411,17 +411,55 @@ def test_resident_bucket_many_rows_and_full_table(tg, oracle_cpu, capi, bucket_f
         assert_bits_equal(host(outs[i]), ref, f"message[{i}] n={x.size}")
 
 
+def test_resident_bucket_groups_of_a_large_call(tg, oracle_cpu, capi, bucket_forced):
+    # 77 M elements: more than the chip holds, so the call becomes three resident launches (5 + 5 + 3 tensors);
+    # then a call whose widths change half way: two launches
+    capi.set_option("terngrad_resident_min", 10 << 20)
+    rng = np.random.default_rng(34)
+    sizes = [6_000_000 + int(d) for d in rng.integers(-3, 4, 11)] + [1000, 5_000_003]
+    xs = [rng.normal(0, 1e-2, n).astype(np.float32) for n in sizes]
+    dx = [dev(x) for x in xs]
+    seeds = [int(s) for s in rng.integers(0, 2**63, len(sizes))]
+    before = _bucket_launches(capi)
+    outs = tg.encode(dx, [2] * len(xs), [1] * len(xs), seeds)
+    torch.cuda.synchronize()
+    assert _bucket_launches(capi) == before + 3
+    for i, x in enumerate(xs):
+        rc, ref = oracle_cpu.terngrad_encode(x, 2, 1, seeds[i])
+        assert_bits_equal(host(outs[i]), ref, f"message[{i}] n={x.size}")
+    bws = [2, 2, 2, 4, 4, 4]
+    before = _bucket_launches(capi)
+    outs = tg.encode(dx[:6], bws, [1] * 6, seeds[:6])
+    torch.cuda.synchronize()
+    assert _bucket_launches(capi) == before + 2
+    for i in range(6):
+        rc, ref = oracle_cpu.terngrad_encode(xs[i], bws[i], 1, seeds[i])
+        assert_bits_equal(host(outs[i]), ref, f"message[{i}] b={bws[i]}")
+    # a group too small for the threshold between two that reach it: tiled kernels for that one, same bytes
+    bws = [2, 2, 4, 2, 2]
+    sz = [0, 1, 11, 2, 3]                       # tensor 11 has 1000 elements
+    before = _bucket_launches(capi)
+    outs = tg.encode([dx[k] for k in sz], bws, [1] * 5, [seeds[k] for k in sz])
+    torch.cuda.synchronize()
+    assert _bucket_launches(capi) == before + 2
+    for i, k in enumerate(sz):
+        rc, ref = oracle_cpu.terngrad_encode(xs[k], bws[i], 1, seeds[k])
+        assert_bits_equal(host(outs[i]), ref, f"message[{i}] b={bws[i]}")
+
+
 def test_resident_bucket_falls_back(tg, oracle_cpu, capi, bucket_forced):
     rng = np.random.default_rng(33)
     xs = [rng.normal(0, 1e-2, n).astype(np.float32) for n in (5000, 70001, 1234)]
     before = _bucket_launches(capi)
-    # mixed widths or rounding modes: every tensor on its own
+    # alternating widths or rounding modes: no two neighbours can share a launch
     _check(tg, oracle_cpu, xs, [2, 4, 2], [1, 1, 1], [1, 2, 3], [0, 0, 0], rng)
     _check(tg, oracle_cpu, xs, [2, 2, 2], [1, 0, 1], [1, 2, 3], [0, 0, 0], rng)
-    # more tensors than one table holds
+    assert _bucket_launches(capi) == before
+    # more tensors than one table holds: 192 in one launch, the last one on its own
     many = [rng.normal(0, 1e-2, 300).astype(np.float32) for _ in range(193)]
     _check(tg, oracle_cpu, many, [2] * 193, [1] * 193, list(range(193)), [0] * 193, rng)
-    assert _bucket_launches(capi) == before
+    assert _bucket_launches(capi) == before + 1
+    before += 1
     # below the threshold
     capi.set_option("terngrad_resident_min", 1 << 20)
     _check(tg, oracle_cpu, xs, [2, 2, 2], [1, 1, 1], [1, 2, 3], [0, 0, 0], rng)

@@ -1271,6 +1271,48 @@ int launch_resident_bits(const ResArgs& ra, int num_cus, hipStream_t st) {
   return launch_resident_as<B, true, 0>(ra, num_cus, st);
 }
 
+// The tag of the next launch that uses the reduction slots / the exchange memory.
+int next_slot_epoch(hpx::Workspace* ws, hipStream_t st) {
+  if (++ws->epoch == 0) {
+    // The 32-bit tag wrapped: start over from cleared slots.
+    HPX_HIP(hipStreamSynchronize(st));
+    HPX_HIP(hipMemset(ws->slots, 0, ws->slot_words * sizeof(uint64_t)));
+    ws->epoch = 1;
+  }
+  return HPX_OK;
+}
+int next_barrier_generation(hpx::Workspace* ws, hipStream_t st) {
+  if (++ws->bar_gen == 0) {
+    // The 32-bit generation wrapped: start over from cleared exchange memory.
+    HPX_HIP(hipStreamSynchronize(st));
+    HPX_HIP(hipMemset(ws->bar, 0, hpx::kBarWords * sizeof(uint32_t)));
+    ws->bar_gen = 1;
+  }
+  return HPX_OK;
+}
+
+// How many of the first tensors of a list can share one resident launch: they have the width and rounding
+// mode of the first, are at most kCapLarge, and their pieces at the largest row count fit the chip.
+int resident_multi_extent(int count, const int32_t* in_sizes, const uint8_t* bitwidths, const int32_t* enable_randoms,
+                          const hpx::Workspace* ws) {
+  if (ws->num_cus <= 0 || ws->num_cus > kBarMaxWorkgroups) return 0;
+  const int bits = bitwidths[0];
+  const bool random = enable_randoms[0] != 0;
+  const int unit = (8 / bits) > 4 ? (8 / bits) : 4;
+  const int h = unit / 4;
+  const int64_t rows_max = res_reg_groups(bits, random) / h + kResLdsGroups / h;
+  const int64_t waves = int64_t(ws->num_cus) * (kResThreads / kWave);
+  int64_t pieces = 0;
+  int k = 0;
+  for (; k < count && k < kCapLarge; k++) {
+    if (bitwidths[k] != bits || (enable_randoms[k] != 0) != random) break;
+    const int64_t p = (in_sizes[k] / unit + rows_max * kWave - 1) / (rows_max * kWave);
+    pieces += p < 1 ? 1 : p;
+    if (pieces > waves) break;
+  }
+  return k;
+}
+
 // Rows per piece for a call with several tensors, or false when the call does not qualify: one bit
 // width and rounding mode, a total of at least the resident threshold, and all pieces on the chip at once.
 bool resident_multi_plan(int count, const int32_t* in_sizes, const uint8_t* bitwidths, const int32_t* enable_randoms,
@@ -1541,67 +1583,73 @@ HPX_API int hpx_terngrad_encode(int count, const float* const* ins, const int32_
   if (rc != HPX_OK) return rc;
   rc = hpx::ensure_barrier(ws);
   if (rc != HPX_OK) return rc;
-  if (++ws->epoch == 0) {
-    // The 32-bit tag wrapped: start over from cleared slots.
-    HPX_HIP(hipStreamSynchronize(st));
-    HPX_HIP(hipMemset(ws->slots, 0, ws->slot_words * sizeof(uint64_t)));
-    ws->epoch = 1;
-  }
 
   // Large tensors take the single-launch resident kernel, the rest the tiled pair.
   rc = hpx::check_barrier_expired(ws, "hpx_terngrad_encode");
   if (rc != HPX_OK) return rc;
   uint32_t* expired = reinterpret_cast<uint32_t*>(ws->pinned + hpx::kPinnedFlagOffset);
-  // A call with several tensors that fit the chip together: one resident launch for all of them.
-  if (count >= 2 && !ws->barrier_broken) {
-    ResMultiArgs ma;
-    uint32_t pre_rows = 0;
-    if (resident_multi_plan(count, in_sizes, bitwidths, enable_randoms, ws, ma, pre_rows) && hpx::claim_barrier_kernels(ws)) {
-      for (int i = 0; i < count; i++) {
-        const uint64_t seed = seeds ? seeds[i] : hpx::clock_seed();
-        ma.seg[i] = EncSeg{ins[i], outs[i], in_sizes[i], out_sizes[i], static_cast<uint32_t>(seed), bitwidths[i],
-                           static_cast<uint8_t>(enable_randoms[i] != 0), 0};
-      }
-      if (++ws->bar_gen == 0) {
-        HPX_HIP(hipStreamSynchronize(st));
-        HPX_HIP(hipMemset(ws->bar, 0, hpx::kBarWords * sizeof(uint32_t)));
-        ws->bar_gen = 1;
-      }
-      ma.slots = ws->slots;
-      ma.epoch = ws->epoch;
-      ma.gen = ws->bar_gen;
-      ma.bar = reinterpret_cast<uint64_t*>(ws->bar);
-      ma.host_flag = expired;
-      ma.spin_limit = resident_spin_limit();
-      return launch_resident_multi(ma, bitwidths[0], enable_randoms[0] != 0, pre_rows, ws->num_cus, st);
-    }
-  }
+  // Consecutive tensors of one width and rounding mode that fit the chip together and add up to the
+  // resident threshold take one resident launch per such group; a remaining tensor that is large enough
+  // takes the single-tensor resident kernel; the rest goes to the tiled pair of kernels.
   std::vector<int> tiled;
   tiled.reserve(count);
-  for (int i = 0; i < count; i++) {
-    ResArgs ra;
-    if (ws->barrier_broken || !resident_plan(in_sizes[i], bitwidths[i], enable_randoms[i] != 0, ws, ra) ||
-        !hpx::claim_barrier_kernels(ws)) {
-      tiled.push_back(i);
-      continue;
+  const bool buckets = count >= 2 && hpx::option(hpx::kOptTerngradResidentBucket) != 0 &&
+                       hpx::option(hpx::kOptTerngradResidentMin) >= 0;
+  int i = 0;
+  while (i < count) {
+    int j = i;
+    if (buckets && !ws->barrier_broken) j = i + resident_multi_extent(count - i, in_sizes + i, bitwidths + i, enable_randoms + i, ws);
+    if (j - i >= 2) {
+      ResMultiArgs ma;
+      uint32_t pre_rows = 0;
+      if (resident_multi_plan(j - i, in_sizes + i, bitwidths + i, enable_randoms + i, ws, ma, pre_rows) &&
+          hpx::claim_barrier_kernels(ws)) {
+        for (int k = i; k < j; k++) {
+          const uint64_t seed = seeds ? seeds[k] : hpx::clock_seed();
+          ma.seg[k - i] = EncSeg{ins[k], outs[k], in_sizes[k], out_sizes[k], static_cast<uint32_t>(seed), bitwidths[k],
+                                 static_cast<uint8_t>(enable_randoms[k] != 0), 0};
+        }
+        rc = next_barrier_generation(ws, st);
+        if (rc != HPX_OK) return rc;
+        rc = next_slot_epoch(ws, st);
+        if (rc != HPX_OK) return rc;
+        ma.slots = ws->slots;
+        ma.epoch = ws->epoch;
+        ma.gen = ws->bar_gen;
+        ma.bar = reinterpret_cast<uint64_t*>(ws->bar);
+        ma.host_flag = expired;
+        ma.spin_limit = resident_spin_limit();
+        rc = launch_resident_multi(ma, bitwidths[i], enable_randoms[i] != 0, pre_rows, ws->num_cus, st);
+        if (rc != HPX_OK) return rc;
+        i = j;
+        continue;
+      }
     }
-    const uint64_t seed = seeds ? seeds[i] : hpx::clock_seed();
-    ra.seg = EncSeg{ins[i], outs[i], in_sizes[i], out_sizes[i], static_cast<uint32_t>(seed), bitwidths[i],
-                    static_cast<uint8_t>(enable_randoms[i] != 0), 0};
-    if (++ws->bar_gen == 0) {
-      // The 32-bit generation wrapped: start over from cleared exchange memory.
-      HPX_HIP(hipStreamSynchronize(st));
-      HPX_HIP(hipMemset(ws->bar, 0, hpx::kBarWords * sizeof(uint32_t)));
-      ws->bar_gen = 1;
+    // tensors i .. max(j, i + 1) - 1, each on its own
+    const int stop = j > i ? j : i + 1;
+    for (; i < stop; i++) {
+      ResArgs ra;
+      if (ws->barrier_broken || !resident_plan(in_sizes[i], bitwidths[i], enable_randoms[i] != 0, ws, ra) ||
+          !hpx::claim_barrier_kernels(ws)) {
+        tiled.push_back(i);
+        continue;
+      }
+      const uint64_t seed = seeds ? seeds[i] : hpx::clock_seed();
+      ra.seg = EncSeg{ins[i], outs[i], in_sizes[i], out_sizes[i], static_cast<uint32_t>(seed), bitwidths[i],
+                      static_cast<uint8_t>(enable_randoms[i] != 0), 0};
+      rc = next_barrier_generation(ws, st);
+      if (rc != HPX_OK) return rc;
+      ra.gen = ws->bar_gen;
+      ra.bar = reinterpret_cast<uint64_t*>(ws->bar);
+      ra.host_flag = expired;
+      ra.spin_limit = resident_spin_limit();
+      rc = launch_resident(ra, ws->num_cus, st);
+      if (rc != HPX_OK) return rc;
     }
-    ra.gen = ws->bar_gen;
-    ra.bar = reinterpret_cast<uint64_t*>(ws->bar);
-    ra.host_flag = expired;
-    ra.spin_limit = resident_spin_limit();
-    rc = launch_resident(ra, ws->num_cus, st);
-    if (rc != HPX_OK) return rc;
   }
   if (tiled.empty()) return HPX_OK;
+  rc = next_slot_epoch(ws, st);  // its own tag: the slots may hold words of a resident launch of this call
+  if (rc != HPX_OK) return rc;
   if (int(tiled.size()) == count) {
     if (count <= kCapSmall)
       return launch_encode<kCapSmall>(count, ins, in_sizes, outs, out_sizes, bitwidths, enable_randoms, seeds,
