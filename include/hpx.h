@@ -142,7 +142,13 @@ int hpx_tbq_decode(int count, float* const* outs, const int32_t* sizes,
  * to the two-launch path).  The wait is bounded: if it ever expires (the GPU is
  * shared with another process's barrier kernels, say) the call's output is
  * invalid, the NEXT hpx_terngrad_encode on the stream returns -2 once and the
- * stream falls back to the two-launch path for good. */
+ * stream falls back to the two-launch path for good.
+ * A call with several tensors is first cut into groups of consecutive tensors
+ * of one bit width and rounding mode (at most 192) that fit the chip together;
+ * a group of two or more that adds up to "terngrad_resident_min" elements is
+ * encoded by one launch of the same kind (option "terngrad_resident_bucket",
+ * same conditions on `stream`); what is left over goes tensor by tensor as
+ * described above.  The bytes written do not depend on the route. */
 int hpx_terngrad_encode(int count, const float* const* ins, const int32_t* in_sizes,
                         uint8_t* const* outs, const int32_t* out_sizes,
                         const uint8_t* bitwidths, const int32_t* enable_randoms,
