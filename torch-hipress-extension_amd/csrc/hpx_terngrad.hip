@@ -1347,8 +1347,11 @@ bool resident_multi_plan(int count, const int32_t* in_sizes, const uint8_t* bitw
   if (rows > reg_rows + lds_rows_max) return false;
   ma.rows = static_cast<uint32_t>(rows);
   ma.lds_rows = rows > reg_rows ? static_cast<uint32_t>(rows - reg_rows) : 0u;
+  // prepared rows: the full set, or half of it when the tensors' LDS rows leave no room for more
   const int spare_rows = (kResLdsTotalGroups - int(ma.lds_rows) * h) / h;
-  pre_rows = (random && spare_rows >= res_pre_rows(bits)) ? static_cast<uint32_t>(res_pre_rows(bits)) : 0u;
+  pre_rows = 0u;
+  if (random && spare_rows >= res_pre_rows(bits)) pre_rows = static_cast<uint32_t>(res_pre_rows(bits));
+  else if (random && spare_rows >= res_pre_rows(bits) / 2) pre_rows = static_cast<uint32_t>(res_pre_rows(bits) / 2);
   ma.nseg = count;
   ma.piece_start[0] = 0;
   for (int i = 0; i < count; i++) {
@@ -1385,7 +1388,8 @@ int launch_resident_multi_as(const ResMultiArgs& ma, int num_cus, hipStream_t st
 template <int B>
 int launch_resident_multi_bits(const ResMultiArgs& ma, bool random, uint32_t pre_rows, int num_cus, hipStream_t st) {
   if (!random) return launch_resident_multi_as<B, false, 0>(ma, num_cus, st);
-  if (pre_rows) return launch_resident_multi_as<B, true, res_pre_rows(B)>(ma, num_cus, st);
+  if (pre_rows == uint32_t(res_pre_rows(B))) return launch_resident_multi_as<B, true, res_pre_rows(B)>(ma, num_cus, st);
+  if (pre_rows == uint32_t(res_pre_rows(B) / 2)) return launch_resident_multi_as<B, true, res_pre_rows(B) / 2>(ma, num_cus, st);
   return launch_resident_multi_as<B, true, 0>(ma, num_cus, st);
 }
 
