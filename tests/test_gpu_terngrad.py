@@ -447,6 +447,37 @@ def test_resident_bucket_groups_of_a_large_call(tg, oracle_cpu, capi, bucket_for
         assert_bits_equal(host(outs[i]), ref, f"message[{i}] b={bws[i]}")
 
 
+def test_resident_bucket_barrier_expiry_is_reported(tg, oracle_cpu, capi, bucket_forced):
+    # As for the single-tensor kernel: with a zero bound every workgroup gives up at the barrier and leaves, the
+    # next encode on the stream reports it, and the stream keeps to the tiled kernels afterwards.
+    rng = np.random.default_rng(35)
+    xs = [rng.normal(0, 1e-2, n).astype(np.float32) for n in (1_500_000, 70_001, 900_000)]
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    assert capi.load().hpx_release_workspaces() == 0       # the side stream becomes the owner of the barrier kernels
+    old_ms = capi.set_option("terngrad_barrier_ms", 0)
+    try:
+        with torch.cuda.stream(side):
+            dx = [dev(x) for x in xs]
+            before = _bucket_launches(capi)
+            tg.encode(dx, [2] * 3, [1] * 3, [9, 10, 11])
+            side.synchronize()
+            assert _bucket_launches(capi) == before + 1
+            capi.set_option("terngrad_barrier_ms", old_ms)
+            tg.encode(dx, [2] * 3, [1] * 3, [9, 10, 11], expect_rc=-2)
+            assert "barrier" in capi.last_error()
+            outs = tg.encode(dx, [2] * 3, [1] * 3, [9, 10, 11])
+            side.synchronize()
+            assert _bucket_launches(capi) == before + 1
+            for i, x in enumerate(xs):
+                rc, ref = oracle_cpu.terngrad_encode(x, 2, 1, 9 + i)
+                assert_bits_equal(host(outs[i]), ref, f"message[{i}] after fallback")
+    finally:
+        capi.set_option("terngrad_barrier_ms", old_ms)
+        torch.cuda.synchronize()
+        assert capi.load().hpx_release_workspaces() == 0
+
+
 def test_resident_bucket_falls_back(tg, oracle_cpu, capi, bucket_forced):
     rng = np.random.default_rng(33)
     xs = [rng.normal(0, 1e-2, n).astype(np.float32) for n in (5000, 70001, 1234)]
