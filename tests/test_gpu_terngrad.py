@@ -427,6 +427,16 @@ def test_resident_bucket_groups_of_a_large_call(tg, oracle_cpu, capi, bucket_for
     for i, x in enumerate(xs):
         rc, ref = oracle_cpu.terngrad_encode(x, 2, 1, seeds[i])
         assert_bits_equal(host(outs[i]), ref, f"message[{i}] n={x.size}")
+    # the same call again, then decoded: the launches of the second call wait for nothing they should not
+    outs2 = tg.encode(dx, [2] * len(xs), [1] * len(xs), seeds)
+    back = [torch.empty(x.size, device="cuda") for x in xs]
+    tg.decode(outs2, back, [0] * len(xs))
+    torch.cuda.synchronize()
+    for i, x in enumerate(xs):
+        rc, ref = oracle_cpu.terngrad_encode(x, 2, 1, seeds[i])
+        assert_bits_equal(host(outs2[i]), ref, f"second call, message[{i}]")
+        rc, dec = oracle_cpu.terngrad_decode(ref, x.size)
+        assert_bits_equal(host(back[i]), dec, f"decoded[{i}]")
     bws = [2, 2, 2, 4, 4, 4]
     before = _bucket_launches(capi)
     outs = tg.encode(dx[:6], bws, [1] * 6, seeds[:6])
