@@ -195,6 +195,34 @@ def test_several_messages_into_one_tensor(tg, oracle_cpu, n):
     assert tg.status() == 0
 
 
+@pytest.mark.parametrize("n", [4095, 4096, 8192 + 3, 16384, 5 * 16384 + 4096 + 17, 1_000_003])
+@pytest.mark.parametrize("count", [2, 7, 8, 9])
+def test_several_two_bit_messages_into_one_tensor(tg, oracle_cpu, n, count):
+    # the configuration the reference ships with (2-bit messages): whole sub-tiles of 4096 elements take the
+    # decoder's pipelined path when there are at most 8 messages; offsets make the payloads start at odd addresses
+    rng = np.random.default_rng(1000 * count + n % 997)
+    msgs, dm = [], []
+    for k in range(count):
+        x = rng.normal(0, 1e-2 * (k + 1), n).astype(np.float32)
+        rc, m = oracle_cpu.terngrad_encode(x, 2, 1, 500 + k)
+        assert rc == 0
+        msgs.append(m)
+        buf = torch.zeros(m.size + 8, dtype=torch.uint8, device="cuda")
+        view = buf[k % 5:k % 5 + m.size]
+        view.copy_(dev(m))
+        dm.append(view)
+    for adds in ([1] * count, [0] + [1] * (count - 1), [1] + [0] + [1] * (count - 2)):
+        base = rng.normal(0, 1, n).astype(np.float32)
+        out = dev(base)
+        tg.decode(dm, [out] * count, adds)
+        torch.cuda.synchronize()
+        ref = base.copy()
+        for m, add in zip(msgs, adds):
+            rc, ref = oracle_cpu.terngrad_decode(m, n, ref, add)
+        assert_bits_equal(host(out), ref, f"accumulated n={n} count={count} adds={adds}")
+    assert tg.status() == 0
+
+
 def test_many_tensors_each_with_several_messages(tg, oracle_cpu):
     rng = np.random.default_rng(78)
     sizes = [int(s) for s in np.exp(rng.uniform(np.log(5), np.log(20000), 70))]

@@ -1049,6 +1049,102 @@ __device__ __forceinline__ uint32_t code_at(const uint8_t* __restrict__ pay, siz
   return (uint32_t(pay[i / dpb]) >> ((i % dpb) * bits)) & ((1u << bits) - 1u);
 }
 
+// The common case of the multi-message decoder (NS complete 2-bit messages, 2 <= NS <= 8), for the sub-tiles of
+// the workgroup that lie wholly inside the tensor; returns how many of its kMultiRep sub-tiles it has done.
+// A wave owns kDIters * 64 consecutive groups, i.e. that many consecutive payload bytes of every message: each
+// message costs the wave ONE load (a dword per lane) and the lanes pick their bytes out of it with cross-lane
+// reads.  NS is a compile-time constant and the loads are unconditional: under per-message branches the
+// compiler made every load wait for the one before, and each message then cost every sub-tile one more memory
+// latency (7 messages: 71 us against 36 for one).  The loads of the next sub-tile are requested before the
+// current one is folded.
+template <int NS>
+__device__ __forceinline__ uint32_t decode_two_bit_pipelined(float* __restrict__ op, uint32_t n, bool need_old, uint32_t sub0,
+                                                             const uint8_t* const* s_pay, const float* s_gap,
+                                                             const float* s_mn, const int32_t* s_add) {
+  static_assert(kDIters * 4 <= kWave && kMultiRep % 2 == 0, "a wave's bytes of one message fit one dword per lane; sub-tiles go in pairs");
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const uint32_t whole = n / uint32_t(kThreads * kDIters * 4);  // sub-tiles wholly inside the tensor
+  const uint32_t nfull = whole > sub0 ? (whole - sub0 < uint32_t(kMultiRep) ? whole - sub0 : uint32_t(kMultiRep)) : 0u;
+  // per-message constants as wave-uniform values in scalar registers
+  const uint8_t* pay[NS];
+  float gap[NS], mn[NS];
+  uint32_t addm = 0;
+#pragma unroll
+  for (int j = 0; j < NS; j++) {
+    const uint64_t pj = reinterpret_cast<uint64_t>(s_pay[j]);
+    // (the builtin returns a signed int: without the cast to uint32_t a low half with its top bit set would
+    // be sign-extended over the high half)
+    const uint32_t plo = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(uint32_t(pj))));
+    const uint32_t phi = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(uint32_t(pj >> 32))));
+    pay[j] = reinterpret_cast<const uint8_t*>(uint64_t(plo) | (uint64_t(phi) << 32));
+    gap[j] = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(s_gap[j])));
+    mn[j] = __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(s_mn[j])));
+    addm |= (__builtin_amdgcn_readfirstlane(s_add[j]) != 0 ? 1u : 0u) << j;
+  }
+  const bool all_add = addm == (1u << NS) - 1u;  // the root's gather-decode: no select per value then
+  const uint32_t pick = (lane / 4) * 4, shift = 8 * (lane & 3);
+  auto first_group = [&](uint32_t rep) {  // the wave's first group of sub-tile rep
+    return (sub0 + rep) * uint32_t(kThreads * kDIters) + (threadIdx.x / kWave) * uint32_t(kDIters * kWave);
+  };
+  auto request = [&](uint32_t rep, float4 (&acc)[kDIters], uint32_t (&dw)[NS]) {
+    const uint32_t gw = first_group(rep);
+    if (need_old) {
+#pragma unroll
+      for (int k = 0; k < kDIters; k++) acc[k] = ld4_stream(op + size_t(gw + k * kWave + lane) * 4);
+    } else {
+#pragma unroll
+      for (int k = 0; k < kDIters; k++) acc[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+#pragma unroll
+    for (int j = 0; j < NS; j++) dw[j] = reinterpret_cast<const u32u*>(pay[j] + gw + lane * 4)->v;  // the payload starts at byte 10
+  };
+  auto fold_store = [&](uint32_t rep, float4 (&acc)[kDIters], const uint32_t (&dw)[NS]) {
+    const uint32_t gw = first_group(rep);
+    if (all_add) {
+#pragma unroll
+      for (int j = 0; j < NS; j++)
+#pragma unroll
+        for (int k = 0; k < kDIters; k++) {
+          const uint32_t byte = (__builtin_amdgcn_ds_bpermute(int(k * kWave + pick), int(dw[j])) >> shift) & 0xFFu;
+          const float4 v = group_values<2>(byte, gap[j], mn[j]);
+          acc[k].x = v.x + acc[k].x; acc[k].y = v.y + acc[k].y; acc[k].z = v.z + acc[k].z; acc[k].w = v.w + acc[k].w;
+        }
+    } else {
+#pragma unroll
+      for (int j = 0; j < NS; j++) {
+        const bool add = (addm >> j) & 1u;
+#pragma unroll
+        for (int k = 0; k < kDIters; k++) {
+          const uint32_t byte = (__builtin_amdgcn_ds_bpermute(int(k * kWave + pick), int(dw[j])) >> shift) & 0xFFu;
+          const float4 v = group_values<2>(byte, gap[j], mn[j]);
+          acc[k].x = add ? v.x + acc[k].x : v.x; acc[k].y = add ? v.y + acc[k].y : v.y;
+          acc[k].z = add ? v.z + acc[k].z : v.z; acc[k].w = add ? v.w + acc[k].w : v.w;
+        }
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < kDIters; k++) {
+      st4_stream(op + size_t(gw + k * kWave + lane) * 4, acc[k]);
+      __asm__ volatile("" ::: "memory");
+    }
+  };
+  float4 acc0[kDIters], acc1[kDIters];
+  uint32_t dw0[NS], dw1[NS];
+  if (nfull > 0) request(0, acc0, dw0);
+#pragma unroll
+  for (uint32_t rep = 0; rep < uint32_t(kMultiRep); rep += 2) {
+    if (rep < nfull) {
+      if (rep + 1 < nfull) request(rep + 1, acc1, dw1);
+      fold_store(rep, acc0, dw0);
+    }
+    if (rep + 1 < nfull) {
+      if (rep + 2 < nfull) request(rep + 2, acc0, dw0);
+      fold_store(rep + 1, acc1, dw1);
+    }
+  }
+  return nfull;
+}
+
 __global__ __launch_bounds__(kThreads) void terngrad_decode_multi_kernel(const MArgs a) {
   __shared__ float s_mn[kMultiSlotsPerSeg], s_gap[kMultiSlotsPerSeg];
   __shared__ uint32_t s_cnt[kMultiSlotsPerSeg], s_bits[kMultiSlotsPerSeg];
@@ -1092,7 +1188,21 @@ __global__ __launch_bounds__(kThreads) void terngrad_decode_multi_kernel(const M
   bool all_two_bit = true;  // ... and is a 2-bit message (the configuration the reference ships with)
   for (int j = 0; j < ns; j++) all_two_bit = all_two_bit && s_bits[j] == 2u;
   // The headers are parsed once per workgroup and serve kMultiRep consecutive sub-tiles.
-  for (uint32_t rep = 0; rep < uint32_t(kMultiRep); rep++) {
+  uint32_t rep_begin = 0;
+  if (all_cover && all_two_bit && ns <= 8) {
+    const uint32_t sub0 = static_cast<uint32_t>(tile - a.tile_start[s]) * kMultiRep;
+    switch (ns) {  // the number of messages as a compile-time constant: straight-line code, all loads of a sub-tile in flight together
+      case 2: rep_begin = decode_two_bit_pipelined<2>(op, n, need_old, sub0, s_pay, s_gap, s_mn, s_add); break;
+      case 3: rep_begin = decode_two_bit_pipelined<3>(op, n, need_old, sub0, s_pay, s_gap, s_mn, s_add); break;
+      case 4: rep_begin = decode_two_bit_pipelined<4>(op, n, need_old, sub0, s_pay, s_gap, s_mn, s_add); break;
+      case 5: rep_begin = decode_two_bit_pipelined<5>(op, n, need_old, sub0, s_pay, s_gap, s_mn, s_add); break;
+      case 6: rep_begin = decode_two_bit_pipelined<6>(op, n, need_old, sub0, s_pay, s_gap, s_mn, s_add); break;
+      case 7: rep_begin = decode_two_bit_pipelined<7>(op, n, need_old, sub0, s_pay, s_gap, s_mn, s_add); break;
+      case 8: rep_begin = decode_two_bit_pipelined<8>(op, n, need_old, sub0, s_pay, s_gap, s_mn, s_add); break;
+      default: break;
+    }
+  }
+  for (uint32_t rep = rep_begin; rep < uint32_t(kMultiRep); rep++) {
   const uint32_t g0 = (static_cast<uint32_t>(tile - a.tile_start[s]) * kMultiRep + rep) * uint32_t(kThreads * kDIters) + threadIdx.x;
   if (uint64_t(g0 - threadIdx.x) * 4 >= n) break;
   if (all_cover && all_two_bit && uint64_t(g0 - threadIdx.x + kThreads * kDIters) * 4 <= n) {
