@@ -224,6 +224,32 @@ def test_several_messages_into_one_tensor(tbq, oracle_cpu, n):
         assert_bits_equal(host(out), ref, f"accumulated n={n} adds={adds}")
 
 
+@pytest.mark.parametrize("count", [2, 3, 5, 8, 9])
+def test_message_counts_of_the_straight_line_path(tbq, oracle_cpu, count):
+    # whole tiles with 2 to 8 messages take code generated per message count; payloads start at odd addresses
+    rng = np.random.default_rng(300 + count)
+    n = 3 * 4096 + 4096 // 2 + 3
+    msgs, thrs, dm = [], [], []
+    for k in range(count):
+        thr = float(np.float32(rng.uniform(1e-3, 5e-3))) * (-1 if k == 1 else 1)
+        g = rng.normal(0, 2e-3, n).astype(np.float32)
+        m = oracle_cpu.tbq_encode(g, np.zeros(n, np.float32), abs(thr))
+        msgs.append(m); thrs.append(thr)
+        buf = torch.zeros(m.size + 8, dtype=torch.uint8, device="cuda")
+        view = buf[k % 5:k % 5 + m.size]
+        view.copy_(dev(m))
+        dm.append(view)
+    for adds in ([1] * count, [0] + [1] * (count - 1), [1, 0] + [1] * (count - 2)):
+        base = rng.normal(0, 1, n).astype(np.float32)
+        out = dev(base)
+        tbq.decode(dm, [out] * count, thrs, adds)
+        torch.cuda.synchronize()
+        ref = base.copy()
+        for m, thr, add in zip(msgs, thrs, adds):
+            ref = oracle_cpu.tbq_decode(m, n, thr, ref, add)
+        assert_bits_equal(host(out), ref, f"accumulated count={count} adds={adds}")
+
+
 def test_many_tensors_each_with_several_messages(tbq, oracle_cpu):
     rng = np.random.default_rng(77)
     sizes = [int(s) for s in np.exp(rng.uniform(np.log(5), np.log(20000), 70))]

@@ -1055,13 +1055,13 @@ __device__ __forceinline__ uint32_t code_at(const uint8_t* __restrict__ pay, siz
 // message costs the wave ONE load (a dword per lane) and the lanes pick their bytes out of it with cross-lane
 // reads.  NS is a compile-time constant and the loads are unconditional: under per-message branches the
 // compiler made every load wait for the one before, and each message then cost every sub-tile one more memory
-// latency (7 messages: 71 us against 36 for one).  The loads of the next sub-tile are requested before the
-// current one is folded.
+// latency (7 messages into 25.5 M elements: 75 us; now 65, of which about 30 are the 22 operations per group
+// and message).
 template <int NS>
-__device__ __forceinline__ uint32_t decode_two_bit_pipelined(float* __restrict__ op, uint32_t n, bool need_old, uint32_t sub0,
+__device__ __forceinline__ uint32_t decode_two_bit_whole(float* __restrict__ op, uint32_t n, bool need_old, uint32_t sub0,
                                                              const uint8_t* const* s_pay, const float* s_gap,
                                                              const float* s_mn, const int32_t* s_add) {
-  static_assert(kDIters * 4 <= kWave && kMultiRep % 2 == 0, "a wave's bytes of one message fit one dword per lane; sub-tiles go in pairs");
+  static_assert(kDIters * 4 <= kWave, "a wave's bytes of one message must fit one dword per lane");
   const uint32_t lane = threadIdx.x & (kWave - 1);
   const uint32_t whole = n / uint32_t(kThreads * kDIters * 4);  // sub-tiles wholly inside the tensor
   const uint32_t nfull = whole > sub0 ? (whole - sub0 < uint32_t(kMultiRep) ? whole - sub0 : uint32_t(kMultiRep)) : 0u;
@@ -1128,19 +1128,13 @@ __device__ __forceinline__ uint32_t decode_two_bit_pipelined(float* __restrict__
       __asm__ volatile("" ::: "memory");
     }
   };
-  float4 acc0[kDIters], acc1[kDIters];
-  uint32_t dw0[NS], dw1[NS];
-  if (nfull > 0) request(0, acc0, dw0);
-#pragma unroll
-  for (uint32_t rep = 0; rep < uint32_t(kMultiRep); rep += 2) {
-    if (rep < nfull) {
-      if (rep + 1 < nfull) request(rep + 1, acc1, dw1);
-      fold_store(rep, acc0, dw0);
-    }
-    if (rep + 1 < nfull) {
-      if (rep + 2 < nfull) request(rep + 2, acc0, dw0);
-      fold_store(rep + 1, acc1, dw1);
-    }
+  // One sub-tile at a time: requesting the next one ahead does not help, because the compiler lets a fold
+  // wait for every load in flight, the new ones included; more waves per SIMD hide the latency instead.
+  float4 acc0[kDIters];
+  uint32_t dw0[NS];
+  for (uint32_t rep = 0; rep < nfull; rep++) {
+    request(rep, acc0, dw0);
+    fold_store(rep, acc0, dw0);
   }
   return nfull;
 }
@@ -1192,13 +1186,13 @@ __global__ __launch_bounds__(kThreads) void terngrad_decode_multi_kernel(const M
   if (all_cover && all_two_bit && ns <= 8) {
     const uint32_t sub0 = static_cast<uint32_t>(tile - a.tile_start[s]) * kMultiRep;
     switch (ns) {  // the number of messages as a compile-time constant: straight-line code, all loads of a sub-tile in flight together
-      case 2: rep_begin = decode_two_bit_pipelined<2>(op, n, need_old, sub0, s_pay, s_gap, s_mn, s_add); break;
-      case 3: rep_begin = decode_two_bit_pipelined<3>(op, n, need_old, sub0, s_pay, s_gap, s_mn, s_add); break;
-      case 4: rep_begin = decode_two_bit_pipelined<4>(op, n, need_old, sub0, s_pay, s_gap, s_mn, s_add); break;
-      case 5: rep_begin = decode_two_bit_pipelined<5>(op, n, need_old, sub0, s_pay, s_gap, s_mn, s_add); break;
-      case 6: rep_begin = decode_two_bit_pipelined<6>(op, n, need_old, sub0, s_pay, s_gap, s_mn, s_add); break;
-      case 7: rep_begin = decode_two_bit_pipelined<7>(op, n, need_old, sub0, s_pay, s_gap, s_mn, s_add); break;
-      case 8: rep_begin = decode_two_bit_pipelined<8>(op, n, need_old, sub0, s_pay, s_gap, s_mn, s_add); break;
+      case 2: rep_begin = decode_two_bit_whole<2>(op, n, need_old, sub0, s_pay, s_gap, s_mn, s_add); break;
+      case 3: rep_begin = decode_two_bit_whole<3>(op, n, need_old, sub0, s_pay, s_gap, s_mn, s_add); break;
+      case 4: rep_begin = decode_two_bit_whole<4>(op, n, need_old, sub0, s_pay, s_gap, s_mn, s_add); break;
+      case 5: rep_begin = decode_two_bit_whole<5>(op, n, need_old, sub0, s_pay, s_gap, s_mn, s_add); break;
+      case 6: rep_begin = decode_two_bit_whole<6>(op, n, need_old, sub0, s_pay, s_gap, s_mn, s_add); break;
+      case 7: rep_begin = decode_two_bit_whole<7>(op, n, need_old, sub0, s_pay, s_gap, s_mn, s_add); break;
+      case 8: rep_begin = decode_two_bit_whole<8>(op, n, need_old, sub0, s_pay, s_gap, s_mn, s_add); break;
       default: break;
     }
   }
@@ -1251,16 +1245,16 @@ __global__ __launch_bounds__(kThreads) void terngrad_decode_multi_kernel(const M
     continue;
   }
   if (all_cover && uint64_t(g0 - threadIdx.x + kThreads * kDIters) * 4 <= n) {
-    // Whole tile, every message complete, other widths: old values and the code bytes of up to 8 messages x 4
+    // Whole tile, every message complete, other widths: old values and the code bytes of up to 4 messages x 4
     // groups are requested together, then folded in message order.
     float4 acc[kDIters];
 #pragma unroll
     for (int k = 0; k < kDIters; k++)
       acc[k] = need_old ? ld4_stream(op + size_t(g0 + k * kThreads) * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int j0 = 0; j0 < ns; j0 += 8) {
-      uint32_t raw[8][kDIters];
+    for (int j0 = 0; j0 < ns; j0 += 4) {
+      uint32_t raw[4][kDIters];
 #pragma unroll
-      for (int jj = 0; jj < 8; jj++)
+      for (int jj = 0; jj < 4; jj++)
 #pragma unroll
         for (int k = 0; k < kDIters; k++) {
           raw[jj][k] = 0;
@@ -1275,7 +1269,7 @@ __global__ __launch_bounds__(kThreads) void terngrad_decode_multi_kernel(const M
           }
         }
 #pragma unroll
-      for (int jj = 0; jj < 8; jj++) {
+      for (int jj = 0; jj < 4; jj++) {
         if (j0 + jj < ns) {
           const uint32_t bits = s_bits[j0 + jj];
           const float gap = s_gap[j0 + jj], mn = s_mn[j0 + jj];
