@@ -199,6 +199,18 @@ __device__ __forceinline__ int find_segment(const int32_t (&start)[CAP + 1], int
   }
 }
 
+// A pointer that has been kept in LDS, or put together from integers, has lost its address space, and a load
+// through it becomes a FLAT instruction.  The compiler must assume that FLAT loads finish out of order with all
+// other memory operations, so with one of them in flight every wait becomes a wait for everything
+// (s_waitcnt vmcnt(0) lgkmcnt(0)) and nothing overlaps.  as_global says what the pointer points to; the load has
+// to go through the returned pointer itself (a cast back to an ordinary pointer undoes it).
+template <typename T>
+using global_ptr = const __attribute__((address_space(1))) T*;
+template <typename T>
+__device__ __forceinline__ global_ptr<T> as_global(const T* p) {
+  return (global_ptr<T>)p;
+}
+
 // ---- grid-wide exchange / barrier --------------------------------------------
 // For kernels launched with at most kBarMaxWorkgroups workgroups that are all
 // resident at once (the host guarantees it: grid <= CUs, one workgroup fits a CU,

@@ -334,7 +334,7 @@ __global__ __launch_bounds__(kThreads) void tbq_decode_multi_kernel(const MArgs 
       for (int jj = 0; jj < 8; jj++) {
         dw[jj] = 0u;
         if (j0 + jj < ns && lane < uint32_t(kIters * kWave / 4)) {
-          dw[jj] = reinterpret_cast<const u32u*>(s_in[j0 + jj] + gw + lane * 4)->v;  // messages start at any byte
+          dw[jj] = as_global(reinterpret_cast<const u32u*>(s_in[j0 + jj] + gw + lane * 4))->v;  // messages start at any byte
         }
       }
       uint32_t q[8][kIters];
@@ -374,7 +374,7 @@ __global__ __launch_bounds__(kThreads) void tbq_decode_multi_kernel(const MArgs 
     for (uint32_t i = 0; i < lim; i++) {
       float acc = need_old ? op[e + i] : 0.f;
       for (int j = 0; j < ns; j++) {
-        const uint32_t q = s_in[j][grp];
+        const uint32_t q = as_global(s_in[j])[grp];
         const float v = (static_cast<float>((q >> (2 * i)) & 3) - 1) * s_thr[j];
         acc = s_add[j] ? v + acc : v;
       }

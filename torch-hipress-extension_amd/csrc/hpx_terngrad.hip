@@ -1096,7 +1096,7 @@ __device__ __forceinline__ uint32_t decode_two_bit_whole(float* __restrict__ op,
       for (int k = 0; k < kDIters; k++) acc[k] = make_float4(0.f, 0.f, 0.f, 0.f);
     }
 #pragma unroll
-    for (int j = 0; j < NS; j++) dw[j] = reinterpret_cast<const u32u*>(pay[j] + gw + lane * 4)->v;  // the payload starts at byte 10
+    for (int j = 0; j < NS; j++) dw[j] = as_global(reinterpret_cast<const u32u*>(pay[j] + gw + lane * 4))->v;  // the payload starts at byte 10
   };
   auto fold_store = [&](uint32_t rep, float4 (&acc)[kDIters], const uint32_t (&dw)[NS]) {
     const uint32_t gw = first_group(rep);
@@ -1128,8 +1128,6 @@ __device__ __forceinline__ uint32_t decode_two_bit_whole(float* __restrict__ op,
       __asm__ volatile("" ::: "memory");
     }
   };
-  // One sub-tile at a time: requesting the next one ahead does not help, because the compiler lets a fold
-  // wait for every load in flight, the new ones included; more waves per SIMD hide the latency instead.
   float4 acc0[kDIters];
   uint32_t dw0[NS];
   for (uint32_t rep = 0; rep < nfull; rep++) {
@@ -1217,7 +1215,7 @@ __global__ __launch_bounds__(kThreads) void terngrad_decode_multi_kernel(const M
       for (int jj = 0; jj < 8; jj++) {
         dw[jj] = 0u;
         if (j0 + jj < ns && lane < uint32_t(kDIters * kWave / 4))
-          dw[jj] = reinterpret_cast<const u32u*>(s_pay[j0 + jj] + gw + lane * 4)->v;  // the payload starts at byte 10
+          dw[jj] = as_global(reinterpret_cast<const u32u*>(s_pay[j0 + jj] + gw + lane * 4))->v;  // the payload starts at byte 10
       }
 #pragma unroll
       for (int jj = 0; jj < 8; jj++) {
