@@ -50,6 +50,13 @@ const char* hpx_last_error(void);
  * No call may be in flight.  No counterpart in the reference (its scratch is
  * the caller's output buffer). */
 int hpx_release_workspaces(void);
+/* Waits for `stream`, then frees the workspace the library keeps for (current
+ * device, stream) and hands back the stream's claim on the grid-barrier kernels
+ * (see hpx_terngrad_encode), so that another stream can take it.  Call it before
+ * destroying a stream on which codecs ran; no other call may use the stream at
+ * the same time.  A stream that is used again afterwards simply gets a new
+ * workspace.  No counterpart in the reference. */
+int hpx_release_stream(hpx_stream_t stream);
 
 /* ---- tuning options -------------------------------------------------------
  * No counterpart in the reference.  An option starts from the environment
@@ -139,10 +146,21 @@ int hpx_tbq_decode(int count, float* const* outs, const int32_t* sizes,
  * barrier needs every CU of the device to be reachable from `stream` (no CU
  * mask), and two such kernels must never run at once, so per device only the
  * first stream that encodes a large tensor uses this kernel (other streams keep
- * to the two-launch path).  The wait is bounded: if it ever expires (the GPU is
- * shared with another process's barrier kernels, say) the call's output is
- * invalid, the NEXT hpx_terngrad_encode on the stream returns -2 once and the
- * stream falls back to the two-launch path for good.
+ * to the two-launch path; hpx_release_stream hands the claim back).  The wait is
+ * bounded: if it ever expires (the GPU is shared with another process's barrier
+ * kernels, say) that launch leaves its message unwritten.  The library keeps a
+ * record of every tensor such a launch encoded; hpx_terngrad_encode_status
+ * (below) waits for the stream and, if a barrier expired, encodes those tensors
+ * again through the two-launch path, with the seeds they were given, so the
+ * message that should have come out does.  A later hpx_terngrad_encode on the
+ * stream that finds the expiry does the same before its own work, without
+ * waiting.  Either way the stream keeps to the two-launch path from then on.
+ * The reference's driver returns with a valid message (it synchronises,
+ * hp_cuda_kernel.cu:30-65): a caller that reads a message on the host, or hands
+ * it on, calls hpx_terngrad_encode_status first, and leaves the inputs
+ * untouched until then.
+ * Not recordable into a HIP graph (per-call tags travel in the kernel
+ * arguments): returns -3 on a stream that is being captured.
  * A call with several tensors is first cut into groups of consecutive tensors
  * of one bit width and rounding mode (at most 192) that fit the chip together;
  * a group of two or more that adds up to "terngrad_resident_min" elements is
@@ -153,6 +171,19 @@ int hpx_terngrad_encode(int count, const float* const* ins, const int32_t* in_si
                         uint8_t* const* outs, const int32_t* out_sizes,
                         const uint8_t* bitwidths, const int32_t* enable_randoms,
                         const uint64_t* seeds, hpx_stream_t stream);
+
+/* The completion contract of hp_cuda_terngrad (hp_cuda_kernel.cu:30-65 returns
+ * only once terngrad_body has synchronised and the message is complete,
+ * terngrad_body.h:195, :273).  Returns 0 at once if no grid-barrier launch of
+ * hpx_terngrad_encode is outstanding on `stream` (the two-launch path cannot
+ * fail).  Otherwise waits for the stream; if a barrier wait expired, encodes the
+ * tensors of those launches again through the two-launch path on the same
+ * stream and waits for that too.  On return 0 every message of every
+ * hpx_terngrad_encode call made on the stream so far is valid; -2 if the repair
+ * itself failed.  hpx_terngrad_repaired counts the tensors ever encoded again
+ * on the stream (a diagnostic). */
+int hpx_terngrad_encode_status(hpx_stream_t stream);
+int64_t hpx_terngrad_repaired(hpx_stream_t stream);
 
 /* Replaces hp_cuda_terngradr (hp_cuda.cpp:31-38, hp_cuda_kernel.cu:200-230;
  * body terngrad_body.h:309-409).  The header is parsed on the device, so the
@@ -187,7 +218,8 @@ int hpx_terngrad_decode_status(hpx_stream_t stream);
  * Unlike the reference, bytes of outs[t] past the message are left untouched
  * (scratch lives in the library workspace), so outs[t] needs only
  * 4 + 8*ceil(N*(1-drop)) bytes.  The call waits for the stream once per tensor
- * (the reference waits three times). */
+ * (the reference waits three times) and therefore returns -3 on a stream that
+ * is being captured into a graph; so do hpx_gd_decode and the two DGC calls. */
 int hpx_gd_encode(int count, const float* const* grads, const int32_t* Ns,
                   float* const* residuals, uint8_t* const* outs,
                   const double* sample_rates, const double* drop_ratios,

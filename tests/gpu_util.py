@@ -87,3 +87,9 @@ class Terngrad:
 
     def status(self):
         return self.L.hpx_terngrad_decode_status(stream_ptr())
+
+    def encode_status(self):
+        return self.L.hpx_terngrad_encode_status(stream_ptr())
+
+    def repaired(self):
+        return self.L.hpx_terngrad_repaired(stream_ptr())

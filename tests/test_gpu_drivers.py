@@ -69,6 +69,34 @@ def test_terngrad_drivers(drv, oracle_cpu):
         assert float(np.abs(host(outs[i]) - xs[i]).max()) <= gap * 1.001 + 1e-7
 
 
+def test_terngrad_driver_returns_a_valid_message_when_the_barrier_expires(drv, oracle_cpu, capi):
+    # The reference's hp_cuda_terngrad never returns with an invalid message (hp_cuda_kernel.cu:30-65).  Here only
+    # the single-launch encode, which waits at a grid barrier, can fail to write one; its bound is set to zero
+    # from the host, so every workgroup gives up and leaves normally, and the driver must still hand back the
+    # message of THIS call (it asks hpx_terngrad_encode_status, which encodes again through the other kernels).
+    rng = np.random.default_rng(40)
+    n = 3_000_001
+    x = rng.normal(0, 1e-2, n).astype(np.float32)
+    rc, ref = oracle_cpu.terngrad_encode(x, 2, 0, 0)       # round to nearest: the driver takes its seed from the clock
+    L = capi.load()
+    torch.cuda.synchronize()
+    assert L.hpx_release_workspaces() == 0                  # this stream becomes the owner of the barrier kernels
+    old = [capi.set_option("terngrad_resident_min", 1 << 21), capi.set_option("terngrad_resident_bucket", 0),
+           capi.set_option("terngrad_barrier_ms", 0)]
+    try:
+        dx = dev(x)
+        msg = torch.full((ref.size,), 0x5A, dtype=torch.uint8, device="cuda")
+        torch.cuda.synchronize()
+        drv.hp_cuda_terngrad([dx], [msg], [2], [0])
+        assert L.hpx_terngrad_repaired(torch.cuda.current_stream().cuda_stream) == 1   # the barrier did expire
+        assert_bits_equal(host(msg), ref, "message of the call whose barrier expired")
+    finally:
+        for name, v in zip(("terngrad_resident_min", "terngrad_resident_bucket", "terngrad_barrier_ms"), old):
+            capi.set_option(name, v)
+        torch.cuda.synchronize()
+        assert L.hpx_release_workspaces() == 0
+
+
 def test_graddrop_drivers(drv, oracle_cpu):
     rng = np.random.default_rng(5)
     n, sr, dr_ = 500_009, 0.02, 0.99

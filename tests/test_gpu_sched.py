@@ -93,6 +93,41 @@ def test_terngrad_comp_decomp_root(hp, oracle_cpu, pinned):
     assert hp.error_count() == 0, hp.last_error()
 
 
+def test_terngrad_comp_task_survives_an_expired_barrier(hp, oracle_cpu, capi):
+    # A COMP task whose tensor takes the single-launch encode, with that kernel's barrier bound forced to zero
+    # from the host (all workgroups give up and leave normally): the scheduler asks for the encode status
+    # before it copies B to C, so the name is published with the valid message of that very task in C.
+    rng = np.random.default_rng(41)
+    n, b, seed = 3_000_001, 2, 77
+    x = rng.normal(0, 1e-2, n).astype(np.float32)
+    rc, ref = oracle_cpu.terngrad_encode(x, b, 1, seed)
+    L = capi.load()
+    torch.cuda.synchronize()
+    assert L.hpx_release_workspaces() == 0                  # the worker's compute stream will own the barrier kernels
+    old = [capi.set_option("terngrad_resident_min", 1 << 21), capi.set_option("terngrad_resident_bucket", 0),
+           capi.set_option("terngrad_barrier_ms", 0)]
+    L.hpx_profile_reset(); L.hpx_profile_enable(1)
+    try:
+        assert hp.init("terngrad", {"enable_random": 1, "bitwidth": b, "seed": seed}, 0, 0, 2)
+        dx = dev(x)
+        B = torch.full((ref.size,), 0x5A, dtype=torch.uint8, device="cuda")
+        Cc = _host_buf(ref.size, 1)
+        torch.cuda.synchronize()
+        assert hp.submit_task("big.weight", dx, B, Cc, 0, 10)
+        _collect(hp, 10, ["big.weight"])
+        assert_bits_equal(Cc.numpy(), ref, "COMP message in C after the barrier expired")
+        assert hp.error_count() == 0, hp.last_error()
+        assert capi.profile_query("terngrad_resident_kernel")[1] == 1      # the single-launch encode ran (and gave up) ...
+        assert capi.profile_query("terngrad_quant_kernel")[1] == 1         # ... and the two-launch path encoded it again
+    finally:
+        L.hpx_profile_enable(0); L.hpx_profile_reset()
+        for name, v in zip(("terngrad_resident_min", "terngrad_resident_bucket", "terngrad_barrier_ms"), old):
+            capi.set_option(name, v)
+        hp.end()
+        torch.cuda.synchronize()
+        assert L.hpx_release_workspaces() == 0
+
+
 @pytest.mark.parametrize("lo,hi,count", [(5, 70_000, 24), (2 << 20, 5 << 20, 18)])
 def test_tbq_batch_of_mixed_tasks(hp, oracle_cpu, lo, hi, count):
     # the large case: messages of 0.5 to 1.25 MB, so the batch's transfers and codec calls are cut into several runs

@@ -323,11 +323,17 @@ def test_resident_and_tiled_tensors_in_one_call(tg, oracle_cpu, resident_from_2m
     _check(tg, oracle_cpu, xs, [2, 4, 1, 8, 2, 2], [1, 0, 1, 1, 0, 1], [5, 6, 7, 8, 9, 10], [0] * len(sizes), rng)
 
 
-def test_resident_barrier_expiry_is_reported(tg, oracle_cpu, capi, resident_from_2m):
-    # A zero bound makes the barrier wait give up at once: every workgroup still leaves normally, the
-    # next encode on that stream reports it, and the stream then uses the two-launch path.
+def test_resident_barrier_expiry_is_repaired(tg, oracle_cpu, capi, resident_from_2m):
+    # A zero bound makes the barrier wait give up at once: every workgroup still leaves normally and the
+    # launch writes no message.  hpx_terngrad_encode_status then finds the expiry and encodes the SAME
+    # call's tensor again through the two-launch path: the message of that call is valid when it returns,
+    # as the reference's driver guarantees (hp_cuda_kernel.cu:30-65).  The stream keeps to the two-launch
+    # path afterwards.
     rng = np.random.default_rng(5)
     x = rng.normal(0, 1e-2, 3_000_000).astype(np.float32)
+    y = rng.normal(0, 1e-2, 2_500_003).astype(np.float32)
+    rc, ref_x = oracle_cpu.terngrad_encode(x, 2, 1, 9)
+    rc, ref_y = oracle_cpu.terngrad_encode(y, 4, 1, 10)
     side = torch.cuda.Stream()
     # Only one stream per device may launch barrier kernels (the first that asks): forget the
     # workspaces so that the side stream becomes that stream here, and again afterwards so that the
@@ -337,20 +343,108 @@ def test_resident_barrier_expiry_is_reported(tg, oracle_cpu, capi, resident_from
     old_ms = capi.set_option("terngrad_barrier_ms", 0)
     try:
         with torch.cuda.stream(side):
-            dx = dev(x)
-            tg.encode([dx], [2], [1], [9])
+            dx, dy = dev(x), dev(y)
+            assert tg.encode_status() == 0                     # nothing outstanding: returns at once
+            out = torch.full((tg.packed_size(x.size, 2),), 0x5A, dtype=torch.uint8, device="cuda")
+            tg.encode([dx], [2], [1], [9], outs=[out])
+            assert tg.encode_status() == 0, capi.last_error()
+            assert tg.repaired() == 1
+            assert_bits_equal(host(out), ref_x, "the expired call's own message after the status call")
+            capi.set_option("terngrad_barrier_ms", old_ms)
+            out2 = tg.encode([dx], [2], [1], [9])[0]           # two-launch path from now on
+            assert tg.encode_status() == 0 and tg.repaired() == 1
+            side.synchronize()
+            assert_bits_equal(host(out2), ref_x, "message after fallback")
+        # The same without a status call in between: the next encode on the stream finds the expiry and
+        # queues the repair before its own work.
+        torch.cuda.synchronize()
+        assert capi.load().hpx_release_workspaces() == 0
+        capi.set_option("terngrad_barrier_ms", 0)
+        with torch.cuda.stream(side):
+            out = torch.full((tg.packed_size(x.size, 2),), 0x5A, dtype=torch.uint8, device="cuda")
+            tg.encode([dx], [2], [1], [9], outs=[out])
             side.synchronize()
             capi.set_option("terngrad_barrier_ms", old_ms)
-            tg.encode([dx], [2], [1], [9], expect_rc=-2)
-            assert "barrier" in capi.last_error()
-            out = tg.encode([dx], [2], [1], [9])[0]
-            side.synchronize()
-            rc, ref = oracle_cpu.terngrad_encode(x, 2, 1, 9)
-            assert_bits_equal(host(out), ref, "message after fallback")
+            out_y = tg.encode([dy], [4], [1], [10])[0]
+            assert tg.repaired() == 1
+            assert tg.encode_status() == 0, capi.last_error()
+            assert_bits_equal(host(out), ref_x, "earlier call's message, repaired by the next encode")
+            assert_bits_equal(host(out_y), ref_y, "the next encode's own message")
     finally:
         capi.set_option("terngrad_barrier_ms", old_ms)
         torch.cuda.synchronize()
         assert capi.load().hpx_release_workspaces() == 0
+
+
+def test_release_stream_hands_the_resident_kernel_on(tg, oracle_cpu, capi, resident_from_2m):
+    # The first stream that encodes a large tensor owns the barrier kernels; once it has been released
+    # (as the scheduler's worker does before it destroys its stream) another stream gets them.
+    rng = np.random.default_rng(8)
+    x = rng.normal(0, 1e-2, 3_000_000).astype(np.float32)
+    rc, ref = oracle_cpu.terngrad_encode(x, 2, 1, 9)
+    L = capi.load()
+    torch.cuda.synchronize()
+    assert L.hpx_release_workspaces() == 0
+    a, b = torch.cuda.Stream(), torch.cuda.Stream()
+    capi.load().hpx_profile_enable(1)
+    try:
+        def resident_launches():
+            return capi.profile_query("terngrad_resident_kernel")[1]
+        L.hpx_profile_reset()
+        with torch.cuda.stream(a):
+            dx = dev(x)
+            out_a = tg.encode([dx], [2], [1], [9])[0]
+            a.synchronize()
+        assert resident_launches() == 1
+        with torch.cuda.stream(b):
+            out_b = tg.encode([dx], [2], [1], [9])[0]
+            b.synchronize()
+        assert resident_launches() == 1                       # b does not own them
+        assert L.hpx_release_stream(a.cuda_stream) == 0
+        with torch.cuda.stream(b):
+            out_b2 = tg.encode([dx], [2], [1], [9])[0]
+            b.synchronize()
+        assert resident_launches() == 2                       # now it does
+        for o, what in ((out_a, "owner"), (out_b, "other stream"), (out_b2, "new owner")):
+            assert_bits_equal(host(o), ref, what)
+    finally:
+        L.hpx_profile_enable(0)
+        L.hpx_profile_reset()
+        torch.cuda.synchronize()
+        assert L.hpx_release_workspaces() == 0
+
+
+def test_calls_that_cannot_be_recorded_refuse_a_capturing_stream(tg, capi):
+    # hpx_terngrad_encode tags its kernels per call and the GradDrop calls wait for the stream: recorded into a
+    # graph they would replay stale tags / deadlock.  They return -3 instead; the capture itself ends cleanly.
+    L = capi.load()
+    c = capi
+    x = torch.randn(70_001, device="cuda")
+    r = torch.zeros_like(x)
+    msg = torch.zeros(tg.packed_size(x.numel(), 2), dtype=torch.uint8, device="cuda")
+    gd_out = torch.zeros(4 + 8 * 1024, dtype=torch.uint8, device="cuda")
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        tg.encode([x], [2], [1], [3], outs=[msg])          # eager once: workspaces exist
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            sp = torch.cuda.current_stream().cuda_stream
+            tg.encode([x], [2], [1], [3], outs=[msg], expect_rc=-3)
+            assert "captured" in capi.last_error()
+            assert L.hpx_terngrad_encode_status(sp) == -3
+            assert L.hpx_terngrad_decode_status(sp) == -3
+            rc = L.hpx_gd_encode(1, c.ptr_array([x.data_ptr()]), c.i32_array([x.numel()]), c.ptr_array([r.data_ptr()]),
+                                 c.ptr_array([gd_out.data_ptr()]), c.f64_array([0.05]), c.f64_array([0.99]), c.u64_array([1]), sp)
+            assert rc == -3
+            rc = L.hpx_gd_decode(1, c.ptr_array([gd_out.data_ptr()]), c.i32_array([gd_out.numel()]), c.ptr_array([r.data_ptr()]),
+                                 c.i32_array([r.numel()]), c.i32_array([1]), sp)
+            assert rc == -3
+            r.add_(1.0)                                     # something recordable, so that the graph is not empty
+    graph.replay()
+    torch.cuda.synchronize()
+    assert float(r[0]) == 1.0
 
 
 def test_resident_kernel_belongs_to_one_stream(tg, oracle_cpu, capi, resident_from_2m):
@@ -485,9 +579,9 @@ def test_resident_bucket_groups_of_a_large_call(tg, oracle_cpu, capi, bucket_for
         assert_bits_equal(host(outs[i]), ref, f"message[{i}] b={bws[i]}")
 
 
-def test_resident_bucket_barrier_expiry_is_reported(tg, oracle_cpu, capi, bucket_forced):
-    # As for the single-tensor kernel: with a zero bound every workgroup gives up at the barrier and leaves, the
-    # next encode on the stream reports it, and the stream keeps to the tiled kernels afterwards.
+def test_resident_bucket_barrier_expiry_is_repaired(tg, oracle_cpu, capi, bucket_forced):
+    # As for the single-tensor kernel: with a zero bound every workgroup gives up at the barrier and leaves; the
+    # status call encodes all tensors of that launch again, and the stream keeps to the tiled kernels afterwards.
     rng = np.random.default_rng(35)
     xs = [rng.normal(0, 1e-2, n).astype(np.float32) for n in (1_500_000, 70_001, 900_000)]
     side = torch.cuda.Stream()
@@ -498,12 +592,14 @@ def test_resident_bucket_barrier_expiry_is_reported(tg, oracle_cpu, capi, bucket
         with torch.cuda.stream(side):
             dx = [dev(x) for x in xs]
             before = _bucket_launches(capi)
-            tg.encode(dx, [2] * 3, [1] * 3, [9, 10, 11])
-            side.synchronize()
-            assert _bucket_launches(capi) == before + 1
+            outs = [torch.full((tg.packed_size(x.size, 2),), 0x5A, dtype=torch.uint8, device="cuda") for x in xs]
+            tg.encode(dx, [2] * 3, [1] * 3, [9, 10, 11], outs=outs)
+            assert tg.encode_status() == 0, capi.last_error()
+            assert _bucket_launches(capi) == before + 1 and tg.repaired() == 3
+            for i, x in enumerate(xs):
+                rc, ref = oracle_cpu.terngrad_encode(x, 2, 1, 9 + i)
+                assert_bits_equal(host(outs[i]), ref, f"message[{i}] of the expired call")
             capi.set_option("terngrad_barrier_ms", old_ms)
-            tg.encode(dx, [2] * 3, [1] * 3, [9, 10, 11], expect_rc=-2)
-            assert "barrier" in capi.last_error()
             outs = tg.encode(dx, [2] * 3, [1] * 3, [9, 10, 11])
             side.synchronize()
             assert _bucket_launches(capi) == before + 1

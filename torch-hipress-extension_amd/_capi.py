@@ -14,6 +14,7 @@ SYMBOLS = (
     "hpx_version",
     "hpx_last_error",
     "hpx_release_workspaces",
+    "hpx_release_stream",
     "hpx_set_option",
     "hpx_get_option",
     "hpx_profile_enable",
@@ -23,6 +24,8 @@ SYMBOLS = (
     "hpx_tbq_encode",
     "hpx_tbq_decode",
     "hpx_terngrad_encode",
+    "hpx_terngrad_encode_status",
+    "hpx_terngrad_repaired",
     "hpx_terngrad_decode",
     "hpx_terngrad_decode_status",
     "hpx_gd_encode",
@@ -90,6 +93,10 @@ def load():
     L.hpx_tbq_encode.argtypes = [i32, pp, p, pp, pp, p, p]
     L.hpx_tbq_decode.argtypes = [i32, pp, p, pp, p, p, p]
     L.hpx_terngrad_encode.argtypes = [i32, pp, p, pp, p, p, p, p, p]
+    L.hpx_terngrad_encode_status.argtypes = [p]
+    L.hpx_terngrad_repaired.argtypes = [p]
+    L.hpx_terngrad_repaired.restype = C.c_int64
+    L.hpx_release_stream.argtypes = [p]
     L.hpx_terngrad_decode.argtypes = [i32, pp, p, pp, p, p, p]
     L.hpx_terngrad_decode_status.argtypes = [p]
     L.hpx_gd_encode.argtypes = [i32, pp, p, pp, pp, p, p, p, p]

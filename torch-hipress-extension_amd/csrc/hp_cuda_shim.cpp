@@ -21,6 +21,10 @@ SHIM_API void hp_cuda_terngrad(std::vector<float*>& in_floats, std::vector<int32
   int ret = hpx_terngrad_encode(static_cast<int>(in_floats.size()), cptrs(in_floats), in_float_sizes.data(),
                                 out_uint8_ts.data(), out_uint8_t_sizes.data(), bitwidths.data(),
                                 enable_randoms.data(), nullptr, stream);
+  // The reference returns with complete messages (terngrad_body synchronises, terngrad_body.h:195, :273).
+  // Here only a launch that waits at a grid barrier can fail to write one; the status call waits for such
+  // launches and encodes again what an expired barrier left unwritten.
+  if (!ret) ret = hpx_terngrad_encode_status(stream);
   if (ret) printf("ret=%d %s\n", ret, hpx_last_error());  // hp_cuda_kernel.cu:63
 }
 

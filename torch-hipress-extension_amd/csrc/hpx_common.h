@@ -4,6 +4,7 @@
 #include <stdint.h>
 
 #include <mutex>
+#include <vector>
 
 #include "hpx.h"
 
@@ -70,6 +71,18 @@ struct Workspace {
   uint32_t bar_gen = 0;
   int num_cus = 0;
   bool barrier_broken = false;  // a barrier wait expired on this stream: barrier kernels stay off
+  // Tensors that barrier kernels have encoded on this stream since the stream was last known to be
+  // good: if one of those kernels gave up at its barrier, its messages are encoded again from
+  // these records by the kernels that need no barrier (hpx_terngrad_encode_status).
+  struct ResidentRec {
+    const float* x;
+    uint8_t* out;
+    int32_t n, out_size;
+    uint64_t seed;
+    uint8_t bits, random;
+  };
+  std::vector<ResidentRec> resident_log;
+  uint64_t repaired = 0;  // tensors encoded again after an expired barrier, ever
 };
 constexpr size_t kStateWords = 4096;       // 16 KiB
 constexpr size_t kStatusWord = kStateWords - 16;  // sticky flags live here
@@ -91,12 +104,16 @@ int ensure_barrier(Workspace* ws);
 // for.  So only one stream per device may launch them: the first that asks.
 // Returns whether `ws` is (now) that stream's workspace.
 bool claim_barrier_kernels(Workspace* ws);
-// Call with ws->mu held and the workspace ensured, before queueing work: if a barrier kernel of an
-// earlier call on this stream gave up waiting, reports it once (HPX_ERR_HIP, text names `who`) and
-// turns barrier kernels off for the stream.
-int check_barrier_expired(Workspace* ws, const char* who);
+// Whether a barrier kernel on this stream has raised the pinned expiry flag (ws->mu held, workspace ensured).
+bool barrier_expired(const Workspace* ws);
+// Frees the workspace of (current device, `stream`) and hands back its claim on the barrier kernels.
+int release_stream_workspace(hipStream_t stream);
 
 uint64_t clock_seed();
+
+// HPX_ERR_ARG (text names `who`) when `stream` is being captured into a graph: for entry points that wait for
+// the stream or put per-call tags into their kernel arguments, neither of which a replayed graph could repeat.
+int reject_capture(hipStream_t stream, const char* who);
 
 // Copies `count` byte ranges in as few launches as their number allows (one kernel, a table of ranges in
 // its arguments).  Either side may be device memory or pinned host memory: the scheduler moves all

@@ -773,6 +773,7 @@ HPX_API int hpx_gd_encode(int count, const float* const* grads, const int32_t* N
     HPX_ARG((reinterpret_cast<uintptr_t>(outs[i]) & 3) == 0, "hpx_gd_encode: output %d is not 4-byte aligned", i);
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (const int rcc = hpx::reject_capture(st, "hpx_gd_encode")) return rcc;
   hpx::Workspace* ws = hpx::workspace_record(st);
   if (!ws) return HPX_ERR_HIP;
   std::lock_guard<std::mutex> lock(ws->mu);
@@ -802,6 +803,7 @@ int decode_messages(int count, const uint8_t* const* ins, const int32_t* in_size
     HPX_ARG((reinterpret_cast<uintptr_t>(ins[i]) & 3) == 0, "hpx_gd_decode: message %d is not 4-byte aligned", i);
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (const int rcc = hpx::reject_capture(st, zero_fill ? "hpx_gd_decode" : "hpx_dgc_decode")) return rcc;
   hpx::Workspace* ws = hpx::workspace_record(st);
   if (!ws) return HPX_ERR_HIP;
   std::lock_guard<std::mutex> lock(ws->mu);
@@ -862,6 +864,7 @@ HPX_API int hpx_dgc_encode(int count, float* const* grads, const int32_t* Ns, ui
     HPX_ARG((reinterpret_cast<uintptr_t>(outs[i]) & 3) == 0, "hpx_dgc_encode: output %d is not 4-byte aligned", i);
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (const int rcc = hpx::reject_capture(st, "hpx_dgc_encode")) return rcc;
   hpx::Workspace* ws = hpx::workspace_record(st);
   if (!ws) return HPX_ERR_HIP;
   std::lock_guard<std::mutex> lock(ws->mu);

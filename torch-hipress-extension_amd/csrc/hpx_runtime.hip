@@ -27,6 +27,7 @@ void clear_error() { g_err[0] = 0; }
 
 static std::mutex g_ws_mu;
 static std::map<std::pair<int, hipStream_t>, std::unique_ptr<Workspace>> g_ws;
+static std::map<int, Workspace*> g_barrier_owner;  // guarded by g_ws_mu
 
 Workspace* workspace_record(hipStream_t stream) {
   int device = 0;
@@ -111,8 +112,6 @@ int ensure_slots(Workspace* ws, size_t words) {
   return HPX_OK;
 }
 
-static std::map<int, Workspace*> g_barrier_owner;  // guarded by g_ws_mu
-
 bool claim_barrier_kernels(Workspace* ws) {
   std::lock_guard<std::mutex> g(g_ws_mu);
   auto it = g_barrier_owner.find(ws->device);
@@ -123,14 +122,40 @@ bool claim_barrier_kernels(Workspace* ws) {
   return it->second == ws;
 }
 
-int check_barrier_expired(Workspace* ws, const char* who) {
-  volatile uint32_t* expired = reinterpret_cast<volatile uint32_t*>(ws->pinned + kPinnedFlagOffset);
-  if (!*expired) return HPX_OK;
-  *expired = 0;
-  ws->barrier_broken = true;
-  set_error("%s: the grid barrier of an earlier call on this stream expired; that call's output is invalid. "
-            "Kernels that use a grid barrier are now off for this stream.", who);
-  return HPX_ERR_HIP;
+bool barrier_expired(const Workspace* ws) {
+  return ws->pinned && *reinterpret_cast<volatile const uint32_t*>(ws->pinned + kPinnedFlagOffset) != 0;
+}
+
+namespace {
+int free_workspace(Workspace* ws) {
+  int rc = HPX_OK;
+  if (ws->dev && hipFree(ws->dev) != hipSuccess) rc = HPX_ERR_HIP;
+  if (ws->state && hipFree(ws->state) != hipSuccess) rc = HPX_ERR_HIP;
+  if (ws->slots && hipFree(ws->slots) != hipSuccess) rc = HPX_ERR_HIP;
+  if (ws->bar && hipFree(ws->bar) != hipSuccess) rc = HPX_ERR_HIP;
+  if (ws->pinned && hipHostFree(ws->pinned) != hipSuccess) rc = HPX_ERR_HIP;
+  ws->dev = nullptr; ws->state = nullptr; ws->slots = nullptr; ws->bar = nullptr; ws->pinned = nullptr;
+  return rc;
+}
+}  // namespace
+
+int release_stream_workspace(hipStream_t stream) {
+  int device = 0;
+  HPX_HIP(hipGetDevice(&device));
+  std::unique_ptr<Workspace> ws;
+  {
+    std::lock_guard<std::mutex> g(g_ws_mu);
+    auto it = g_ws.find({device, stream});
+    if (it == g_ws.end()) return HPX_OK;
+    ws = std::move(it->second);
+    g_ws.erase(it);
+    auto own = g_barrier_owner.find(device);
+    if (own != g_barrier_owner.end() && own->second == ws.get()) g_barrier_owner.erase(own);
+  }
+  // Nothing can find the record any more; a call that had found it before holds its mutex until it has queued its work.
+  { std::lock_guard<std::mutex> g(ws->mu); }
+  HPX_HIP(hipStreamSynchronize(stream));
+  return free_workspace(ws.get());
 }
 
 int ensure_barrier(Workspace* ws) {
@@ -310,6 +335,18 @@ __global__ __launch_bounds__(kProbeThreads) void probe_stream_kernel(float* __re
 }
 }  // namespace
 
+int reject_capture(hipStream_t stream, const char* who) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
+    (void)hipGetLastError();  // the query itself is refused for some streams while another one captures: not this call's business
+    return HPX_OK;
+  }
+  if (status == hipStreamCaptureStatusNone) return HPX_OK;
+  set_error("%s: the stream is being captured into a graph; this entry point cannot be recorded "
+            "(it waits for the stream or tags its kernels per call)", who);
+  return HPX_ERR_ARG;
+}
+
 uint64_t clock_seed() {
   return static_cast<uint64_t>(
       std::chrono::high_resolution_clock::now().time_since_epoch().count());
@@ -330,16 +367,17 @@ HPX_API int hpx_release_workspaces(void) {
     hpx::Workspace* ws = kv.second.get();
     std::lock_guard<std::mutex> g2(ws->mu);
     if (hipSetDevice(ws->device) != hipSuccess) { rc = HPX_ERR_HIP; continue; }
-    if (ws->dev && hipFree(ws->dev) != hipSuccess) rc = HPX_ERR_HIP;
-    if (ws->state && hipFree(ws->state) != hipSuccess) rc = HPX_ERR_HIP;
-    if (ws->slots && hipFree(ws->slots) != hipSuccess) rc = HPX_ERR_HIP;
-    if (ws->bar && hipFree(ws->bar) != hipSuccess) rc = HPX_ERR_HIP;
-    if (ws->pinned && hipHostFree(ws->pinned) != hipSuccess) rc = HPX_ERR_HIP;
+    if (hpx::free_workspace(ws) != HPX_OK) rc = HPX_ERR_HIP;
   }
   hpx::g_ws.clear();
   hpx::g_barrier_owner.clear();
   if (cur >= 0) (void)hipSetDevice(cur);
   return rc;
+}
+
+HPX_API int hpx_release_stream(hpx_stream_t stream) {
+  hpx::clear_error();
+  return hpx::release_stream_workspace(static_cast<hipStream_t>(stream));
 }
 
 HPX_API int hpx_set_option(const char* name, int64_t value) {

@@ -384,6 +384,10 @@ void run_codec_batch(Worker& w, const Params& p, const std::vector<Task>& batch)
       std::vector<int32_t> rnd(n, p.enable_random);
       codec(hpx_terngrad_encode(n, in.data(), in_size.data(), out.data(), out_size.data(), bw.data(), rnd.data(),
                                 p.has_seed ? seeds.data() : nullptr, w.compute), what);
+      // Before the messages leave B: a launch that waits at a grid barrier is the one kind that can fail to
+      // write its message.  Returns at once when the run took none; otherwise waits for the compute stream
+      // and encodes again what an expired barrier left unwritten.
+      codec(hpx_terngrad_encode_status(w.compute), "hpx_terngrad_encode_status");
     } else if (p.alg == kTbq) {
       std::vector<float> thr(n, p.threshold);
       codec(hpx_tbq_encode(n, in.data(), in_size.data(), res.data(), out.data(), thr.data(), w.compute), what);
@@ -570,6 +574,10 @@ void worker_main() {
   for (hipEvent_t e : w.events) (void)hipEventDestroy(e);
   w.pinned_arena.release();
   w.device_arena.release();
+  // The codec workspaces of the two streams go with them, and with the compute stream's its claim on the
+  // grid-barrier kernels: the worker of a later init() gets the resident TernGrad encode again.
+  (void)hpx_release_stream(w.compute);
+  (void)hpx_release_stream(w.data);
   (void)hipStreamDestroy(w.compute);
   (void)hipStreamDestroy(w.data);
 }

@@ -1516,7 +1516,9 @@ int launch_resident(const ResArgs& ra, int num_cus, hipStream_t st) {
 template <int CAP>
 int launch_encode(int count, const float* const* ins, const int32_t* in_sizes, uint8_t* const* outs,
                   const int32_t* out_sizes, const uint8_t* bitwidths, const int32_t* enable_randoms,
-                  const uint64_t* seeds, uint64_t* slot_base, uint32_t epoch, hipStream_t st) {
+                  const uint64_t* seeds, uint64_t* slot_base, uint32_t epoch, hipStream_t st, bool timed = true) {
+  // timed = false: the launches are never bracketed by profiling events (creating an event allocates)
+  const bool prof = timed && hpx::g_prof_on;
   EncArgs<CAP> a;
   int i = 0;
   while (i < count) {
@@ -1542,10 +1544,14 @@ int launch_encode(int count, const float* const* ins, const int32_t* in_sizes, u
       a.nseg++;
       i++;
     }
-    HPX_LAUNCH("terngrad_minmax_kernel", terngrad_minmax_kernel<CAP>, dim3(a.tile_start[a.nseg]), dim3(kThreads), st, a);
+    if (prof) hpx::prof_begin("terngrad_minmax_kernel", st);
+    hipLaunchKernelGGL(terngrad_minmax_kernel<CAP>, dim3(a.tile_start[a.nseg]), dim3(kThreads), 0, st, a);
+    if (prof) hpx::prof_end(st);
     HPX_HIP(hipGetLastError());
     for (int k = 0; k <= a.nseg; k++) a.tile_start[k] = qstart[k];
-    HPX_LAUNCH("terngrad_quant_kernel", terngrad_quant_kernel<CAP>, dim3(a.tile_start[a.nseg]), dim3(kThreads), st, a);
+    if (prof) hpx::prof_begin("terngrad_quant_kernel", st);
+    hipLaunchKernelGGL(terngrad_quant_kernel<CAP>, dim3(a.tile_start[a.nseg]), dim3(kThreads), 0, st, a);
+    if (prof) hpx::prof_end(st);
     HPX_HIP(hipGetLastError());
   }
   return HPX_OK;
@@ -1656,6 +1662,62 @@ int launch_decode_multi(int count, float* const* outs, const int32_t* out_sizes,
   return HPX_OK;
 }
 
+// Encodes the listed tensors with the tiled pair of kernels (ws->mu held).  `seeds` may be null (wall clock).
+int encode_tiled(hpx::Workspace* ws, hipStream_t st, int count, const float* const* ins, const int32_t* in_sizes,
+                 uint8_t* const* outs, const int32_t* out_sizes, const uint8_t* bitwidths, const int32_t* enable_randoms,
+                 const uint64_t* seeds) {
+  int rc = hpx::ensure_slots(ws, size_t(count) * kSlotsPerTensor);
+  if (rc != HPX_OK) return rc;
+  rc = next_slot_epoch(ws, st);  // its own tag: the slots may hold words of an earlier launch of the same call
+  if (rc != HPX_OK) return rc;
+  if (count <= kCapSmall)
+    return launch_encode<kCapSmall>(count, ins, in_sizes, outs, out_sizes, bitwidths, enable_randoms, seeds, ws->slots,
+                                    ws->epoch, st);
+  return launch_encode<kCapLarge>(count, ins, in_sizes, outs, out_sizes, bitwidths, enable_randoms, seeds, ws->slots,
+                                  ws->epoch, st);
+}
+
+// A barrier kernel on this stream gave up waiting (ws->mu held): barrier kernels are switched off for the
+// stream and every tensor they have encoded since the stream was last known to be good is queued again
+// through the tiled kernels, with the seed it was given the first time, so the same message comes out.
+int repair_resident_log(hpx::Workspace* ws, hipStream_t st) {
+  ws->barrier_broken = true;
+  if (ws->resident_log.empty()) return HPX_OK;
+  const int m = int(ws->resident_log.size());
+  std::vector<const float*> t_in(m);
+  std::vector<uint8_t*> t_out(m);
+  std::vector<int32_t> t_isz(m), t_osz(m), t_rnd(m);
+  std::vector<uint8_t> t_bits(m);
+  std::vector<uint64_t> t_seed(m);
+  for (int k = 0; k < m; k++) {
+    const hpx::Workspace::ResidentRec& r = ws->resident_log[k];
+    t_in[k] = r.x; t_out[k] = r.out; t_isz[k] = r.n; t_osz[k] = r.out_size;
+    t_rnd[k] = r.random; t_bits[k] = r.bits; t_seed[k] = r.seed;
+  }
+  ws->resident_log.clear();
+  ws->repaired += uint64_t(m);
+  return encode_tiled(ws, st, m, t_in.data(), t_isz.data(), t_out.data(), t_osz.data(), t_bits.data(), t_rnd.data(),
+                      t_seed.data());
+}
+
+// Waits for the stream and settles the log of barrier-kernel encodes: cleared if they all got through, encoded
+// again if one gave up (ws->mu held).
+int settle_resident_log(hpx::Workspace* ws, hipStream_t st) {
+  HPX_HIP(hipStreamSynchronize(st));
+  if (!hpx::barrier_expired(ws)) {
+    ws->resident_log.clear();
+    return HPX_OK;
+  }
+  // every kernel of the stream has finished: nothing can raise the flag again behind this
+  *reinterpret_cast<volatile uint32_t*>(ws->pinned + hpx::kPinnedFlagOffset) = 0;
+  const int rc = repair_resident_log(ws, st);
+  if (rc != HPX_OK) return rc;
+  HPX_HIP(hipStreamSynchronize(st));
+  return HPX_OK;
+}
+
+constexpr size_t kResidentLogMax = 4096;  // records kept before hpx_terngrad_encode settles the log itself
+
 }  // namespace
 
 HPX_API int hpx_terngrad_encode(int count, const float* const* ins, const int32_t* in_sizes,
@@ -1680,19 +1742,30 @@ HPX_API int hpx_terngrad_encode(int count, const float* const* ins, const int32_
             static_cast<long long>(need), out_sizes[i]);
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
+  int rc = hpx::reject_capture(st, "hpx_terngrad_encode");
+  if (rc != HPX_OK) return rc;
   hpx::Workspace* ws = hpx::workspace_record(st);
   if (!ws) return HPX_ERR_HIP;
   std::lock_guard<std::mutex> lock(ws->mu);
-  int rc = hpx::ensure_workspace(ws, 0);
+  rc = hpx::ensure_workspace(ws, 0);
   if (rc != HPX_OK) return rc;
   rc = hpx::ensure_slots(ws, size_t(count) * kSlotsPerTensor);
   if (rc != HPX_OK) return rc;
   rc = hpx::ensure_barrier(ws);
   if (rc != HPX_OK) return rc;
 
-  // Large tensors take the single-launch resident kernel, the rest the tiled pair.
-  rc = hpx::check_barrier_expired(ws, "hpx_terngrad_encode");
-  if (rc != HPX_OK) return rc;
+  // A barrier kernel of an earlier call on this stream gave up waiting: its messages are queued again
+  // through the tiled kernels before this call's work, and this call takes the tiled kernels too.  (The
+  // flag stays up until hpx_terngrad_encode_status has waited for the stream: workgroups of that
+  // kernel may still be on their way out.)
+  if (!ws->barrier_broken && hpx::barrier_expired(ws)) {
+    rc = repair_resident_log(ws, st);
+    if (rc != HPX_OK) return rc;
+  }
+  if (ws->resident_log.size() + size_t(count) > kResidentLogMax) {
+    rc = settle_resident_log(ws, st);
+    if (rc != HPX_OK) return rc;
+  }
   uint32_t* expired = reinterpret_cast<uint32_t*>(ws->pinned + hpx::kPinnedFlagOffset);
   // Consecutive tensors of one width and rounding mode that fit the chip together and add up to the
   // resident threshold take one resident launch per such group; a remaining tensor that is large enough
@@ -1701,6 +1774,9 @@ HPX_API int hpx_terngrad_encode(int count, const float* const* ins, const int32_
   tiled.reserve(count);
   const bool buckets = count >= 2 && hpx::option(hpx::kOptTerngradResidentBucket) != 0 &&
                        hpx::option(hpx::kOptTerngradResidentMin) >= 0;
+  auto log_resident = [&](const EncSeg& sg, uint64_t seed) {
+    ws->resident_log.push_back(hpx::Workspace::ResidentRec{sg.x, sg.out, sg.n, sg.out_size, seed, sg.bits, sg.random});
+  };
   int i = 0;
   while (i < count) {
     int j = i;
@@ -1714,6 +1790,7 @@ HPX_API int hpx_terngrad_encode(int count, const float* const* ins, const int32_
           const uint64_t seed = seeds ? seeds[k] : hpx::clock_seed();
           ma.seg[k - i] = EncSeg{ins[k], outs[k], in_sizes[k], out_sizes[k], static_cast<uint32_t>(seed), bitwidths[k],
                                  static_cast<uint8_t>(enable_randoms[k] != 0), 0};
+          log_resident(ma.seg[k - i], seed);
         }
         rc = next_barrier_generation(ws, st);
         if (rc != HPX_OK) return rc;
@@ -1743,6 +1820,7 @@ HPX_API int hpx_terngrad_encode(int count, const float* const* ins, const int32_
       const uint64_t seed = seeds ? seeds[i] : hpx::clock_seed();
       ra.seg = EncSeg{ins[i], outs[i], in_sizes[i], out_sizes[i], static_cast<uint32_t>(seed), bitwidths[i],
                       static_cast<uint8_t>(enable_randoms[i] != 0), 0};
+      log_resident(ra.seg, seed);
       rc = next_barrier_generation(ws, st);
       if (rc != HPX_OK) return rc;
       ra.gen = ws->bar_gen;
@@ -1754,15 +1832,8 @@ HPX_API int hpx_terngrad_encode(int count, const float* const* ins, const int32_
     }
   }
   if (tiled.empty()) return HPX_OK;
-  rc = next_slot_epoch(ws, st);  // its own tag: the slots may hold words of a resident launch of this call
-  if (rc != HPX_OK) return rc;
-  if (int(tiled.size()) == count) {
-    if (count <= kCapSmall)
-      return launch_encode<kCapSmall>(count, ins, in_sizes, outs, out_sizes, bitwidths, enable_randoms, seeds,
-                                      ws->slots, ws->epoch, st);
-    return launch_encode<kCapLarge>(count, ins, in_sizes, outs, out_sizes, bitwidths, enable_randoms, seeds, ws->slots,
-                                    ws->epoch, st);
-  }
+  if (int(tiled.size()) == count)
+    return encode_tiled(ws, st, count, ins, in_sizes, outs, out_sizes, bitwidths, enable_randoms, seeds);
   const int m = int(tiled.size());
   std::vector<const float*> t_in(m);
   std::vector<uint8_t*> t_out(m);
@@ -1775,11 +1846,29 @@ HPX_API int hpx_terngrad_encode(int count, const float* const* ins, const int32_
     t_rnd[k] = enable_randoms[i]; t_bits[k] = bitwidths[i];
     t_seed[k] = seeds ? seeds[i] : hpx::clock_seed();
   }
-  if (m <= kCapSmall)
-    return launch_encode<kCapSmall>(m, t_in.data(), t_isz.data(), t_out.data(), t_osz.data(), t_bits.data(),
-                                    t_rnd.data(), t_seed.data(), ws->slots, ws->epoch, st);
-  return launch_encode<kCapLarge>(m, t_in.data(), t_isz.data(), t_out.data(), t_osz.data(), t_bits.data(), t_rnd.data(),
-                                  t_seed.data(), ws->slots, ws->epoch, st);
+  return encode_tiled(ws, st, m, t_in.data(), t_isz.data(), t_out.data(), t_osz.data(), t_bits.data(), t_rnd.data(),
+                      t_seed.data());
+}
+
+HPX_API int hpx_terngrad_encode_status(hpx_stream_t stream) {
+  hpx::clear_error();
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  int rc = hpx::reject_capture(st, "hpx_terngrad_encode_status");
+  if (rc != HPX_OK) return rc;
+  hpx::Workspace* ws = hpx::workspace_record(st);
+  if (!ws) return HPX_ERR_HIP;
+  std::lock_guard<std::mutex> lock(ws->mu);
+  if (!ws->pinned) return HPX_OK;  // nothing has been encoded on this stream
+  if (ws->resident_log.empty() && !hpx::barrier_expired(ws)) return HPX_OK;  // no barrier kernel is outstanding
+  return settle_resident_log(ws, st);
+}
+
+HPX_API int64_t hpx_terngrad_repaired(hpx_stream_t stream) {
+  hpx::clear_error();
+  hpx::Workspace* ws = hpx::workspace_record(static_cast<hipStream_t>(stream));
+  if (!ws) return -1;
+  std::lock_guard<std::mutex> lock(ws->mu);
+  return int64_t(ws->repaired);
 }
 
 HPX_API int hpx_terngrad_decode(int count, float* const* outs, const int32_t* out_sizes,
@@ -1815,6 +1904,7 @@ HPX_API int hpx_terngrad_decode(int count, float* const* outs, const int32_t* ou
 HPX_API int hpx_terngrad_decode_status(hpx_stream_t stream) {
   hpx::clear_error();
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (const int rcc = hpx::reject_capture(st, "hpx_terngrad_decode_status")) return rcc;
   hpx::Workspace* ws = hpx::workspace_record(st);
   if (!ws) return HPX_ERR_HIP;
   std::lock_guard<std::mutex> lock(ws->mu);
