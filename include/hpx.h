@@ -185,6 +185,22 @@ int hpx_terngrad_encode(int count, const float* const* ins, const int32_t* in_si
 int hpx_terngrad_encode_status(hpx_stream_t stream);
 int64_t hpx_terngrad_repaired(hpx_stream_t stream);
 
+/* hpx_terngrad_encode for callers that cannot allocate: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart
+ * in the reference.  Same arguments, same bytes out; always the two-launch path
+ * (min/max, then quantise), whose reduction slots live in a fixed device array
+ * of 576 KiB inside the library instead of a workspace, so the call makes no
+ * hipMalloc / hipFree, takes no workspace, never waits for the stream and puts
+ * no per-call tag into its kernels (it clears the slots it uses with a small
+ * kernel first), which also makes it recordable into a graph (seeds == NULL then
+ * freezes the clock value of the capture).  Limits: at most 192 tensors per call
+ * (-3 beyond that).  Every call on a GPU shares that GPU's array: calls that
+ * overlap in time on one GPU - on any streams - race; order them. */
+int hpx_terngrad_encode_noalloc(int count, const float* const* ins, const int32_t* in_sizes,
+                                uint8_t* const* outs, const int32_t* out_sizes,
+                                const uint8_t* bitwidths, const int32_t* enable_randoms,
+                                const uint64_t* seeds, hpx_stream_t stream);
+
 /* Replaces hp_cuda_terngradr (hp_cuda.cpp:31-38, hp_cuda_kernel.cu:200-230;
  * body terngrad_body.h:309-409).  The header is parsed on the device, so the
  * call does not wait for the stream (the reference copies it to the host and

@@ -93,3 +93,14 @@ class Terngrad:
 
     def repaired(self):
         return self.L.hpx_terngrad_repaired(stream_ptr())
+
+    def encode_noalloc(self, xs, bits_, randoms, seeds, outs=None, expect_rc=0):
+        c = self.c
+        if outs is None:
+            outs = [torch.zeros(self.packed_size(x.numel(), b), dtype=torch.uint8, device="cuda") for x, b in zip(xs, bits_)]
+        rc = self.L.hpx_terngrad_encode_noalloc(len(xs), c.ptr_array([x.data_ptr() for x in xs]), c.i32_array([x.numel() for x in xs]),
+                                                c.ptr_array([o.data_ptr() for o in outs]), c.i32_array([o.numel() for o in outs]),
+                                                c.u8_array(bits_), c.i32_array(randoms),
+                                                c.u64_array(seeds) if seeds is not None else None, stream_ptr())
+        assert rc == expect_rc, (rc, c.last_error())
+        return outs

@@ -26,6 +26,7 @@ SYMBOLS = (
     "hpx_terngrad_encode",
     "hpx_terngrad_encode_status",
     "hpx_terngrad_repaired",
+    "hpx_terngrad_encode_noalloc",
     "hpx_terngrad_decode",
     "hpx_terngrad_decode_status",
     "hpx_gd_encode",
@@ -93,6 +94,7 @@ def load():
     L.hpx_tbq_encode.argtypes = [i32, pp, p, pp, pp, p, p]
     L.hpx_tbq_decode.argtypes = [i32, pp, p, pp, p, p, p]
     L.hpx_terngrad_encode.argtypes = [i32, pp, p, pp, p, p, p, p, p]
+    L.hpx_terngrad_encode_noalloc.argtypes = [i32, pp, p, pp, p, p, p, p, p]
     L.hpx_terngrad_encode_status.argtypes = [p]
     L.hpx_terngrad_repaired.argtypes = [p]
     L.hpx_terngrad_repaired.restype = C.c_int64

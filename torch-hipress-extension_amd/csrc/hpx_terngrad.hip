@@ -34,6 +34,11 @@
 
 #include "hpx_common.h"
 
+// Reduction slots of hpx_terngrad_encode_noalloc: 192 tensors x 3 x 128 words of 8 bytes = 576 KiB, held by
+// every GPU the library runs on until the process ends.  In host code this name only stands for the
+// symbol; the device address comes from hipGetSymbolAddress (scratch_address below).
+static __device__ __align__(256) unsigned long long scratch[192 * 3 * 128];
+
 namespace {
 using namespace hpx;
 
@@ -50,7 +55,7 @@ constexpr int kDecTile = kThreads * kDIters * 4;
 // Per tensor, 3 x kSlotWays epoch-tagged slots: first the largest ordered key of x, then the
 // largest complemented key (i.e. the minimum), then the largest complemented
 // index of a tile that holds a zero (i.e. the first such tile).
-constexpr int kSlotWays = 128;  // a multiple of 64; with 64 the min/max pass over one 25.5 M tensor took 24.1 us, with 128 or 256: 20.2
+constexpr int kSlotWays = 128;  // a multiple of 64 (the size of `scratch` above is written out from this and kCapLarge); with 64 the min/max pass over one 25.5 M tensor took 24.1 us, with 128 or 256: 20.2
 constexpr int kSlotsPerTensor = 3 * kSlotWays;
 
 struct EncSeg {
@@ -1716,6 +1721,36 @@ int settle_resident_log(hpx::Workspace* ws, hipStream_t st) {
   return HPX_OK;
 }
 
+// ---- encode without allocation ------------------------------------------------------
+constexpr int kNoAllocMaxTensors = kCapLarge;
+constexpr uint32_t kNoAllocWords = uint32_t(kNoAllocMaxTensors) * kSlotsPerTensor;
+static_assert(sizeof(scratch) == size_t(kNoAllocWords) * sizeof(unsigned long long), "scratch must hold the slots of one full table");
+
+__global__ __launch_bounds__(kThreads) void terngrad_scratch_clear_kernel(unsigned long long* __restrict__ p, uint32_t words) {
+  const uint32_t i = blockIdx.x * kThreads + threadIdx.x;
+  if (i < words) p[i] = 0ull;
+}
+
+// Device address of `scratch` on the current device (every GPU holds its own copy at its own address),
+// looked up once per device.
+constexpr int kNoAllocMaxDevices = 64;
+int scratch_address(unsigned long long** out) {
+  static std::mutex mu;
+  static unsigned long long* ptr[kNoAllocMaxDevices] = {};
+  int dev = 0;
+  HPX_HIP(hipGetDevice(&dev));
+  HPX_ARG(dev >= 0 && dev < kNoAllocMaxDevices, "hpx_terngrad_encode_noalloc: device %d (at most %d devices)", dev, kNoAllocMaxDevices);
+  std::lock_guard<std::mutex> g(mu);
+  if (!ptr[dev]) {
+    unsigned long long* p = nullptr;
+    HPX_HIP(hipGetSymbolAddress(reinterpret_cast<void**>(&p), HIP_SYMBOL(scratch)));
+    HPX_ARG(p != nullptr, "hpx_terngrad_encode_noalloc: no device address for the scratch array");
+    ptr[dev] = p;
+  }
+  *out = ptr[dev];
+  return HPX_OK;
+}
+
 constexpr size_t kResidentLogMax = 4096;  // records kept before hpx_terngrad_encode settles the log itself
 
 }  // namespace
@@ -1848,6 +1883,53 @@ HPX_API int hpx_terngrad_encode(int count, const float* const* ins, const int32_
   }
   return encode_tiled(ws, st, m, t_in.data(), t_isz.data(), t_out.data(), t_osz.data(), t_bits.data(), t_rnd.data(),
                       t_seed.data());
+}
+
+HPX_API int hpx_terngrad_encode_noalloc(int count, const float* const* ins, const int32_t* in_sizes,
+                                        uint8_t* const* outs, const int32_t* out_sizes,
+                                        const uint8_t* bitwidths, const int32_t* enable_randoms,
+                                        const uint64_t* seeds, hpx_stream_t stream) {
+  hpx::clear_error();
+  HPX_ARG(count >= 0, "hpx_terngrad_encode_noalloc: negative count");
+  if (count == 0) return HPX_OK;
+  HPX_ARG(count <= kNoAllocMaxTensors, "hpx_terngrad_encode_noalloc: %d tensors in one call, at most %d (the fixed scratch array holds %d x %d slots)",
+          count, kNoAllocMaxTensors, kNoAllocMaxTensors, kSlotsPerTensor);
+  HPX_ARG(ins && in_sizes && outs && out_sizes && bitwidths && enable_randoms,
+          "hpx_terngrad_encode_noalloc: null argument array");
+  int64_t red_tiles = 0, quant_tiles = 0;
+  for (int i = 0; i < count; i++) {
+    const uint8_t b = bitwidths[i];
+    if (!(b == 1 || b == 2 || b == 4 || b == 8)) {
+      hpx::set_error("Invalid value of bitwidth, check value: bitwidth=%d", int(b));
+      return HPX_ERR_BODY;
+    }
+    HPX_ARG(in_sizes[i] > 0, "hpx_terngrad_encode_noalloc: tensor %d has size %d (must be positive)", i, in_sizes[i]);
+    HPX_ARG(ins[i] && outs[i], "hpx_terngrad_encode_noalloc: tensor %d has a null pointer", i);
+    const int64_t need = 10 + (int64_t(in_sizes[i]) + 8 / b - 1) / (8 / b);
+    HPX_ARG(out_sizes[i] >= need, "hpx_terngrad_encode_noalloc: tensor %d needs %lld output bytes, got %d", i,
+            static_cast<long long>(need), out_sizes[i]);
+    const int unit = (8 / b) > 4 ? (8 / b) : 4;
+    red_tiles += ceil_div(in_sizes[i], kRedTile);
+    quant_tiles += ceil_div(ceil_div(in_sizes[i], unit), kThreads * kQIters);
+  }
+  // one table, one pair of launches: the scratch array has room for exactly that
+  HPX_ARG(red_tiles <= INT32_MAX && quant_tiles <= INT32_MAX, "hpx_terngrad_encode_noalloc: the tensors of one call add up to too many tiles (%lld)",
+          static_cast<long long>(red_tiles));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  unsigned long long* slots = nullptr;
+  int rc = scratch_address(&slots);
+  if (rc != HPX_OK) return rc;
+  // The array keeps what the last call left: the slots this call uses start from zero again (a fill
+  // kernel, not a memset node, so that the sequence can be recorded into a graph), and the epoch tag is
+  // a constant.
+  const uint32_t words = uint32_t(count) * kSlotsPerTensor;
+  hipLaunchKernelGGL(terngrad_scratch_clear_kernel, dim3((words + kThreads - 1) / kThreads), dim3(kThreads), 0, st, slots, words);
+  HPX_HIP(hipGetLastError());
+  if (count <= kCapSmall)
+    return launch_encode<kCapSmall>(count, ins, in_sizes, outs, out_sizes, bitwidths, enable_randoms, seeds,
+                                    reinterpret_cast<uint64_t*>(slots), 1u, st, false);
+  return launch_encode<kCapLarge>(count, ins, in_sizes, outs, out_sizes, bitwidths, enable_randoms, seeds,
+                                  reinterpret_cast<uint64_t*>(slots), 1u, st, false);
 }
 
 HPX_API int hpx_terngrad_encode_status(hpx_stream_t stream) {
