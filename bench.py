@@ -13,10 +13,9 @@ its input in the 256 MB Infinity Cache from the step before.
 Prints ONE JSON line:  value = GB/s of fp32 gradient (4*N bytes per step) over
 the whole timed region; "roofline" prices the dominant kernel against the HBM
 peak with its duration measured by HIP events on the launch stream;
-"cpu_baseline" is the reference's own CPU bodies (their host build, where it
-exists; else the plain-C oracle, a port of them) timed on the host cores of the
-same box; "extra" carries the other codecs of
-the path at their configuration sizes.
+"cpu_baseline" is the plain-C/OpenMP port of the reference's CPU bodies (the
+oracle) timed on the host cores of the same box; "extra" carries the other
+codecs of the path at their configuration sizes.
 """
 import argparse
 import ctypes as C
@@ -280,34 +279,6 @@ def cpu_baseline(np, n, budget_s):
     sec1 = (time.perf_counter() - t0) / 2
     cpu.set_threads(threads)
     res["one_thread"] = {"value": round(4.0 * n / sec1 / 1e9, 3), "ms_per_step": round(sec1 * 1e3, 2)}
-    # The reference's own header bodies (terngrad_body / terngrad_r_body under thrust::omp::par), where the
-    # host build of them exists: it is made from a reference checkout and travels as a built library.
-    from oracle import ref
-    if ref.available():
-        msg = np.zeros(10 + (n + 3) // 4, np.uint8)
-
-        def ref_one():
-            rc = ref.lib().ref_terngrad_encode(ref._f32(x), n, ref._u8(msg), msg.size, 2, 1, 1)
-            rc2, _ = ref.terngrad_decode(msg, n, out, 0, 1)
-            assert rc == 0 and rc2 == 0
-
-        ref_one()
-        t0 = time.perf_counter()
-        r_reps, laps = 0, []
-        while r_reps < 3 or (time.perf_counter() - t0 < budget_s / 2 and r_reps < 200):
-            t1 = time.perf_counter()
-            ref_one()
-            laps.append(time.perf_counter() - t1)
-            r_reps += 1
-        rsec = float(np.median(laps))
-        # the reference's own code is the baseline proper; the port's figures stay beside it
-        port = {k: res[k] for k in ("value", "ms_per_step", "one_thread", "sample")}
-        res = {"value": round(4.0 * n / rsec / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "reference",
-               "sample": f"median of {r_reps} full encode+decode passes of the same {n}-element workload through the reference's "
-                         f"terngrad_body / terngrad_r_body compiled for the host, thrust::omp::par over {threads} threads "
-                         f"(clock-seeded; os.cpu_count()={os.cpu_count()}); the bodies' memcpy/sync policy shim is the "
-                         "harness's own, all arithmetic and Thrust calls are the reference's",
-               "ms_per_step": round(rsec * 1e3, 2), "port": port}
     return res
 
 

@@ -12,18 +12,32 @@
  * multiply-add is fused: the reference's x86-64 CPU build rounds the multiply
  * and the add separately.
  *
- * Parity status of each function (what pins it, beyond this restatement):
- *   orc_lcg_*            known answers of the ANSI-C LCG + closed-form jumps
- *   orc_tbq_*            hand-derived known-answer vector, invariants,
- *                        compiled reference headers (oracle/_ref) where built
- *   orc_terngrad_*       known-answer payload bytes, decode error bounds,
- *                        compiled reference headers where built
- *   orc_gd_*             brute force on small inputs (numpy), invariants,
- *                        compiled reference functors where built.  The
- *                        truncation branch's tie order is implementation
- *                        defined in the reference (unstable sort): PARITY
- *                        UNPINNED for ties at the cut, by design; tests assert
- *                        there are none.
+ * Parity status of each function: what pins it to the reference's source text
+ * beyond this restatement.  No build of the reference is involved (its bodies
+ * include Thrust's CUDA backend unconditionally and cannot be built without a
+ * CUDA toolchain); every pin below is a literal derived by hand from the cited
+ * lines (tests/kat_vectors.py), a brute force or an invariant.
+ *   orc_lcg_*, orc_u01   textbook draws of the ANSI-C LCG from seed 0; jump
+ *                        constants from the recurrence; u for draws whose
+ *                        quotient sits on a rounding boundary, among them the
+ *                        one that is rounded twice (0xFFFFFF7F -> 1.0f)
+ *   orc_tbq_*            two hand-derived byte vectors with residuals and
+ *                        decodes; decode + residual == residual + gradient
+ *   orc_terngrad_encode  hand-derived whole messages: draw-to-slot mapping from
+ *                        seed 0 (bytes 0 and 1: seed + byte index), the partial
+ *                        last byte (always rounds to nearest), a code that
+ *                        reaches 4 and is OR-ed into the next slot, the twice-
+ *                        rounded draw, ties-to-even without random rounding; an
+ *                        independent numpy model of the payload; error bounds
+ *   orc_terngrad_decode  hand-derived decode (write and add), closed form
+ *   orc_gd_*             hand-derived 16-element messages (index stream
+ *                        (9k + 14) mod 16, threshold, both branches, residual);
+ *                        numpy brute force with full sorts on small inputs;
+ *                        exact-reconstruction invariants.  The cut branch's
+ *                        order among EQUAL |r| is implementation-defined in the
+ *                        reference (unstable sort): PARITY UNPINNED for ties at
+ *                        the cut, by design; tests assert there are none.
+ *   orc_dgc_*            numpy brute force; equals orc_gd_* with a zero residual
  */
 #include <math.h>
 #include <stdint.h>

@@ -44,18 +44,3 @@ def oracle_cpu():
     from oracle import cpu
     cpu.lib()
     return cpu
-
-
-@pytest.fixture(scope="session")
-def oracle_ref():
-    """The reference's own bodies compiled for the host; optional."""
-    from oracle import ref
-    if not ref.available():
-        try:
-            ref.build()
-        except Exception:
-            pass
-    if not ref.available():
-        pytest.skip("oracle/_ref not built (no reference checkout here)")
-    ref.lib()
-    return ref

@@ -110,42 +110,29 @@ def test_gd_all_zero_gradient_selects_nothing(oracle_cpu):
     assert msg.size == 4 and info["kept"] == 0
 
 
-@pytest.mark.parametrize("policy", [0, 1])
-def test_gd_against_reference_functors(oracle_cpu, oracle_ref, policy):
-    rng = np.random.default_rng(1)
-    cut = kept = 0
-    for n in [1000, 4096, 10007, 100003, 1000003]:
-        for sr, dr in [(0.01, 0.999), (0.05, 0.99), (0.1, 0.9), (0.5, 0.5)]:
-            for seed in (0, 1, 7, 2**40 + 5, 2**64 - 2):
-                g = rng.laplace(0, 1e-3, n).astype(np.float32)
-                r0 = rng.normal(0, 1e-4, n).astype(np.float32)
-                ra, rb = r0.copy(), r0.copy()
-                ma, ia = oracle_cpu.gd_encode(g, ra, sr, dr, seed)
-                mb, ib = oracle_ref.gd_encode_seeded(g.copy(), rb, sr, dr, seed, policy)
-                assert ia == ib, (n, sr, dr, seed)
-                assert np.array_equal(ra.view(np.uint32), rb.view(np.uint32))
-                # continuous random data: no |r| ties, so even the cut branch agrees byte for byte
-                assert np.array_equal(ma, mb)
-                if ia["candidates"] > ia["kept"]:
-                    cut += 1
-                else:
-                    kept += 1
-    assert cut > 5 and kept > 5      # both branches were exercised
-    s = oracle_ref.gd_sample(np.arange(1000, dtype=np.float32), 50, 12345)
-    assert s.astype(np.int64).tolist() == [oracle_cpu.gd_sample_index(12345, x, 1000) for x in range(50)]
-
-
-def test_gd_decode_against_reference(oracle_cpu, oracle_ref):
+def test_gd_decode_against_numpy_scatter(oracle_cpu):
+    # gd_r_body, gd_body.h:283-353: write mode clears the whole output and scatters, add mode accumulates
+    # (indices inside one message are unique, so numpy's fancy-index update is the same operation); a message
+    # longer than the bytes provided is refused with -1 before anything is written (gd_body.h:317-325)
     rng = np.random.default_rng(3)
     for n in (1000, 100003):
         g = rng.laplace(0, 1e-3, n).astype(np.float32); r = np.zeros(n, np.float32)
         m, _ = oracle_cpu.gd_encode(g, r, 0.05, 0.99, 3)
+        idx, val = oracle_cpu.gd_split(m)
+        assert np.unique(idx).size == idx.size
         for add in (0, 1):
             base = rng.normal(0, 1, n).astype(np.float32)
-            a, b = base.copy(), base.copy()
-            assert oracle_cpu.gd_decode(m, a, add) == 0 and oracle_ref.gd_decode(m, b, add) == 0
-            assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
-        assert oracle_ref.gd_decode(m, b, 0, in_size=m.size - 1) == -1
+            a = base.copy()
+            want = base.copy() if add else np.zeros(n, np.float32)
+            if add:
+                want[idx] = val + want[idx]
+            else:
+                want[idx] = val
+            assert oracle_cpu.gd_decode(m, a, add) == 0
+            assert np.array_equal(a.view(np.uint32), want.view(np.uint32))
+        untouched = base.copy()
+        assert oracle_cpu.gd_decode(m, untouched, 0, in_size=m.size - 1) == -1
+        assert np.array_equal(untouched, base)
 
 
 # ---- the sparsifier without residual (dgc_body.h) ------------------------------------------------
