@@ -367,19 +367,64 @@ __global__ __launch_bounds__(kThreads) void tbq_decode_multi_kernel(const MArgs 
     }
     return;
   }
+  // The tile that holds the end of the tensor.  Its whole groups are handled like the ones above, one byte
+  // load per group and message, with the loads of all of a lane's groups and of up to 8 messages in flight
+  // together; only the last, partial group goes element by element.  (Done element by element for the whole
+  // tile, every element waited for its own loads, message after message: up to 16 x (1 + messages) memory
+  // latencies in a row in ONE workgroup, tens of microseconds that the rest of the grid could not hide.)
+  float4 acc[kIters];
+  bool live[kIters];
+#pragma unroll
   for (int k = 0; k < kIters; k++) {
     const uint32_t grp = g0 + k * kThreads;
-    const size_t e = size_t(grp) * 4;
-    const uint32_t lim = grp < full ? 4u : (grp == full ? (n & 3u) : 0u);
-    for (uint32_t i = 0; i < lim; i++) {
-      float acc = need_old ? op[e + i] : 0.f;
-      for (int j = 0; j < ns; j++) {
-        const uint32_t q = as_global(s_in[j])[grp];
-        const float v = (static_cast<float>((q >> (2 * i)) & 3) - 1) * s_thr[j];
-        acc = s_add[j] ? v + acc : v;
+    live[k] = grp < full;
+    acc[k] = (live[k] && need_old) ? ld4(op + size_t(grp) * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+  for (int j0 = 0; j0 < ns; j0 += 8) {
+    uint32_t q[8][kIters];
+#pragma unroll
+    for (int jj = 0; jj < 8; jj++)
+#pragma unroll
+      for (int k = 0; k < kIters; k++) {
+        q[jj][k] = 85u;
+        if (j0 + jj < ns && live[k]) q[jj][k] = as_global(s_in[j0 + jj])[g0 + k * kThreads];
       }
-      op[e + i] = acc;
+#pragma unroll
+    for (int jj = 0; jj < 8; jj++) {
+      if (j0 + jj < ns) {
+        const float thr = s_thr[j0 + jj];
+        const bool add = s_add[j0 + jj] != 0;
+#pragma unroll
+        for (int k = 0; k < kIters; k++) {
+          const float4 v = tbq_values(q[jj][k], thr);
+          if (add) {
+            acc[k].x = v.x + acc[k].x; acc[k].y = v.y + acc[k].y; acc[k].z = v.z + acc[k].z; acc[k].w = v.w + acc[k].w;
+          } else {
+            acc[k] = v;
+          }
+        }
+      }
     }
+  }
+#pragma unroll
+  for (int k = 0; k < kIters; k++)
+    if (live[k]) st4(op + size_t(g0 + k * kThreads) * 4, acc[k]);
+  // the partial group, if the tensor has one and it belongs to this lane
+  const uint32_t rest = n & 3u;
+  if (rest && full >= g0 && (full - g0) % kThreads == 0 && (full - g0) / kThreads < uint32_t(kIters)) {
+    const size_t e = size_t(full) * 4;
+    float tail[3];
+    for (uint32_t i = 0; i < rest; i++) tail[i] = need_old ? op[e + i] : 0.f;
+    for (int j = 0; j < ns; j++) {
+      const uint32_t q = as_global(s_in[j])[full];
+      const float thr = s_thr[j];
+      const bool add = s_add[j] != 0;
+      for (uint32_t i = 0; i < rest; i++) {
+        const float v = (static_cast<float>((q >> (2 * i)) & 3) - 1) * thr;
+        tail[i] = add ? v + tail[i] : v;
+      }
+    }
+    for (uint32_t i = 0; i < rest; i++) op[e + i] = tail[i];
   }
 }
 

@@ -1300,6 +1300,85 @@ __global__ __launch_bounds__(kThreads) void terngrad_decode_multi_kernel(const M
     }
     continue;
   }
+  if (all_cover) {
+    // The sub-tile that holds the end of the tensor, every message complete.  Its whole groups are handled like
+    // the ones above, with the loads of all of a lane's groups and of up to 8 messages in flight together; only
+    // the tensor's last, partial group goes element by element.  (Done element by element for the whole
+    // sub-tile, each element waited for its own loads, message after message: up to 16 x (1 + messages)
+    // memory latencies in a row in ONE workgroup.  Depending on n mod 4096 that tail alone took up to 35 us and
+    // made the time of a 7-message decode jump up and down with the size of the tensor.)
+    float4 acc[kDIters];
+    bool live[kDIters];
+#pragma unroll
+    for (int k = 0; k < kDIters; k++) {
+      const size_t e = size_t(g0 + k * kThreads) * 4;
+      live[k] = e + 4 <= n;
+      acc[k] = (live[k] && need_old) ? ld4(op + e) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    for (int j0 = 0; j0 < ns; j0 += 8) {
+      uint32_t raw[8][kDIters];
+#pragma unroll
+      for (int jj = 0; jj < 8; jj++)
+#pragma unroll
+        for (int k = 0; k < kDIters; k++) {
+          raw[jj][k] = 0;
+          if (j0 + jj < ns && live[k]) {
+            const size_t e = size_t(g0 + k * kThreads) * 4;
+            const uint32_t bits = s_bits[j0 + jj];
+            global_ptr<uint8_t> pay = as_global(s_pay[j0 + jj]);
+            if (bits == 1) raw[jj][k] = (uint32_t(pay[e >> 3]) >> (e & 4)) & 0xFu;
+            else if (bits == 2) raw[jj][k] = pay[e >> 2];
+            else if (bits == 4) raw[jj][k] = uint32_t(pay[e >> 1]) | (uint32_t(pay[(e >> 1) + 1]) << 8);
+            else raw[jj][k] = uint32_t(pay[e]) | (uint32_t(pay[e + 1]) << 8) | (uint32_t(pay[e + 2]) << 16) | (uint32_t(pay[e + 3]) << 24);
+          }
+        }
+#pragma unroll
+      for (int jj = 0; jj < 8; jj++) {
+        if (j0 + jj < ns) {
+          const uint32_t bits = s_bits[j0 + jj];
+          const float gap = s_gap[j0 + jj], mn = s_mn[j0 + jj];
+          const bool add = s_add[j0 + jj] != 0;
+#pragma unroll
+          for (int k = 0; k < kDIters; k++) {
+            float4 v;
+            if (bits == 1) v = group_values<1>(raw[jj][k], gap, mn);
+            else if (bits == 2) v = group_values<2>(raw[jj][k], gap, mn);
+            else if (bits == 4) v = group_values<4>(raw[jj][k], gap, mn);
+            else v = group_values<8>(raw[jj][k], gap, mn);
+            if (add) {
+              acc[k].x = v.x + acc[k].x; acc[k].y = v.y + acc[k].y; acc[k].z = v.z + acc[k].z; acc[k].w = v.w + acc[k].w;
+            } else {
+              acc[k] = v;
+            }
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < kDIters; k++)
+      if (live[k]) st4(op + size_t(g0 + k * kThreads) * 4, acc[k]);
+    // the tensor's last 1..3 elements, if this lane owns them
+#pragma unroll
+    for (int k = 0; k < kDIters; k++) {
+      const size_t e = size_t(g0 + k * kThreads) * 4;
+      if (e < n && !live[k]) {
+        float tail[3];
+        const int lim = int(n - e);
+        for (int i = 0; i < lim; i++) tail[i] = need_old ? op[e + i] : 0.f;
+        for (int j = 0; j < ns; j++) {
+          const float gap = s_gap[j], mn = s_mn[j];
+          const bool add = s_add[j] != 0;
+          for (int i = 0; i < lim; i++) {
+            const float v = float(int(code_at(s_pay[j], e + i, s_bits[j]))) * gap + mn;  // terngrad_body.h:127, :158
+            tail[i] = add ? v + tail[i] : v;
+          }
+        }
+        for (int i = 0; i < lim; i++) op[e + i] = tail[i];
+      }
+    }
+    continue;
+  }
+  // Messages that cover different numbers of elements (a clamped or malformed header): element by element.
   for (int k = 0; k < kDIters; k++) {
     const size_t e = size_t(g0 + k * kThreads) * 4;
     if (e >= n) break;
