@@ -233,9 +233,19 @@ int hpx_terngrad_decode_status(hpx_stream_t stream);
  * ascending index).  seeds == NULL takes the wall clock (gd_body.h:138-140).
  * Unlike the reference, bytes of outs[t] past the message are left untouched
  * (scratch lives in the library workspace), so outs[t] needs only
- * 4 + 8*ceil(N*(1-drop)) bytes.  The call waits for the stream once per tensor
- * (the reference waits three times) and therefore returns -3 on a stream that
- * is being captured into a graph; so do hpx_gd_decode and the two DGC calls. */
+ * 4 + 8*ceil(N*(1-drop)) bytes.
+ * All tensors of a call go through each phase together (one launch per phase
+ * for up to 128 tensors), so hand over whole buckets, as the reference's
+ * scheduler does (hp_cuda.cpp:284-301).  The reference waits for the stream
+ * three times per tensor; this call never waits for the stream: it polls
+ * pinned host words in which a kernel reports the candidate count of every
+ * tensor (while later kernels are still running), queues the sort-and-cut for
+ * the tensors that overshoot and returns; results are stream-ordered.  Because
+ * of that dependence on the host it returns -3 on a stream that is being
+ * captured into a graph; so do hpx_gd_decode and the two DGC calls.
+ * A tensor whose parameters make no sense (threshold index outside the sample)
+ * is skipped and makes the call return -3; the other tensors are encoded, as
+ * the reference driver prints and goes on (hp_cuda_kernel.cu:90-92). */
 int hpx_gd_encode(int count, const float* const* grads, const int32_t* Ns,
                   float* const* residuals, uint8_t* const* outs,
                   const double* sample_rates, const double* drop_ratios,
@@ -259,7 +269,7 @@ int hpx_gd_decode(int count, const uint8_t* const* ins, const int32_t* in_sizes,
  * sample_cnt = ceil(N*sample_rate) sampled |G|, entries beyond it (at most
  * ceil(N*s_percent), the largest first if there are more) go into the message
  * and are CLEARED IN grads[t].  Same message layout, same output size
- * 4 + 8*ceil(N*s_percent), same one wait on the stream.
+ * 4 + 8*ceil(N*s_percent), same way of learning the counts.
  * Decode differs from hpx_gd_decode in write mode only: the output is not
  * cleared first (dgc_body.h:283-289). */
 int hpx_dgc_encode(int count, float* const* grads, const int32_t* Ns, uint8_t* const* outs,

@@ -178,6 +178,83 @@ def test_several_tensors_and_messages(gd, oracle_cpu):
     assert_bits_equal(host(dout), ref, "accumulated decode")
 
 
+def test_bucket_of_ragged_tensors_in_one_call(gd, oracle_cpu, capi):
+    # The scheduler hands hpx_gd_encode whole batches (hp_cuda.cpp:284-301).  160 tensors - more than one launch
+    # table holds - of ragged sizes in ONE call: every phase is one launch for a table of tensors, the host
+    # learns all counts at once, and only the tensors that overshoot are sorted and cut afterwards.  Among them:
+    # tensors that are cut and tensors that are not, one that selects nothing, one whose candidates are far
+    # more than the space reserved for the cut, single-element and tile-edge sizes.
+    rng = np.random.default_rng(60)
+    sizes = [int(np.exp(rng.uniform(np.log(50), np.log(400_000)))) for _ in range(150)]
+    sizes += [1, 2, 4095, 4096, 4097, 8191, 65_536, 262_145, 1_000_003, 400_003]
+    srs = [float(rng.choice([0.01, 0.05, 0.2, 0.5])) for _ in sizes]
+    drs = [float(rng.choice([0.9, 0.99, 0.999])) for _ in sizes]
+    seeds = [int(x) for x in rng.integers(0, 2**63, len(sizes))]
+    gs = [rng.laplace(0, 1e-3, n).astype(np.float32) for n in sizes]
+    rs = [rng.normal(0, 1e-4, n).astype(np.float32) for n in sizes]
+    for i, n in enumerate(sizes):                                 # parameters the reference itself would accept
+        sc = int(np.ceil(n * srs[i]))
+        if not (sc > 0 and int(sc * (1 - drs[i])) < sc):
+            srs[i], drs[i] = 1.0, 0.5
+    zero_at = 17                                                  # nothing selected: header only
+    gs[zero_at][:] = 0; rs[zero_at][:] = 0
+    flood_at = len(sizes) - 1                                     # nearly everything is a candidate
+    n_f = sizes[flood_at]
+    srs[flood_at], drs[flood_at] = 0.01, 0.999
+    gs[flood_at][np.abs(gs[flood_at]) < 1e-5] = 1e-5
+    sampled = np.array([oracle_cpu.gd_sample_index(seeds[flood_at], x, n_f) for x in range(int(np.ceil(n_f * 0.01)))])
+    gs[flood_at][sampled] = (1e-7 * (1 + np.arange(sampled.size) / sampled.size)).astype(np.float32)
+    rs[flood_at][:] = 0
+    dgs, drs_ = [dev(g) for g in gs], [dev(r) for r in rs]
+    guard = 64
+    outs = [torch.full((_out_bytes(n, d) + guard,), 0xEE, dtype=torch.uint8, device="cuda") for n, d in zip(sizes, drs)]
+    L = capi.load()
+    L.hpx_profile_reset(); L.hpx_profile_enable(1)
+    try:
+        gd.encode(dgs, drs_, outs, srs, drs, seeds)
+        torch.cuda.synchronize()
+        stream_launches = capi.profile_query("gd_stream_kernel")[1]
+    finally:
+        L.hpx_profile_enable(0); L.hpx_profile_reset()
+    assert stream_launches == 2, stream_launches                  # 160 tensors: two launch tables, not 160 launches
+    cut = kept_all = 0
+    for i, n in enumerate(sizes):
+        r_ref = rs[i].copy()
+        msg, info = oracle_cpu.gd_encode(gs[i], r_ref, srs[i], drs[i], seeds[i])
+        got = host(outs[i])
+        size = _out_bytes(n, drs[i])
+        assert_bits_equal(got[:msg.size], msg, f"message[{i}] n={n} sr={srs[i]} dr={drs[i]} info={info}")
+        assert np.all(got[size:] == 0xEE), f"tensor {i}: wrote past 4 + 8*expected bytes"
+        assert_bits_equal(host(drs_[i]), r_ref, f"residual[{i}]")
+        assert_bits_equal(host(dgs[i]), gs[i], f"gradient[{i}] untouched")
+        cut += info["candidates"] > info["kept"]
+        kept_all += info["candidates"] <= info["kept"]
+        if i == zero_at:
+            assert msg.size == 4
+        if i == flood_at:
+            assert info["candidates"] > info["kept"] + 65536       # more than the cut path's buffers were laid out for
+    assert cut >= 10 and kept_all >= 10, (cut, kept_all)
+
+
+def test_bad_tensor_in_a_bucket_is_reported_and_skipped(gd, oracle_cpu):
+    # like the reference driver, which prints and goes on (hp_cuda_kernel.cu:90-92): the call returns the failure,
+    # the other tensors are encoded
+    rng = np.random.default_rng(61)
+    sizes = [5000, 100, 70_001]
+    gs = [rng.laplace(0, 1e-3, n).astype(np.float32) for n in sizes]
+    rs = [rng.normal(0, 1e-4, n).astype(np.float32) for n in sizes]
+    dgs, drs_ = [dev(g) for g in gs], [dev(r) for r in rs]
+    outs = [torch.zeros(_out_bytes(n, 0.9) + 64, dtype=torch.uint8, device="cuda") for n in sizes]
+    gd.encode(dgs, drs_, outs, [0.05, 0.05, 0.05], [0.9, 0.0, 0.9], [1, 2, 3], expect_rc=-3)   # tensor 1: threshold index out of range
+    torch.cuda.synchronize()
+    for i in (0, 2):
+        r_ref = rs[i].copy()
+        msg, _ = oracle_cpu.gd_encode(gs[i], r_ref, 0.05, 0.9, [1, 2, 3][i])
+        assert_bits_equal(host(outs[i])[:msg.size], msg, f"message[{i}]")
+        assert_bits_equal(host(drs_[i]), r_ref, f"residual[{i}]")
+    assert_bits_equal(host(drs_[1]), rs[1], "the skipped tensor's residual is untouched")
+
+
 def test_decode_errors(gd, oracle_cpu):
     n = 5000
     rng = np.random.default_rng(1)

@@ -58,6 +58,8 @@ struct Workspace {
   hipStream_t stream = nullptr;
   uint8_t* dev = nullptr;
   size_t dev_bytes = 0;
+  uint8_t* aux = nullptr;  // second grow-only block, for the rare call whose needs are only known half-way through
+  size_t aux_bytes = 0;
   uint32_t* state = nullptr;
   uint8_t* pinned = nullptr;
   // Epoch-tagged 64-bit reduction slots (see ensure_slots): memory that only ever
@@ -95,6 +97,8 @@ constexpr size_t kPinnedFlagOffset = kPinnedBytes - 64;   // host word raised by
 // the call needs (may wait for the stream when the block has to grow).
 Workspace* workspace_record(hipStream_t stream);
 int ensure_workspace(Workspace* ws, size_t dev_bytes);
+// The same for the second block (ws->aux); waits for the stream when it has to grow.
+int ensure_aux(Workspace* ws, size_t bytes);
 // At least `words` zero-initialised-at-allocation 64-bit slots, never used for anything else.
 int ensure_slots(Workspace* ws, size_t words);
 // Zeroed barrier exchange memory and the CU count of the device (both created once).

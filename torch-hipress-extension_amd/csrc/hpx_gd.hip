@@ -3,7 +3,9 @@
 //
 // Semantics follow gd_body.h:102-232 (encode) and :283-353 (decode).  The
 // reference makes a pass for R += G, a gather for the sample, a full sort of
-// the sample, a two-pass copy_if and waits for the stream three times.  Here:
+// the sample, a two-pass copy_if and waits for the stream three times, tensor
+// after tensor.  Here every phase is ONE launch for all tensors of a call (a
+// table of tensors in the kernel arguments, as in the TBQ and TernGrad paths):
 //
 //   sample      |G[i]+R[i]| at the reference's LCG index stream, gathered
 //               BEFORE the update (the same fp32 sum the update will store)
@@ -11,19 +13,24 @@
 //               passes over the fp32 bit pattern (11+11+10 bits); no sort
 //   stream      ONE pass over the tensor: r = g + r, store r, compare with the
 //               threshold, wave64 ballot -> one 64-bit word per 64 elements
-//               (bit i = element i) and a popcount per workgroup
-//   scan        two-level exclusive prefix of the per-workgroup counts
+//               (bit i = element i), a popcount and the largest |r| per workgroup
+//   scan        two-level exclusive prefix of the per-workgroup counts; reports
+//               count, threshold and largest |r| of each tensor to the host
 //   expand      bit words -> ascending indices at the scanned offsets, values
 //               out, residual entries zeroed, header written
 //
 // The stream pass moves 12 bytes per element (g, r in; r out) plus 1/8 byte of
-// mask; everything else touches O(sample + selected) data.  The host waits for
-// the stream once, after the common case (no cut) has been queued in full, to
-// learn whether the cut to `expected` entries is needed.  The expand launch has
-// by then left the candidates, their keys and the first digit's counts where
-// the cut path wants them, so that path is four more launches: a stable LSD radix
-// sort by |r| (ties keep ascending index) whose last pass writes the message.
+// mask; everything else touches O(sample + selected) data.  The host learns the
+// candidate counts from pinned memory while the expand launch is still running
+// (it polls the words the scan launch writes; no wait for the stream), and only
+// for tensors with more than `expected` candidates queues the cut: a stable LSD
+// radix sort by |r| (ties keep ascending index) over as many byte digits as the
+// largest key has, whose last pass writes the message.  The expand launch has
+// by then left the candidates and their keys where the sort wants them.
 #include <cmath>
+#include <vector>
+
+#include <immintrin.h>
 
 #include "hpx_common.h"
 
@@ -37,6 +44,9 @@ constexpr int kWaveTile = kWave * kPerLane;      // 1024 elements per wave
 constexpr int kSelThreads = 1024;
 constexpr int kSelBlocksMax = 128;               // few blocks: their bins meet in global atomics
 constexpr int kBins1 = 2048, kBins2 = 2048, kBins3 = 1024;  // key = d1:11 | d2:11 | d3:10
+constexpr int kHistWords = kBins1 + kBins2 + kBins3;
+constexpr int kCapLarge = 128;                   // tensors per launch table (8.7 KiB of kernel arguments)
+constexpr int kCapSmall = 4;                     // calls with a few tensors pass a table of a few hundred bytes
 
 struct GdState {
   uint32_t total;     // candidates found by the stream pass
@@ -47,17 +57,79 @@ struct GdState {
 constexpr int kScanChunk = 4096;   // per-tile counts scanned by one workgroup
 constexpr int kMaxChunks = 128;    // 2^31 elements / kTile / kScanChunk
 
-struct SelArgs {
-  const float* g;
-  const float* r;
+__host__ __device__ constexpr size_t align256(size_t x) { return (x + 255) & ~size_t(255); }
+__host__ __device__ constexpr uint32_t cdiv(uint64_t a, uint64_t b) { return static_cast<uint32_t>((a + b - 1) / b); }
+
+// Where the pieces of one tensor's workspace block lie (the same arithmetic on the host and in the kernels).
+struct GdLayout {
+  size_t state, hist, samples, masks, cnt, mx, off, ctot, cmax, coff, end;
+};
+__host__ __device__ inline GdLayout gd_layout(uint32_t n, uint32_t sample_cnt) {
+  const size_t ntiles = cdiv(n, kTile);
+  GdLayout l;
+  size_t at = 0;
+  l.state = at;   at += align256(sizeof(GdState));
+  l.hist = at;    at += align256(sizeof(uint32_t) * kHistWords);
+  l.samples = at; at += align256(sizeof(uint32_t) * size_t(sample_cnt));
+  l.masks = at;   at += align256(sizeof(uint64_t) * ntiles * kWave);      // one bit per element
+  l.cnt = at;     at += align256(sizeof(uint32_t) * ntiles);              // candidates per tile
+  l.mx = at;      at += align256(sizeof(uint32_t) * ntiles);              // largest |r| per tile, as bits
+  l.off = at;     at += align256(sizeof(uint32_t) * ntiles);              // exclusive prefix within the chunk
+  l.ctot = at;    at += align256(sizeof(uint32_t) * kMaxChunks);
+  l.cmax = at;    at += align256(sizeof(uint32_t) * kMaxChunks);
+  l.coff = at;    at += align256(sizeof(uint32_t) * kMaxChunks);
+  l.end = at;
+  return l;
+}
+// The cut path's buffers for up to `pairs` candidates: two copies of keys and indices, and the sort's counts.
+constexpr int kSortThreads = 1024;
+constexpr int kSortPer = 8;
+constexpr int kSortTile = kSortThreads * kSortPer;   // tiles of 8192 pairs
+constexpr int kSortWaves = kSortThreads / kWave;
+struct CutLayout {
+  size_t ka, kb, ia, ib, sc, end;
+};
+__host__ __device__ inline CutLayout cut_layout(uint64_t pairs) {
+  CutLayout c;
+  size_t at = 0;
+  c.ka = at; at += align256(sizeof(uint32_t) * size_t(pairs));
+  c.kb = at; at += align256(sizeof(uint32_t) * size_t(pairs));
+  c.ia = at; at += align256(sizeof(int32_t) * size_t(pairs));
+  c.ib = at; at += align256(sizeof(int32_t) * size_t(pairs));
+  c.sc = at; at += align256(sizeof(uint32_t) * 256 * size_t(cdiv(pairs, kSortTile)));
+  c.end = at;
+  return c;
+}
+
+// One tensor of a call.  64 bytes.
+struct GdSeg {
+  const float* g;      // the gradient
+  float* r;            // the array whose entries are selected and cleared: the residual, or (without one) the gradient
+  uint8_t* out;        // the message
+  uint8_t* ws;         // this tensor's workspace block (gd_layout)
+  uint8_t* cut;        // ... and its cut-path buffers (cut_layout)
   uint32_t n;
   uint32_t sample_cnt;
-  uint32_t seed;        // low 32 bits of the 64-bit seed
-  uint32_t thr_index;   // rank (descending, 0-based) of the threshold in the sample
-  uint32_t* samples;    // |g+r| bit patterns
-  uint32_t* hist;       // kBins1 + kBins2 + kBins3 counters, zero on entry
-  GdState* st;
+  uint32_t seed;       // low 32 bits of the 64-bit seed
+  uint32_t thr_index;  // rank (descending, 0-based) of the threshold in the sample
+  uint32_t limit;      // `expected`: more candidates than this are cut to this many
+  uint32_t cap;        // pairs the cut-path buffers hold
 };
+static_assert(sizeof(GdSeg) == 64, "segment record");
+// What the scan launch reports per tensor in pinned host memory.
+constexpr int kReportWords = 4;  // count of candidates, threshold bits, bits of the largest |r|, unused
+constexpr uint32_t kNotReported = 0xFFFFFFFFu;  // a count is < 2^31
+template <int CAP>
+struct GdArgs {
+  int32_t nseg;
+  int32_t residual;             // 0: the sparsifier without residual (dgc_body.h)
+  int32_t tile_start[CAP + 1];  // exclusive prefix of this launch's workgroups per tensor
+  GdSeg seg[CAP];
+  uint32_t* report;             // pinned host memory, kReportWords per tensor of this table
+};
+static_assert(sizeof(GdArgs<kCapLarge>) <= 9600, "kernel-argument budget");
+
+__device__ __forceinline__ GdState* seg_state(const GdSeg& sg) { return reinterpret_cast<GdState*>(sg.ws); }
 
 // Rank search in a descending cumulative histogram: returns the bin holding
 // rank `rank_in` (0-based from the top) and the rank left inside that bin.
@@ -110,27 +182,35 @@ __device__ __forceinline__ uint32_t sample_index(uint32_t seed, uint32_t x, uint
 
 // One sample per lane: all the random gathers of the sample are in flight at
 // once.  The same launch clears the histograms and the counters of this call.
-__global__ __launch_bounds__(kThreads) void gd_sample_kernel(const SelArgs a) {
-  const uint32_t x = blockIdx.x * kThreads + threadIdx.x;
-  if (x < uint32_t(kBins1 + kBins2 + kBins3)) a.hist[x] = 0;
+template <int CAP>
+__global__ __launch_bounds__(kThreads) void gd_sample_kernel(const GdArgs<CAP> a) {
+  const int tile = blockIdx.x;
+  const int s = find_segment<CAP>(a.tile_start, a.nseg, tile);
+  const GdSeg& sg = a.seg[s];
+  const GdLayout l = gd_layout(sg.n, sg.sample_cnt);
+  uint32_t* hist = reinterpret_cast<uint32_t*>(sg.ws + l.hist);
+  uint32_t* samples = reinterpret_cast<uint32_t*>(sg.ws + l.samples);
+  const uint32_t x = uint32_t(tile - a.tile_start[s]) * kThreads + threadIdx.x;
+  if (x < uint32_t(kHistWords)) hist[x] = 0;
   if (x == 0) {
-    a.st->total = 0;
-    a.st->arrive = 0;
+    seg_state(sg)->total = 0;
+    seg_state(sg)->arrive = 0;
   }
-  if (x < a.sample_cnt) {
-    const uint32_t i = sample_index(a.seed, x, a.n);
+  if (x < sg.sample_cnt) {
+    const uint32_t i = sample_index(sg.seed, x, sg.n);
     // with a residual: |G[i] + R[i]|, the value the update is about to store; without (dgc_body.h:18-30): |G[i]|
-    a.samples[x] = __float_as_uint(__builtin_fabsf(a.r ? a.g[i] + a.r[i] : a.g[i]));
+    samples[x] = __float_as_uint(__builtin_fabsf(a.residual ? sg.g[i] + sg.r[i] : sg.g[i]));
   }
 }
 
 template <int PASS>
-__device__ __forceinline__ void hist_accumulate(const SelArgs& a, uint32_t* s_hist, uint32_t prefix) {
+__device__ __forceinline__ void hist_accumulate(const uint32_t* __restrict__ samples, uint32_t sample_cnt, uint32_t block,
+                                                uint32_t nblocks, uint32_t* s_hist, uint32_t prefix) {
   // PASS 1: all keys, digit = key >> 21.  PASS 2: keys with key>>21 == prefix,
   // digit = (key >> 10) & 2047.  PASS 3: keys with key>>10 == prefix, digit = key & 1023.
-  const uint32_t stride = gridDim.x * kSelThreads;
-  for (uint32_t x = blockIdx.x * kSelThreads + threadIdx.x; x < a.sample_cnt; x += stride) {
-    const uint32_t key = a.samples[x];
+  const uint32_t stride = nblocks * kSelThreads;
+  for (uint32_t x = block * kSelThreads + threadIdx.x; x < sample_cnt; x += stride) {
+    const uint32_t key = samples[x];
     if (PASS == 1) {
       atomicAdd(&s_hist[key >> 21], 1u);
     } else if (PASS == 2) {
@@ -141,59 +221,77 @@ __device__ __forceinline__ void hist_accumulate(const SelArgs& a, uint32_t* s_hi
   }
 }
 
-template <int PASS>
-__global__ __launch_bounds__(kSelThreads) void gd_select_kernel(const SelArgs a) {
+template <int PASS, int CAP>
+__global__ __launch_bounds__(kSelThreads) void gd_select_kernel(const GdArgs<CAP> a) {
   constexpr int BINS = PASS == 1 ? kBins1 : PASS == 2 ? kBins2 : kBins3;
   __shared__ uint32_t s_hist[BINS];
+  const int tile = blockIdx.x;
+  const int s = find_segment<CAP>(a.tile_start, a.nseg, tile);
+  const GdSeg& sg = a.seg[s];
+  const GdLayout l = gd_layout(sg.n, sg.sample_cnt);
+  uint32_t* hist = reinterpret_cast<uint32_t*>(sg.ws + l.hist);
   for (int i = threadIdx.x; i < BINS; i += kSelThreads) s_hist[i] = 0;
   uint32_t prefix = 0;
   if (PASS >= 2) {
     uint32_t d1, rank;
-    find_digit<kBins1>(a.hist, a.thr_index, d1, rank);
+    find_digit<kBins1>(hist, sg.thr_index, d1, rank);
     prefix = d1;
     if (PASS == 3) {
       uint32_t d2;
-      find_digit<kBins2>(a.hist + kBins1, rank, d2, rank);
+      find_digit<kBins2>(hist + kBins1, rank, d2, rank);
       prefix = (d1 << 11) | d2;
     }
   }
   __syncthreads();
-  hist_accumulate<PASS>(a, s_hist, prefix);
+  hist_accumulate<PASS>(reinterpret_cast<const uint32_t*>(sg.ws + l.samples), sg.sample_cnt,
+                        uint32_t(tile - a.tile_start[s]), uint32_t(a.tile_start[s + 1] - a.tile_start[s]), s_hist, prefix);
   __syncthreads();
-  uint32_t* gh = a.hist + (PASS == 1 ? 0 : PASS == 2 ? kBins1 : kBins1 + kBins2);
+  uint32_t* gh = hist + (PASS == 1 ? 0 : PASS == 2 ? kBins1 : kBins1 + kBins2);
   for (int i = threadIdx.x; i < BINS; i += kSelThreads) {
     const uint32_t c = s_hist[i];
     if (c) atomicAdd(&gh[i], c);
   }
 }
 
-__global__ __launch_bounds__(kSelThreads) void gd_threshold_kernel(const SelArgs a) {
+// One workgroup per tensor.
+template <int CAP>
+__global__ __launch_bounds__(kSelThreads) void gd_threshold_kernel(const GdArgs<CAP> a) {
+  const GdSeg& sg = a.seg[blockIdx.x];
+  const GdLayout l = gd_layout(sg.n, sg.sample_cnt);
+  const uint32_t* hist = reinterpret_cast<const uint32_t*>(sg.ws + l.hist);
   uint32_t d1, d2, d3, rank;
-  find_digit<kBins1>(a.hist, a.thr_index, d1, rank);
-  find_digit<kBins2>(a.hist + kBins1, rank, d2, rank);
-  find_digit<kBins3>(a.hist + kBins1 + kBins2, rank, d3, rank);
-  if (threadIdx.x == 0) a.st->thr_bits = (d1 << 21) | (d2 << 10) | d3;
+  find_digit<kBins1>(hist, sg.thr_index, d1, rank);
+  find_digit<kBins2>(hist + kBins1, rank, d2, rank);
+  find_digit<kBins3>(hist + kBins1 + kBins2, rank, d3, rank);
+  if (threadIdx.x == 0) seg_state(sg)->thr_bits = (d1 << 21) | (d2 << 10) | d3;
 }
 
-// The one pass over the tensor.  Lane l of wave w handles elements
+// The one pass over the tensors.  Lane l of wave w handles elements
 // base + w*1024 + c*64 + l for c = 0..15, so ballot number c is the mask word of
 // 64 consecutive elements in natural bit order.
 // RESIDUAL = false is the sparsifier without residual (dgc_body.h:110-117): the
 // values are G itself, nothing is added and nothing is stored (4 bytes per element).
-template <bool RESIDUAL>
-__global__ __launch_bounds__(kThreads) void gd_stream_kernel(const float* __restrict__ g, float* __restrict__ r,
-                                                             uint32_t n, const GdState* __restrict__ st,
-                                                             uint64_t* __restrict__ masks,
-                                                             uint32_t* __restrict__ blk_counts) {
-  const float thr = __uint_as_float(st->thr_bits);
+template <bool RESIDUAL, int CAP>
+__global__ __launch_bounds__(kThreads) void gd_stream_kernel(const GdArgs<CAP> a) {
+  const int tile = blockIdx.x;
+  const int s = find_segment<CAP>(a.tile_start, a.nseg, tile);
+  const GdSeg& sg = a.seg[s];
+  const GdLayout l = gd_layout(sg.n, sg.sample_cnt);
+  const float* __restrict__ g = sg.g;
+  float* __restrict__ r = sg.r;
+  const uint32_t n = sg.n;
+  uint64_t* __restrict__ masks = reinterpret_cast<uint64_t*>(sg.ws + l.masks);
+  const uint32_t t = uint32_t(tile - a.tile_start[s]);
+  const float thr = __uint_as_float(seg_state(sg)->thr_bits);
   const float nthr = -thr;
   const uint32_t lane = threadIdx.x & (kWave - 1);
   const uint32_t wave = threadIdx.x / kWave;
-  const uint32_t base = blockIdx.x * uint32_t(kTile);
+  const uint32_t base = t * uint32_t(kTile);
   const uint32_t wbase = base + wave * uint32_t(kWaveTile);
   uint32_t lo = 0, hi = 0, cnt = 0;
+  float big = 0.0f;  // largest |x| this lane has seen
+  float gv[kPerLane], rv[kPerLane];
   if (n - base >= uint32_t(kTile)) {
-    float gv[kPerLane], rv[kPerLane];
 #pragma unroll
     for (int c = 0; c < kPerLane; c++) {
       gv[c] = __builtin_nontemporal_load(g + size_t(wbase) + c * kWave + lane);
@@ -205,18 +303,28 @@ __global__ __launch_bounds__(kThreads) void gd_stream_kernel(const float* __rest
       if (RESIDUAL) __builtin_nontemporal_store(x, r + size_t(wbase) + c * kWave + lane);
       const uint64_t m = __ballot((x > thr) || (x < nthr));  // gd_body.h:59-67
       cnt += __popcll(m);
+      big = __builtin_fmaxf(big, __builtin_fabsf(x));
       lo = lane == uint32_t(c) ? uint32_t(m) : lo;  // lane c keeps mask word c
       hi = lane == uint32_t(c) ? uint32_t(m >> 32) : hi;
     }
   } else {
+    // The tile that holds the end of the tensor: all its loads first, as above (a load, add, store per
+    // step would make this one workgroup wait for memory sixteen times in a row at the very end of the launch).
+#pragma unroll
+    for (int c = 0; c < kPerLane; c++) {
+      const uint32_t e = wbase + c * kWave + lane;
+      gv[c] = e < n ? g[e] : 0.0f;
+      rv[c] = (RESIDUAL && e < n) ? r[e] : 0.0f;
+    }
 #pragma unroll
     for (int c = 0; c < kPerLane; c++) {
       const uint32_t e = wbase + c * kWave + lane;
       bool p = false;
       if (e < n) {
-        const float x = RESIDUAL ? g[e] + r[e] : g[e];
+        const float x = RESIDUAL ? gv[c] + rv[c] : gv[c];
         if (RESIDUAL) r[e] = x;
         p = (x > thr) || (x < nthr);
+        big = __builtin_fmaxf(big, __builtin_fabsf(x));
       }
       const uint64_t m = __ballot(p);
       cnt += __popcll(m);
@@ -225,28 +333,51 @@ __global__ __launch_bounds__(kThreads) void gd_stream_kernel(const float* __rest
     }
   }
   if (lane < kPerLane) masks[(size_t(wbase) >> 6) + lane] = (uint64_t(hi) << 32) | lo;
-  __shared__ uint32_t s_cnt[kThreads / kWave];
-  if (lane == 0) s_cnt[wave] = cnt;
+  uint32_t bigb = __float_as_uint(big);  // non-negative floats order like their bit patterns; a NaN is not an input
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) { const uint32_t v = __shfl_xor(bigb, o, kWave); bigb = v > bigb ? v : bigb; }
+  __shared__ uint32_t s_cnt[kThreads / kWave], s_big[kThreads / kWave];
+  if (lane == 0) { s_cnt[wave] = cnt; s_big[wave] = bigb; }
   __syncthreads();
-  if (threadIdx.x == 0) blk_counts[blockIdx.x] = s_cnt[0] + s_cnt[1] + s_cnt[2] + s_cnt[3];
+  if (threadIdx.x == 0) {
+    reinterpret_cast<uint32_t*>(sg.ws + l.cnt)[t] = s_cnt[0] + s_cnt[1] + s_cnt[2] + s_cnt[3];
+    const uint32_t m01 = s_big[0] > s_big[1] ? s_big[0] : s_big[1], m23 = s_big[2] > s_big[3] ? s_big[2] : s_big[3];
+    reinterpret_cast<uint32_t*>(sg.ws + l.mx)[t] = m01 > m23 ? m01 : m23;
+  }
 }
 
-// Exclusive prefix of the per-tile counts, two levels.  Workgroup c scans counts
+// Exclusive prefix of the per-tile counts, two levels.  Workgroup c of a tensor scans counts
 // [c*4096, (c+1)*4096) into `off` (relative to its chunk) and publishes the chunk
-// total; the last workgroup to arrive (at most 128 of them, so the shared
-// counter costs microseconds at worst) turns the totals into chunk offsets and
-// the grand total.
-__global__ __launch_bounds__(kSelThreads) void gd_scan_kernel(const uint32_t* __restrict__ cnt, uint32_t* __restrict__ off,
-                                                              uint32_t n, uint32_t* __restrict__ chunk_tot,
-                                                              uint32_t* __restrict__ chunk_off, GdState* __restrict__ st,
-                                                              uint32_t* __restrict__ host_total) {
-  __shared__ uint32_t s_wave[kSelThreads / kWave];
+// total and the chunk's largest |r|; the last workgroup of the tensor to arrive (at most 128 of
+// them, so the shared counter costs microseconds at worst) turns the totals into chunk offsets and
+// the grand total, and reports to the host.
+template <int CAP>
+__global__ __launch_bounds__(kSelThreads) void gd_scan_kernel(const GdArgs<CAP> a) {
+  __shared__ uint32_t s_wave[kSelThreads / kWave], s_wmax[kSelThreads / kWave];
   __shared__ uint32_t s_last;
+  const int tile = blockIdx.x;
+  const int s = find_segment<CAP>(a.tile_start, a.nseg, tile);
+  const GdSeg& sg = a.seg[s];
+  const GdLayout l = gd_layout(sg.n, sg.sample_cnt);
+  const uint32_t* __restrict__ cnt = reinterpret_cast<const uint32_t*>(sg.ws + l.cnt);
+  const uint32_t* __restrict__ mxs = reinterpret_cast<const uint32_t*>(sg.ws + l.mx);
+  uint32_t* __restrict__ off = reinterpret_cast<uint32_t*>(sg.ws + l.off);
+  uint32_t* chunk_tot = reinterpret_cast<uint32_t*>(sg.ws + l.ctot);
+  uint32_t* chunk_max = reinterpret_cast<uint32_t*>(sg.ws + l.cmax);
+  uint32_t* chunk_off = reinterpret_cast<uint32_t*>(sg.ws + l.coff);
+  GdState* st = seg_state(sg);
+  const uint32_t n = cdiv(sg.n, kTile);                                   // tiles of this tensor
+  const uint32_t chunk = uint32_t(tile - a.tile_start[s]);
+  const uint32_t nchunks = uint32_t(a.tile_start[s + 1] - a.tile_start[s]);
   const uint32_t t = threadIdx.x, lane = t & (kWave - 1), wave = t / kWave;
-  const uint32_t i0 = blockIdx.x * uint32_t(kScanChunk) + t * 4;
-  uint32_t c[4];
+  const uint32_t i0 = chunk * uint32_t(kScanChunk) + t * 4;
+  uint32_t c[4], big = 0;
 #pragma unroll
-  for (int j = 0; j < 4; j++) c[j] = (i0 + j < n) ? cnt[i0 + j] : 0u;
+  for (int j = 0; j < 4; j++) {
+    c[j] = (i0 + j < n) ? cnt[i0 + j] : 0u;
+    const uint32_t m = (i0 + j < n) ? mxs[i0 + j] : 0u;
+    big = m > big ? m : big;
+  }
   const uint32_t sum = c[0] + c[1] + c[2] + c[3];
   uint32_t incl = sum;
 #pragma unroll
@@ -254,14 +385,17 @@ __global__ __launch_bounds__(kSelThreads) void gd_scan_kernel(const uint32_t* __
     const uint32_t v = __shfl_up(incl, o, kWave);
     if (lane >= uint32_t(o)) incl += v;
   }
-  if (lane == kWave - 1) s_wave[wave] = incl;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) { const uint32_t v = __shfl_xor(big, o, kWave); big = v > big ? v : big; }
+  if (lane == kWave - 1) { s_wave[wave] = incl; s_wmax[wave] = big; }
   __syncthreads();
-  uint32_t before = 0, all = 0;
+  uint32_t before = 0, all = 0, allmax = 0;
 #pragma unroll
   for (uint32_t w = 0; w < kSelThreads / kWave; w++) {
     const uint32_t v = s_wave[w];
     if (w < wave) before += v;
     all += v;
+    allmax = s_wmax[w] > allmax ? s_wmax[w] : allmax;
   }
   uint32_t run = before + incl - sum;
 #pragma unroll
@@ -270,60 +404,70 @@ __global__ __launch_bounds__(kSelThreads) void gd_scan_kernel(const uint32_t* __
     run += c[j];
   }
   if (t == 0) {
-    chunk_tot[blockIdx.x] = all;
+    chunk_tot[chunk] = all;
+    chunk_max[chunk] = allmax;
     __threadfence();
-    s_last = (atomicAdd(&st->arrive, 1u) == gridDim.x - 1);
+    s_last = (atomicAdd(&st->arrive, 1u) == nchunks - 1);
   }
   __syncthreads();
   if (!s_last) return;
   __threadfence();
   if (t < kWave) {
     // up to 128 chunk totals: two per lane
-    const uint32_t a0 = (2 * t < gridDim.x) ? __hip_atomic_load(&chunk_tot[2 * t], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
-    const uint32_t a1 = (2 * t + 1 < gridDim.x) ? __hip_atomic_load(&chunk_tot[2 * t + 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
-    uint32_t inc2 = a0 + a1;
+    const uint32_t a0 = (2 * t < nchunks) ? __hip_atomic_load(&chunk_tot[2 * t], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+    const uint32_t a1 = (2 * t + 1 < nchunks) ? __hip_atomic_load(&chunk_tot[2 * t + 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+    const uint32_t m0 = (2 * t < nchunks) ? __hip_atomic_load(&chunk_max[2 * t], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+    const uint32_t m1 = (2 * t + 1 < nchunks) ? __hip_atomic_load(&chunk_max[2 * t + 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+    uint32_t inc2 = a0 + a1, mm = m0 > m1 ? m0 : m1;
 #pragma unroll
     for (int o = 1; o < kWave; o <<= 1) {
       const uint32_t v = __shfl_up(inc2, o, kWave);
       if (t >= uint32_t(o)) inc2 += v;
     }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) { const uint32_t v = __shfl_xor(mm, o, kWave); mm = v > mm ? v : mm; }
     const uint32_t ex = inc2 - a0 - a1;
-    if (2 * t < gridDim.x) chunk_off[2 * t] = ex;
-    if (2 * t + 1 < gridDim.x) chunk_off[2 * t + 1] = ex + a0;
+    if (2 * t < nchunks) chunk_off[2 * t] = ex;
+    if (2 * t + 1 < nchunks) chunk_off[2 * t + 1] = ex + a0;
     if (t == kWave - 1) {
       st->total = inc2;
-      // pinned host word: the host reads it after its one wait on the stream, no copy command needed
-      __hip_atomic_store(host_total, inc2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      // Pinned host words the host polls (no copy command, no wait for the stream): threshold and largest
+      // |r| first, the count - whose arrival the host waits for - last.
+      uint32_t* rep = a.report + size_t(s) * kReportWords;
+      __hip_atomic_store(rep + 1, st->thr_bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      __hip_atomic_store(rep + 2, mm, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      __hip_atomic_store(rep + 0, inc2, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
     }
   }
 }
-
-// Shape of the cut path's radix sort (further down): tiles of 8192 pairs.
-constexpr int kSortThreads = 1024;
-constexpr int kSortPer = 8;
-constexpr int kSortTile = kSortThreads * kSortPer;
-constexpr int kSortWaves = kSortThreads / kWave;
 
 // Turns the per-tile bit masks into the ascending index list, one wave per tile,
 // at the offsets the scan produced.  If the stream pass found at most `limit`
 // candidates this is the finish (gd_body.h:193-229): indices, values and header
 // are written and the residual entries cleared.  If it found more, the candidates
-// and their keys (bits of |r|) go to `cand` / `keys` for the cut path instead and
+// and their keys (bits of |r|) go to the cut path's buffers instead and
 // nothing else is touched; more than `cap` candidates do not fit those buffers
-// and the kernel does nothing (the host then calls it again with larger ones and
+// and the kernel does nothing for that tensor (the host then calls it again with larger ones and
 // limit = 0).
-__global__ __launch_bounds__(kThreads) void gd_expand_kernel(const uint64_t* __restrict__ masks,
-                                                             const uint32_t* __restrict__ tile_off,
-                                                             const uint32_t* __restrict__ chunk_off, uint32_t ntiles,
-                                                             const GdState* __restrict__ st, uint32_t limit,
-                                                             uint8_t* __restrict__ out, float* __restrict__ r,
-                                                             int32_t* __restrict__ cand, uint32_t* __restrict__ keys,
-                                                             uint32_t cap) {
+template <int CAP>
+__global__ __launch_bounds__(kThreads) void gd_expand_kernel(const GdArgs<CAP> a) {
+  const int blk = blockIdx.x;
+  const int s = find_segment<CAP>(a.tile_start, a.nseg, blk);
+  const GdSeg& sg = a.seg[s];
+  const GdLayout l = gd_layout(sg.n, sg.sample_cnt);
+  const CutLayout cl = cut_layout(sg.cap);
+  const GdState* st = seg_state(sg);
+  const uint64_t* __restrict__ masks = reinterpret_cast<const uint64_t*>(sg.ws + l.masks);
+  const uint32_t* __restrict__ tile_off = reinterpret_cast<const uint32_t*>(sg.ws + l.off);
+  const uint32_t* __restrict__ chunk_off = reinterpret_cast<const uint32_t*>(sg.ws + l.coff);
+  uint8_t* __restrict__ out = sg.out;
+  float* __restrict__ r = sg.r;
+  const uint32_t ntiles = cdiv(sg.n, kTile);
   const uint32_t total = st->total;
-  const bool cut = total > limit;
-  if (cut && total > cap) return;
+  const bool cut = total > sg.limit;
+  if (cut && total > sg.cap) return;
   const uint32_t lane = threadIdx.x & (kWave - 1);
-  const uint32_t tile = blockIdx.x * (kThreads / kWave) + threadIdx.x / kWave;
+  const uint32_t tile = uint32_t(blk - a.tile_start[s]) * (kThreads / kWave) + threadIdx.x / kWave;
   if (!cut && tile == 0 && lane == 0) *reinterpret_cast<int32_t*>(out) = int32_t(4 + total * 8);
   if (tile >= ntiles) return;
   uint64_t m = masks[size_t(tile) * kWave + lane];
@@ -337,13 +481,15 @@ __global__ __launch_bounds__(kThreads) void gd_expand_kernel(const uint64_t* __r
   uint32_t pos = chunk_off[tile / kScanChunk] + tile_off[tile] + incl - c;
   const uint32_t e0 = tile * uint32_t(kTile) + lane * kWave;
   if (cut) {
+    int32_t* __restrict__ cand = reinterpret_cast<int32_t*>(sg.cut + cl.ia);
+    uint32_t* __restrict__ keys = reinterpret_cast<uint32_t*>(sg.cut + cl.ka);
     const uint32_t thr_bits = st->thr_bits;
     while (m) {
       const uint32_t e = e0 + uint32_t(__builtin_ctzll(m));
       m &= m - 1;
       cand[pos] = int32_t(e);
       // Sort key: distance of |r| above the threshold in fp32 bit patterns (same order as |r|;
-      // the high digits of such keys are mostly zero, which lets the sort skip its last pass).
+      // the high digits of such keys are mostly zero, which lets the sort skip its last passes).
       keys[pos] = __float_as_uint(__builtin_fabsf(r[e])) - thr_bits;
       pos++;
     }
@@ -361,14 +507,56 @@ __global__ __launch_bounds__(kThreads) void gd_expand_kernel(const uint64_t* __r
   }
 }
 
-// generate_S_value, gd_body.h:80-99, plus the header (gd_body.h:193-201), for a
-// message whose k indices are already in place (the cut path).  A launch of its
+// ---- cut to the `expected` largest |r| (gd_body.h:176-187) ------------------
+// Stable LSD radix sort of (key, index) pairs, 8 bits per pass, descending
+// (bin = 255 - digit).  A pass is a count launch and a scatter launch over tiles
+// of 8192 pairs (1024 lanes x 8), counts[tile * 256 + bin]; the last pass writes
+// the message's index block instead of a sorted list.  All tensors of a call that
+// have to be cut share these launches (a table of tensors in the kernel arguments);
+// the number of passes is that of the tensor with the largest key (a pass over a
+// digit that is zero in every key of a tensor leaves that tensor's order as it is).
+// (All passes in one launch
+// with grid-wide barriers was tried and lost: data handed between workgroups
+// inside a launch needs device-scope accesses or whole-L2 fences, either of
+// which costs more than the launches saved.)  (Counting a pass's digits where its
+// input is written, with global atomics, saves the count launches but was five
+// times slower: some 10^5 scattered atomics cost more than the launches.)
+struct SortSeg {           // one tensor that is being cut; 64 bytes
+  uint32_t* keys[2];       // the pass with parity p reads keys[p], idx[p] and writes keys[1 - p], idx[1 - p]
+  int32_t* idx[2];
+  uint32_t* counts;        // [tile][256] of the current pass
+  uint8_t* msg;            // the message: its index block gets the first `keep` indices from the last pass
+  float* r;                // values are read from here, and cleared
+  uint32_t n;              // candidates
+  uint32_t keep;           // `expected`
+};
+static_assert(sizeof(SortSeg) == 64, "segment record");
+template <int CAP>
+struct SortArgs {
+  int32_t nseg;
+  int32_t shift;
+  int32_t parity;
+  int32_t last;            // this pass writes the messages
+  int32_t tile_start[CAP + 1];
+  SortSeg seg[CAP];
+};
+static_assert(sizeof(SortArgs<kCapLarge>) <= 9600, "kernel-argument budget");
+
+// generate_S_value, gd_body.h:80-99, plus the header (gd_body.h:193-201), for
+// messages whose k indices are already in place (the cut path).  A launch of its
 // own with one lane per entry: done by the few workgroups of the last sort pass
-// these random accesses to r took three times as long.
-__global__ __launch_bounds__(kThreads) void gd_gather_kernel(uint8_t* __restrict__ out, float* __restrict__ r, uint32_t k) {
+// these random accesses to r took three times as long.  tile_start counts blocks of
+// kThreads entries here.
+template <int CAP>
+__global__ __launch_bounds__(kThreads) void gd_gather_kernel(const SortArgs<CAP> a) {
+  const int blk = blockIdx.x;
+  const int s = find_segment<CAP>(a.tile_start, a.nseg, blk);
+  uint8_t* __restrict__ out = a.seg[s].msg;
+  float* __restrict__ r = a.seg[s].r;
+  const uint32_t k = a.seg[s].keep;
   const int32_t* idx = reinterpret_cast<const int32_t*>(out + 4);
   float* val = reinterpret_cast<float*>(out + 4 + size_t(k) * 4);
-  const uint32_t x = blockIdx.x * kThreads + threadIdx.x;
+  const uint32_t x = uint32_t(blk - a.tile_start[s]) * kThreads + threadIdx.x;
   if (x == 0) *reinterpret_cast<int32_t*>(out) = int32_t(4 + k * 8);
   if (x < k) {
     const int32_t i = idx[x];
@@ -376,29 +564,6 @@ __global__ __launch_bounds__(kThreads) void gd_gather_kernel(uint8_t* __restrict
     r[i] = 0.0f;
   }
 }
-
-// ---- cut to the `expected` largest |r| (gd_body.h:176-187) ------------------
-// Stable LSD radix sort of (key, index) pairs, 8 bits per pass, descending
-// (bin = 255 - digit).  A pass is a count launch and a scatter launch over tiles
-// of 8192 pairs (1024 lanes x 8), counts[tile * 256 + bin]; the last pass writes
-// the message's index block instead of a sorted list.  (All passes in one launch
-// with grid-wide barriers was tried and lost: data handed between workgroups
-// inside a launch needs device-scope accesses or whole-L2 fences, either of
-// which costs more than the launches saved.)  (Counting a pass's digits where its
-// input is written, with global atomics, saves the count launches but was five
-// times slower: some 10^5 scattered atomics cost more than the launches.)
-struct SortArgs {
-  const uint32_t* keys_in;
-  const int32_t* idx_in;
-  uint32_t n;
-  int shift;
-  const uint32_t* counts;   // this pass, complete
-  uint32_t nblk;
-  uint32_t* keys_out;       // not used by the last pass
-  int32_t* idx_out;
-  uint8_t* msg;             // last pass only: the message, whose index block gets the first `keep` indices
-  uint32_t keep;
-};
 
 // Lanes of the wave whose `bin` equals this lane's, among the lanes in `live`.
 __device__ __forceinline__ uint64_t match_bin(uint32_t bin, bool live) {
@@ -414,13 +579,20 @@ __device__ __forceinline__ uint64_t match_bin(uint32_t bin, bool live) {
 // One LDS atomic per distinct bin of a wave's 64 keys, not one per key: the top
 // digit of keys that are all just above one threshold is the same for nearly all
 // of them, and 8192 atomics on one LDS word took longer than the rest of the pass.
-__global__ __launch_bounds__(kSortThreads) void gd_sort_count_kernel(const uint32_t* __restrict__ keys, uint32_t n,
-                                                                     int shift, uint32_t* __restrict__ counts) {
+template <int CAP>
+__global__ __launch_bounds__(kSortThreads) void gd_sort_count_kernel(const SortArgs<CAP> a) {
+  const int tile = blockIdx.x;
+  const int s = find_segment<CAP>(a.tile_start, a.nseg, tile);
+  const uint32_t* __restrict__ keys = a.seg[s].keys[a.parity];
+  const uint32_t n = a.seg[s].n;
+  const int shift = a.shift;
+  const uint32_t ltile = uint32_t(tile - a.tile_start[s]);
+  uint32_t* __restrict__ counts = a.seg[s].counts;
   __shared__ uint32_t s_hist[256];
   const uint32_t t = threadIdx.x;
   const uint32_t lane = t & (kWave - 1);
   if (t < 256) s_hist[t] = 0;
-  const uint32_t b0 = blockIdx.x * uint32_t(kSortTile);
+  const uint32_t b0 = ltile * uint32_t(kSortTile);
   uint32_t key[kSortPer];
 #pragma unroll
   for (int j = 0; j < kSortPer; j++) {
@@ -436,7 +608,7 @@ __global__ __launch_bounds__(kSortThreads) void gd_sort_count_kernel(const uint3
     if (live && (same & ((uint64_t(1) << lane) - 1)) == 0) atomicAdd(&s_hist[bin], uint32_t(__popcll(same)));
   }
   __syncthreads();
-  if (t < 256) counts[size_t(blockIdx.x) * 256 + t] = s_hist[t];
+  if (t < 256) counts[size_t(ltile) * 256 + t] = s_hist[t];
 }
 
 // A wave owns 512 consecutive pairs of the tile and takes them 64 at a time, so
@@ -447,7 +619,8 @@ __global__ __launch_bounds__(kSortThreads) void gd_sort_count_kernel(const uint3
 // per bin within the tile; the pairs are then put in that order in LDS, so that
 // consecutive lanes write consecutive slots of a bin's run (scattering straight
 // from registers costs one address per lane and made the pass twice as long).
-__global__ __launch_bounds__(kSortThreads) void gd_sort_pass_kernel(const SortArgs a) {
+template <int CAP>
+__global__ __launch_bounds__(kSortThreads) void gd_sort_pass_kernel(const SortArgs<CAP> a) {
   extern __shared__ uint32_t s_stage[];          // [kSortTile] keys, then [kSortTile] indices
   __shared__ uint32_t s_cnt[kSortWaves][256];    // per wave: pairs per bin, then the wave's first place per bin
   __shared__ uint32_t s_first[256];              // first place of the bin within the tile
@@ -457,16 +630,27 @@ __global__ __launch_bounds__(kSortThreads) void gd_sort_pass_kernel(const SortAr
   uint32_t* s_id = s_stage + kSortTile;
   const uint32_t t = threadIdx.x;
   const uint32_t lane = t & (kWave - 1), wave = t / kWave;
-  const uint32_t n = a.n;
-  const uint32_t b0 = blockIdx.x * uint32_t(kSortTile);
+  const int gtile = blockIdx.x;
+  const int sgi = find_segment<CAP>(a.tile_start, a.nseg, gtile);
+  const SortSeg& sg = a.seg[sgi];
+  const uint32_t n = sg.n;
+  const uint32_t blk = uint32_t(gtile - a.tile_start[sgi]);                         // this tensor's tile ...
+  const uint32_t nblk = uint32_t(a.tile_start[sgi + 1] - a.tile_start[sgi]);       // ... of so many
+  const uint32_t* __restrict__ keys_in = sg.keys[a.parity];
+  const int32_t* __restrict__ idx_in = sg.idx[a.parity];
+  uint32_t* __restrict__ keys_out = sg.keys[1 - a.parity];
+  int32_t* __restrict__ idx_out = sg.idx[1 - a.parity];
+  const uint32_t* __restrict__ counts = sg.counts;
+  uint8_t* __restrict__ msg = a.last ? sg.msg : nullptr;
+  const uint32_t b0 = blk * uint32_t(kSortTile);
   const uint32_t x0 = b0 + wave * uint32_t(kSortPer * kWave) + lane;
   uint32_t key[kSortPer];
   int32_t id[kSortPer];
 #pragma unroll
   for (int j = 0; j < kSortPer; j++) {
     const uint32_t x = x0 + j * kWave;
-    key[j] = x < n ? a.keys_in[x] : 0u;
-    id[j] = x < n ? a.idx_in[x] : 0;
+    key[j] = x < n ? keys_in[x] : 0u;
+    id[j] = x < n ? idx_in[x] : 0;
   }
   // bin t (first 256 lanes): pairs in all tiles, in the tiles before this one, in this one.
   // The first 32 tiles are read with independent loads.
@@ -475,27 +659,27 @@ __global__ __launch_bounds__(kSortThreads) void gd_sort_pass_kernel(const SortAr
     constexpr uint32_t kFlat = 32;
     uint32_t c[kFlat];
 #pragma unroll
-    for (uint32_t q = 0; q < kFlat; q++) c[q] = q < a.nblk ? a.counts[size_t(q) * 256 + t] : 0u;
+    for (uint32_t q = 0; q < kFlat; q++) c[q] = q < nblk ? counts[size_t(q) * 256 + t] : 0u;
 #pragma unroll
     for (uint32_t q = 0; q < kFlat; q++) {
       total += c[q];
-      before += q < blockIdx.x ? c[q] : 0u;
-      mine += q == blockIdx.x ? c[q] : 0u;
+      before += q < blk ? c[q] : 0u;
+      mine += q == blk ? c[q] : 0u;
     }
-    for (uint32_t q = kFlat; q < a.nblk; q++) {
-      const uint32_t v = a.counts[size_t(q) * 256 + t];
+    for (uint32_t q = kFlat; q < nblk; q++) {
+      const uint32_t v = counts[size_t(q) * 256 + t];
       total += v;
-      before += q < blockIdx.x ? v : 0u;
-      mine += q == blockIdx.x ? v : 0u;
+      before += q < blk ? v : 0u;
+      mine += q == blk ? v : 0u;
     }
   }
-  if (a.msg) {
+  if (msg) {
     // Last pass: if every key has the same digit the input is already in order.
     if (__syncthreads_or(t < 256 && total == n)) {
 #pragma unroll
       for (int j = 0; j < kSortPer; j++) {
         const uint32_t x = x0 + j * kWave;
-        if (x < n && x < a.keep) reinterpret_cast<int32_t*>(a.msg + 4)[x] = id[j];
+        if (x < n && x < sg.keep) reinterpret_cast<int32_t*>(msg + 4)[x] = id[j];
       }
       return;
     }
@@ -561,12 +745,12 @@ __global__ __launch_bounds__(kSortThreads) void gd_sort_pass_kernel(const SortAr
       const int32_t i = int32_t(s_id[p]);
       const uint32_t b = 255u - ((k >> a.shift) & 255u);
       const uint32_t slot = s_slot[b] + (p - s_first[b]);
-      if (a.msg) {
+      if (msg) {
         // last pass: the indices that survive the cut go straight into the message
-        if (slot < a.keep) reinterpret_cast<int32_t*>(a.msg + 4)[slot] = i;
+        if (slot < sg.keep) reinterpret_cast<int32_t*>(msg + 4)[slot] = i;
       } else {
-        a.keys_out[slot] = k;
-        a.idx_out[slot] = i;
+        keys_out[slot] = k;
+        idx_out[slot] = i;
       }
     }
   }
@@ -594,14 +778,17 @@ __global__ __launch_bounds__(kThreads) void gd_scatter_kernel(const int32_t* __r
   }
 }
 
-inline uint32_t cdiv(uint64_t a, uint64_t b) { return static_cast<uint32_t>((a + b - 1) / b); }
-inline size_t align256(size_t x) { return (x + 255) & ~size_t(255); }
+// One tensor of the cut path as the host sees it.
+struct CutJob {
+  SortSeg seg;
+  int passes;  // byte digits its largest key has
+};
 
-// The four passes of the cut path: (keys_a, idx_a) hold the candidates in index
-// order.  The last pass writes the indices of the `keep` largest into the
-// message `msg`; a gather launch adds values and header and clears the residual.
-int sort_and_cut(uint32_t* keys_a, int32_t* idx_a, uint32_t* keys_b, int32_t* idx_b, uint32_t* counts, uint32_t n,
-                 uint8_t* msg, float* r, uint32_t keep, hipStream_t st) {
+// The cut path for up to CAP tensors: `passes` x (count launch, scatter launch) over all of them, lowest digit
+// first, the last scatter writing the index blocks of the messages; then one gather launch that adds values
+// and headers and clears the residual entries.
+template <int CAP>
+int sort_and_cut(const CutJob* jobs, int count, hipStream_t st) {
   constexpr int kStageBytes = 2 * kSortTile * int(sizeof(uint32_t));
   // The dynamic-LDS limit is a property of the function on one device: raise it once per device.
   static std::mutex attr_mu;
@@ -611,151 +798,259 @@ int sort_and_cut(uint32_t* keys_a, int32_t* idx_a, uint32_t* keys_b, int32_t* id
     HPX_HIP(hipGetDevice(&dev));
     std::lock_guard<std::mutex> g(attr_mu);
     if (dev >= 64 || !(attr_done >> dev & 1)) {
-      HPX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gd_sort_pass_kernel),
+      HPX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gd_sort_pass_kernel<CAP>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, kStageBytes));
       if (dev < 64) attr_done |= uint64_t(1) << dev;
     }
   }
-  const uint32_t nblk = cdiv(n, kSortTile);
-  for (int pass = 0; pass < 4; pass++) {
-    SortArgs a;
-    a.keys_in = keys_a; a.idx_in = idx_a; a.n = n; a.shift = pass * 8;
-    a.counts = counts; a.nblk = nblk;
-    a.keys_out = keys_b; a.idx_out = idx_b;
-    a.msg = pass == 3 ? msg : nullptr;
-    a.keep = keep;
-    HPX_LAUNCH("gd_sort_count_kernel", gd_sort_count_kernel, dim3(nblk), dim3(kSortThreads), st, keys_a, n, a.shift, counts);
+  SortArgs<CAP> a;
+  a.nseg = count;
+  int passes = 1;
+  a.tile_start[0] = 0;
+  for (int i = 0; i < count; i++) {
+    a.seg[i] = jobs[i].seg;
+    a.tile_start[i + 1] = a.tile_start[i] + int32_t(cdiv(jobs[i].seg.n, kSortTile));
+    passes = jobs[i].passes > passes ? jobs[i].passes : passes;
+  }
+  const dim3 grid(uint32_t(a.tile_start[count]));
+  for (int pass = 0; pass < passes; pass++) {
+    a.shift = pass * 8;
+    a.parity = pass & 1;
+    a.last = pass == passes - 1;
+    HPX_LAUNCH("gd_sort_count_kernel", gd_sort_count_kernel<CAP>, grid, dim3(kSortThreads), st, a);
     if (hpx::g_prof_on) hpx::prof_begin("gd_sort_pass_kernel", st);
-    hipLaunchKernelGGL(gd_sort_pass_kernel, dim3(nblk), dim3(kSortThreads), kStageBytes, st, a);
+    hipLaunchKernelGGL(gd_sort_pass_kernel<CAP>, grid, dim3(kSortThreads), kStageBytes, st, a);
     if (hpx::g_prof_on) hpx::prof_end(st);
     HPX_HIP(hipGetLastError());
-    std::swap(keys_a, keys_b);
-    std::swap(idx_a, idx_b);
   }
-  HPX_LAUNCH("gd_gather_kernel", gd_gather_kernel, dim3(cdiv(keep > 0 ? keep : 1, kThreads)), dim3(kThreads), st, msg, r, keep);
+  for (int i = 0; i < count; i++) {
+    const uint32_t k = jobs[i].seg.keep;
+    a.tile_start[i + 1] = a.tile_start[i] + int32_t(cdiv(k > 0 ? k : 1, kThreads));
+  }
+  HPX_LAUNCH("gd_gather_kernel", gd_gather_kernel<CAP>, dim3(uint32_t(a.tile_start[count])), dim3(kThreads), st, a);
   HPX_HIP(hipGetLastError());
   return HPX_OK;
 }
 
-// One tensor.  With a residual (`residual` non-null): gd_body, s_percent = 1 - drop_ratio.  Without:
-// dgc_with_auxiliary_body, where `grad` itself is thresholded and its selected entries cleared.
-int gd_encode_one(float* grad, int32_t N, float* residual, uint8_t* out, double sample_rate, double s_percent,
-                  uint64_t seed, hpx::Workspace* ws, hipStream_t st) {
-  // size arithmetic of gd_body.h:112-115, :153 (dgc_body.h:79-80, :103)
-  const int32_t sample_cnt = static_cast<int32_t>(std::ceil(N * sample_rate));
-  const int32_t expected = static_cast<int32_t>(std::ceil(N * s_percent));
-  const int32_t thr_index = static_cast<int32_t>(sample_cnt * s_percent);
-  HPX_ARG(sample_cnt > 0 && thr_index >= 0 && thr_index < sample_cnt && expected >= 0,
-          "sparsifier encode: N=%d sample_rate=%g kept fraction=%g give sample_cnt=%d threshold index=%d", N, sample_rate,
-          s_percent, sample_cnt, thr_index);
-  const float* g = grad;
-  float* r = residual ? residual : grad;  // the array whose selected entries are read out and cleared
+// What the host works out per tensor before anything is launched (size arithmetic of gd_body.h:112-115, :153;
+// dgc_body.h:79-80, :103).
+struct Plan {
+  GdSeg seg;
+  size_t ws_bytes, cut_bytes;
+  int index;  // position in the call
+};
 
-  const uint32_t n = static_cast<uint32_t>(N);
-  const uint32_t ntiles = cdiv(n, kTile);
-  // workspace layout
-  size_t off = 0;
-  const size_t o_state = off; off += align256(sizeof(GdState));
-  const size_t o_hist = off;  off += align256(sizeof(uint32_t) * (kBins1 + kBins2 + kBins3));
-  const size_t o_samples = off; off += align256(sizeof(uint32_t) * size_t(sample_cnt));
-  const size_t o_masks = off; off += align256(sizeof(uint64_t) * size_t(ntiles) * kWave);
-  const size_t o_cnt = off; off += align256(sizeof(uint32_t) * size_t(ntiles));
-  const size_t o_off = off; off += align256(sizeof(uint32_t) * size_t(ntiles));
-  const size_t o_ctot = off; off += align256(sizeof(uint32_t) * kMaxChunks);
-  const size_t o_coff = off; off += align256(sizeof(uint32_t) * kMaxChunks);
-  // Room for the cut path (two copies of the candidates' keys and indices, and
-  // the sort's counts) is laid out for a typical overshoot before anything is
-  // launched: the expand kernel fills it without the host knowing the count.
-  uint64_t cap64 = uint64_t(expected) * 2 > uint64_t(expected) + 65536 ? uint64_t(expected) * 2 : uint64_t(expected) + 65536;
-  if (cap64 > n) cap64 = n;
-  const uint32_t cap = static_cast<uint32_t>(cap64);
-  struct CutLayout { size_t ka, kb, ia, ib, sc, end; };
-  auto cut_layout = [](size_t at, uint64_t pairs) {
-    CutLayout c;
-    c.ka = at; at += align256(sizeof(uint32_t) * size_t(pairs));
-    c.kb = at; at += align256(sizeof(uint32_t) * size_t(pairs));
-    c.ia = at; at += align256(sizeof(int32_t) * size_t(pairs));
-    c.ib = at; at += align256(sizeof(int32_t) * size_t(pairs));
-    c.sc = at; at += align256(sizeof(uint32_t) * 256 * size_t(cdiv(pairs, kSortTile)));
-    c.end = at;
-    return c;
+// The six phases for up to CAP tensors: six launch sequences, no host wait.
+template <int CAP>
+int launch_phases(const Plan* plans, int count, bool residual, uint32_t* report, hipStream_t st) {
+  GdArgs<CAP> a;
+  a.nseg = count;
+  a.residual = residual ? 1 : 0;
+  a.report = report;
+  for (int i = 0; i < count; i++) a.seg[i] = plans[i].seg;
+  auto tiles = [&](auto per_tensor) {
+    a.tile_start[0] = 0;
+    for (int i = 0; i < count; i++) a.tile_start[i + 1] = a.tile_start[i] + int32_t(per_tensor(a.seg[i]));
+    return dim3(uint32_t(a.tile_start[count]));
   };
-  CutLayout cl = cut_layout(off, cap);
-  int rc = hpx::ensure_workspace(ws, cl.end);
-  if (rc != HPX_OK) return rc;
-  uint8_t* base = ws->dev;
-  GdState* state = reinterpret_cast<GdState*>(base + o_state);
-  uint32_t* hist = reinterpret_cast<uint32_t*>(base + o_hist);
-  uint32_t* samples = reinterpret_cast<uint32_t*>(base + o_samples);
-  uint64_t* masks = reinterpret_cast<uint64_t*>(base + o_masks);
-  uint32_t* blk_cnt = reinterpret_cast<uint32_t*>(base + o_cnt);
-  uint32_t* blk_off = reinterpret_cast<uint32_t*>(base + o_off);
-  uint32_t* chunk_tot = reinterpret_cast<uint32_t*>(base + o_ctot);
-  uint32_t* chunk_off = reinterpret_cast<uint32_t*>(base + o_coff);
-  const uint32_t nchunks = cdiv(ntiles, kScanChunk);
-
-  SelArgs sa{g, residual, n, static_cast<uint32_t>(sample_cnt), static_cast<uint32_t>(seed), static_cast<uint32_t>(thr_index),
-             samples, hist, state};
-  uint32_t sel_blocks = cdiv(sample_cnt, kSelThreads * 8);
-  if (sel_blocks > kSelBlocksMax) sel_blocks = kSelBlocksMax;
-  const uint32_t zero_words = kBins1 + kBins2 + kBins3;
-  HPX_LAUNCH("gd_sample_kernel", gd_sample_kernel,
-             dim3(cdiv(uint32_t(sample_cnt) > zero_words ? uint32_t(sample_cnt) : zero_words, kThreads)), dim3(kThreads), st, sa);
-  HPX_LAUNCH("gd_select_kernel", gd_select_kernel<1>, dim3(sel_blocks), dim3(kSelThreads), st, sa);
-  HPX_LAUNCH("gd_select_kernel", gd_select_kernel<2>, dim3(sel_blocks), dim3(kSelThreads), st, sa);
-  HPX_LAUNCH("gd_select_kernel", gd_select_kernel<3>, dim3(sel_blocks), dim3(kSelThreads), st, sa);
-  HPX_LAUNCH("gd_threshold_kernel", gd_threshold_kernel, dim3(1), dim3(kSelThreads), st, sa);
+  auto sel_blocks = [](const GdSeg& sg) {
+    const uint32_t b = cdiv(sg.sample_cnt, kSelThreads * 8);
+    return b > uint32_t(kSelBlocksMax) ? uint32_t(kSelBlocksMax) : b;
+  };
+  dim3 grid = tiles([](const GdSeg& sg) { return cdiv(sg.sample_cnt > uint32_t(kHistWords) ? sg.sample_cnt : uint32_t(kHistWords), kThreads); });
+  HPX_LAUNCH("gd_sample_kernel", gd_sample_kernel<CAP>, grid, dim3(kThreads), st, a);
+  grid = tiles(sel_blocks);
+  HPX_LAUNCH("gd_select_kernel", (gd_select_kernel<1, CAP>), grid, dim3(kSelThreads), st, a);
+  HPX_LAUNCH("gd_select_kernel", (gd_select_kernel<2, CAP>), grid, dim3(kSelThreads), st, a);
+  HPX_LAUNCH("gd_select_kernel", (gd_select_kernel<3, CAP>), grid, dim3(kSelThreads), st, a);
+  HPX_LAUNCH("gd_threshold_kernel", gd_threshold_kernel<CAP>, dim3(uint32_t(count)), dim3(kSelThreads), st, a);
+  grid = tiles([](const GdSeg& sg) { return cdiv(sg.n, kTile); });
   if (residual)
-    HPX_LAUNCH("gd_stream_kernel", gd_stream_kernel<true>, dim3(ntiles), dim3(kThreads), st, g, r, n, state, masks, blk_cnt);
+    HPX_LAUNCH("gd_stream_kernel", (gd_stream_kernel<true, CAP>), grid, dim3(kThreads), st, a);
   else
-    HPX_LAUNCH("gd_stream_kernel", gd_stream_kernel<false>, dim3(ntiles), dim3(kThreads), st, g, r, n, state, masks, blk_cnt);
-  uint32_t* h_total = reinterpret_cast<uint32_t*>(ws->pinned);
-  HPX_LAUNCH("gd_scan_kernel", gd_scan_kernel, dim3(nchunks), dim3(kSelThreads), st, blk_cnt, blk_off, ntiles, chunk_tot,
-             chunk_off, state, h_total);
+    HPX_LAUNCH("gd_stream_kernel", (gd_stream_kernel<false, CAP>), grid, dim3(kThreads), st, a);
+  grid = tiles([](const GdSeg& sg) { return cdiv(cdiv(sg.n, kTile), kScanChunk); });
+  HPX_LAUNCH("gd_scan_kernel", gd_scan_kernel<CAP>, grid, dim3(kSelThreads), st, a);
   HPX_HIP(hipGetLastError());
-  // Queued before the host knows the count: the finish if nothing has to be cut,
+  // Queued before the host knows the counts: the finish where nothing has to be cut,
   // else the candidate list and keys of the cut path.
-  const uint32_t lim = static_cast<uint32_t>(expected);
-  HPX_LAUNCH("gd_expand_kernel", gd_expand_kernel, dim3(cdiv(ntiles, kThreads / kWave)), dim3(kThreads), st, masks, blk_off,
-             chunk_off, ntiles, state, lim, out, r, reinterpret_cast<int32_t*>(base + cl.ia),
-             reinterpret_cast<uint32_t*>(base + cl.ka), cap);
+  grid = tiles([](const GdSeg& sg) { return cdiv(cdiv(sg.n, kTile), kThreads / kWave); });
+  HPX_LAUNCH("gd_expand_kernel", gd_expand_kernel<CAP>, grid, dim3(kThreads), st, a);
   HPX_HIP(hipGetLastError());
-  HPX_HIP(hipStreamSynchronize(st));
-  const uint32_t total = *reinterpret_cast<volatile uint32_t*>(h_total);
-  if (total <= lim) return HPX_OK;
-
-  // More candidates than `expected`: order them by |r| descending and keep the first `expected`.
-  if (total > cap) {
-    // Far more candidates than reserved for.  Growing would discard the masks;
-    // build the larger block, carry them over and list the candidates again.
-    cl = cut_layout(off, total);
-    uint8_t* old = ws->dev;
-    const size_t old_bytes = ws->dev_bytes;
-    ws->dev = nullptr;
-    ws->dev_bytes = 0;
-    rc = hpx::ensure_workspace(ws, cl.end);
-    if (rc != HPX_OK) { (void)hipFree(old); return rc; }
-    HPX_HIP(hipMemcpyAsync(ws->dev, old, off < old_bytes ? off : old_bytes, hipMemcpyDeviceToDevice, st));
-    HPX_HIP(hipStreamSynchronize(st));
-    HPX_HIP(hipFree(old));
-    base = ws->dev;
-    state = reinterpret_cast<GdState*>(base + o_state);
-    masks = reinterpret_cast<uint64_t*>(base + o_masks);
-    blk_off = reinterpret_cast<uint32_t*>(base + o_off);
-    chunk_off = reinterpret_cast<uint32_t*>(base + o_coff);
-    HPX_LAUNCH("gd_expand_kernel", gd_expand_kernel, dim3(cdiv(ntiles, kThreads / kWave)), dim3(kThreads), st, masks, blk_off,
-               chunk_off, ntiles, state, 0u, out, r, reinterpret_cast<int32_t*>(base + cl.ia),
-               reinterpret_cast<uint32_t*>(base + cl.ka), total);
-    HPX_HIP(hipGetLastError());
-  }
-  uint32_t* ka = reinterpret_cast<uint32_t*>(base + cl.ka);
-  uint32_t* kb = reinterpret_cast<uint32_t*>(base + cl.kb);
-  int32_t* ia = reinterpret_cast<int32_t*>(base + cl.ia);
-  int32_t* ib = reinterpret_cast<int32_t*>(base + cl.ib);
-  uint32_t* sc = reinterpret_cast<uint32_t*>(base + cl.sc);
-  rc = sort_and_cut(ka, ia, kb, ib, sc, total, out, r, lim, st);
-  if (rc != HPX_OK) return rc;
   return HPX_OK;
+}
+
+// Waits until the scan launch has reported every tensor of `count` (the words are in pinned host memory and
+// the kernel writes them with system-scope stores, so they arrive while the stream is still busy with the
+// expand launch).  Polls memory; every 20 us or so it also asks whether the stream has drained, which ends the
+// wait if the words can only be seen once the kernels have finished, or if a launch failed.
+int wait_reports(volatile uint32_t* report, int count, hipStream_t st) {
+  for (int t = 0; t < count; t++) {
+    volatile uint32_t* word = report + size_t(t) * kReportWords;
+    uint32_t spins = 0;
+    while (*word == kNotReported) {
+      _mm_pause();
+      if ((++spins & 511u) == 0) {
+        const hipError_t e = hipStreamQuery(st);
+        if (e == hipErrorNotReady) { (void)hipGetLastError(); continue; }
+        if (e != hipSuccess) {
+          hpx::set_error("sparsifier encode: the stream failed: %s", hipGetErrorString(e));
+          return HPX_ERR_HIP;
+        }
+        if (*word == kNotReported) {  // everything has run and still no report
+          hpx::set_error("sparsifier encode: tensor %d was not reported by the scan launch", t);
+          return HPX_ERR_HIP;
+        }
+      }
+    }
+  }
+  __atomic_thread_fence(__ATOMIC_ACQUIRE);
+  return HPX_OK;
+}
+
+constexpr int kMaxPerWait = int((hpx::kPinnedFlagOffset) / (kReportWords * sizeof(uint32_t)));  // tensors whose reports fit the pinned block
+
+// `count` tensors.  With residuals (`residuals` non-null): gd_body, s_percent = 1 - drop_ratio.  Without:
+// dgc_with_auxiliary_body, where the gradient itself is thresholded and its selected entries cleared.
+// A tensor whose parameters make no sense is reported and skipped, like the reference driver's
+// print-and-continue; the others are encoded.
+int gd_encode_batch(int count, float* const* grads, const int32_t* Ns, float* const* residuals, uint8_t* const* outs,
+                    const double* sample_rates, const double* s_percents, const uint64_t* seeds, hpx::Workspace* ws,
+                    hipStream_t st) {
+  int worst = HPX_OK;
+  std::vector<Plan> plans;
+  plans.reserve(count);
+  size_t ws_total = 0;
+  for (int i = 0; i < count; i++) {
+    const int32_t N = Ns[i];
+    const int32_t sample_cnt = static_cast<int32_t>(std::ceil(N * sample_rates[i]));
+    const int32_t expected = static_cast<int32_t>(std::ceil(N * s_percents[i]));
+    const int32_t thr_index = static_cast<int32_t>(sample_cnt * s_percents[i]);
+    if (!(sample_cnt > 0 && thr_index >= 0 && thr_index < sample_cnt && expected >= 0)) {
+      hpx::set_error("sparsifier encode: tensor %d: N=%d sample_rate=%g kept fraction=%g give sample_cnt=%d threshold index=%d", i,
+                     N, sample_rates[i], s_percents[i], sample_cnt, thr_index);
+      if (worst == HPX_OK) worst = HPX_ERR_ARG;
+      continue;
+    }
+    Plan p;
+    const uint32_t n = static_cast<uint32_t>(N);
+    // Room for the cut path is laid out for a typical overshoot before anything is
+    // launched: the expand kernel fills it without the host knowing the count.
+    uint64_t cap64 = uint64_t(expected) * 2 > uint64_t(expected) + 65536 ? uint64_t(expected) * 2 : uint64_t(expected) + 65536;
+    if (cap64 > n) cap64 = n;
+    const uint64_t seed = seeds ? seeds[i] : hpx::clock_seed();
+    p.seg.g = grads[i];
+    p.seg.r = residuals ? residuals[i] : grads[i];
+    p.seg.out = outs[i];
+    p.seg.ws = nullptr;
+    p.seg.cut = nullptr;
+    p.seg.n = n;
+    p.seg.sample_cnt = static_cast<uint32_t>(sample_cnt);
+    p.seg.seed = static_cast<uint32_t>(seed);
+    p.seg.thr_index = static_cast<uint32_t>(thr_index);
+    p.seg.limit = static_cast<uint32_t>(expected);
+    p.seg.cap = static_cast<uint32_t>(cap64);
+    p.ws_bytes = gd_layout(n, p.seg.sample_cnt).end;
+    p.cut_bytes = cut_layout(cap64).end;
+    p.index = i;
+    ws_total += p.ws_bytes + p.cut_bytes;
+    plans.push_back(p);
+  }
+  if (plans.empty()) return worst;
+  int rc = hpx::ensure_workspace(ws, ws_total);
+  if (rc != HPX_OK) return rc;
+  {
+    size_t at = 0;
+    for (Plan& p : plans) {
+      p.seg.ws = ws->dev + at;  at += p.ws_bytes;
+      p.seg.cut = ws->dev + at; at += p.cut_bytes;
+    }
+  }
+  volatile uint32_t* report = reinterpret_cast<volatile uint32_t*>(ws->pinned);
+  const int total = int(plans.size());
+  for (int first = 0; first < total; first += kMaxPerWait) {
+    const int batch = total - first < kMaxPerWait ? total - first : kMaxPerWait;
+    for (int t = 0; t < batch; t++) report[size_t(t) * kReportWords] = kNotReported;
+    __atomic_thread_fence(__ATOMIC_RELEASE);
+    for (int k = 0; k < batch; k += kCapLarge) {
+      const int m = batch - k < kCapLarge ? batch - k : kCapLarge;
+      uint32_t* rep = const_cast<uint32_t*>(report) + size_t(k) * kReportWords;
+      rc = m <= kCapSmall ? launch_phases<kCapSmall>(&plans[first + k], m, residuals != nullptr, rep, st)
+                          : launch_phases<kCapLarge>(&plans[first + k], m, residuals != nullptr, rep, st);
+      if (rc != HPX_OK) return rc;
+    }
+    rc = wait_reports(report, batch, st);
+    if (rc != HPX_OK) return rc;
+    // More candidates than `expected`: order them by |r| descending and keep the first `expected`
+    // (gd_body.h:176-187), all such tensors of the batch together.
+    std::vector<CutJob> jobs;
+    std::vector<int> overflow;   // jobs whose candidates are more than their buffers were laid out for
+    size_t aux_need = 0;
+    for (int t = 0; t < batch; t++) {
+      const GdSeg& sg = plans[first + t].seg;
+      const uint32_t found = report[size_t(t) * kReportWords];
+      if (found <= sg.limit) continue;
+      const uint32_t thr_bits = report[size_t(t) * kReportWords + 1], max_bits = report[size_t(t) * kReportWords + 2];
+      // keys are |r| bits minus threshold bits: the largest tells how many byte digits are in use
+      const uint32_t max_key = max_bits > thr_bits ? max_bits - thr_bits : 0u;
+      CutJob job;
+      job.passes = max_key >> 24 ? 4 : max_key >> 16 ? 3 : max_key >> 8 ? 2 : 1;
+      job.seg.msg = sg.out;
+      job.seg.r = sg.r;
+      job.seg.n = found;
+      job.seg.keep = sg.limit;
+      job.seg.counts = nullptr;
+      if (found > sg.cap) {
+        overflow.push_back(int(jobs.size()));
+        aux_need += cut_layout(found).end;
+        job.seg.keys[0] = reinterpret_cast<uint32_t*>(uintptr_t(first + t));  // the plan, until the block exists
+      } else {
+        const CutLayout cl = cut_layout(sg.cap);
+        job.seg.keys[0] = reinterpret_cast<uint32_t*>(sg.cut + cl.ka);
+        job.seg.keys[1] = reinterpret_cast<uint32_t*>(sg.cut + cl.kb);
+        job.seg.idx[0] = reinterpret_cast<int32_t*>(sg.cut + cl.ia);
+        job.seg.idx[1] = reinterpret_cast<int32_t*>(sg.cut + cl.ib);
+        job.seg.counts = reinterpret_cast<uint32_t*>(sg.cut + cl.sc);
+      }
+      jobs.push_back(job);
+    }
+    if (!overflow.empty()) {
+      // Far more candidates than reserved for: list them again into a block of their own.
+      rc = hpx::ensure_aux(ws, aux_need);
+      if (rc != HPX_OK) return rc;
+      size_t at = 0;
+      for (int j : overflow) {
+        CutJob& job = jobs[j];
+        const Plan& plan = plans[size_t(reinterpret_cast<uintptr_t>(job.seg.keys[0]))];
+        const CutLayout cl = cut_layout(job.seg.n);
+        uint8_t* cut = ws->aux + at;
+        at += cl.end;
+        job.seg.keys[0] = reinterpret_cast<uint32_t*>(cut + cl.ka);
+        job.seg.keys[1] = reinterpret_cast<uint32_t*>(cut + cl.kb);
+        job.seg.idx[0] = reinterpret_cast<int32_t*>(cut + cl.ia);
+        job.seg.idx[1] = reinterpret_cast<int32_t*>(cut + cl.ib);
+        job.seg.counts = reinterpret_cast<uint32_t*>(cut + cl.sc);
+        GdArgs<kCapSmall> a;
+        a.nseg = 1;
+        a.residual = residuals != nullptr;
+        a.report = const_cast<uint32_t*>(report);  // not written by this kernel
+        a.seg[0] = plan.seg;
+        a.seg[0].cut = cut;
+        a.seg[0].cap = job.seg.n;
+        a.seg[0].limit = 0u;
+        a.tile_start[0] = 0;
+        a.tile_start[1] = int32_t(cdiv(cdiv(plan.seg.n, kTile), kThreads / kWave));
+        HPX_LAUNCH("gd_expand_kernel", gd_expand_kernel<kCapSmall>, dim3(uint32_t(a.tile_start[1])), dim3(kThreads), st, a);
+        HPX_HIP(hipGetLastError());
+      }
+    }
+    for (size_t k = 0; k < jobs.size(); k += kCapLarge) {
+      const int m = int(jobs.size() - k < size_t(kCapLarge) ? jobs.size() - k : size_t(kCapLarge));
+      rc = m <= kCapSmall ? sort_and_cut<kCapSmall>(&jobs[k], m, st) : sort_and_cut<kCapLarge>(&jobs[k], m, st);
+      if (rc != HPX_OK) return rc;
+    }
+  }
+  return worst;
 }
 
 }  // namespace
@@ -777,14 +1072,9 @@ HPX_API int hpx_gd_encode(int count, const float* const* grads, const int32_t* N
   hpx::Workspace* ws = hpx::workspace_record(st);
   if (!ws) return HPX_ERR_HIP;
   std::lock_guard<std::mutex> lock(ws->mu);
-  int worst = HPX_OK;
-  for (int i = 0; i < count; i++) {
-    const uint64_t seed = seeds ? seeds[i] : hpx::clock_seed();
-    const int rc = gd_encode_one(const_cast<float*>(grads[i]), Ns[i], residuals[i], outs[i], sample_rates[i],
-                                 1 - drop_ratios[i], seed, ws, st);
-    if (rc != HPX_OK && worst == HPX_OK) worst = rc;  // like the reference driver: report, go on
-  }
-  return worst;
+  std::vector<double> kept(count);
+  for (int i = 0; i < count; i++) kept[i] = 1 - drop_ratios[i];  // s_percent, gd_body.h:112
+  return gd_encode_batch(count, const_cast<float* const*>(grads), Ns, residuals, outs, sample_rates, kept.data(), seeds, ws, st);
 }
 
 namespace {
@@ -868,12 +1158,5 @@ HPX_API int hpx_dgc_encode(int count, float* const* grads, const int32_t* Ns, ui
   hpx::Workspace* ws = hpx::workspace_record(st);
   if (!ws) return HPX_ERR_HIP;
   std::lock_guard<std::mutex> lock(ws->mu);
-  int worst = HPX_OK;
-  for (int i = 0; i < count; i++) {
-    const uint64_t seed = seeds ? seeds[i] : hpx::clock_seed();
-    const int rc = gd_encode_one(grads[i], Ns[i], nullptr, outs[i], sample_rates[i], s_percents[i], seed, ws, st);
-    if (rc != HPX_OK && worst == HPX_OK) worst = rc;
-  }
-  return worst;
+  return gd_encode_batch(count, grads, Ns, nullptr, outs, sample_rates, s_percents, seeds, ws, st);
 }
-

@@ -49,7 +49,8 @@ int ensure_workspace(Workspace* ws, size_t dev_bytes) {
   if (!ws->state) {
     HPX_HIP(hipMalloc(reinterpret_cast<void**>(&ws->state), kStateWords * sizeof(uint32_t)));
     HPX_HIP(hipMemset(ws->state, 0, kStateWords * sizeof(uint32_t)));
-    HPX_HIP(hipHostMalloc(reinterpret_cast<void**>(&ws->pinned), kPinnedBytes, hipHostMallocDefault));
+    // coherent: words a kernel stores with system scope can be read by the host while the kernel is still running
+    HPX_HIP(hipHostMalloc(reinterpret_cast<void**>(&ws->pinned), kPinnedBytes, hipHostMallocCoherent));
     std::memset(ws->pinned, 0, kPinnedBytes);
   }
   if (dev_bytes > ws->dev_bytes) {
@@ -63,6 +64,18 @@ int ensure_workspace(Workspace* ws, size_t dev_bytes) {
     HPX_HIP(hipMalloc(reinterpret_cast<void**>(&ws->dev), want));
     ws->dev_bytes = want;
   }
+  return HPX_OK;
+}
+
+int ensure_aux(Workspace* ws, size_t bytes) {
+  if (bytes <= ws->aux_bytes) return HPX_OK;
+  HPX_HIP(hipStreamSynchronize(ws->stream));
+  if (ws->aux) HPX_HIP(hipFree(ws->aux));
+  ws->aux = nullptr;
+  ws->aux_bytes = 0;
+  const size_t want = (bytes + bytes / 8 + 255) & ~size_t(255);
+  HPX_HIP(hipMalloc(reinterpret_cast<void**>(&ws->aux), want));
+  ws->aux_bytes = want;
   return HPX_OK;
 }
 
@@ -130,11 +143,12 @@ namespace {
 int free_workspace(Workspace* ws) {
   int rc = HPX_OK;
   if (ws->dev && hipFree(ws->dev) != hipSuccess) rc = HPX_ERR_HIP;
+  if (ws->aux && hipFree(ws->aux) != hipSuccess) rc = HPX_ERR_HIP;
   if (ws->state && hipFree(ws->state) != hipSuccess) rc = HPX_ERR_HIP;
   if (ws->slots && hipFree(ws->slots) != hipSuccess) rc = HPX_ERR_HIP;
   if (ws->bar && hipFree(ws->bar) != hipSuccess) rc = HPX_ERR_HIP;
   if (ws->pinned && hipHostFree(ws->pinned) != hipSuccess) rc = HPX_ERR_HIP;
-  ws->dev = nullptr; ws->state = nullptr; ws->slots = nullptr; ws->bar = nullptr; ws->pinned = nullptr;
+  ws->dev = nullptr; ws->aux = nullptr; ws->state = nullptr; ws->slots = nullptr; ws->bar = nullptr; ws->pinned = nullptr;
   return rc;
 }
 }  // namespace
