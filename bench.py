@@ -53,6 +53,8 @@ def parse():
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="time budget of the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the TBQ / DGC / PowerSGD side measurements")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only", default="", help="profiling aid: run just these side measurements (comma-separated names of "
+                    "EXTRAS below, e.g. powersgd) and print them; no headline, no CPU leg")
     ap.add_argument("--copy-calibration", type=int, default=0,
                     help="also run this many plain 4*N-byte device copies (a kernel of known traffic for scaling "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings)")
@@ -126,6 +128,10 @@ def main():
     L = capi.load()
     stream = torch.cuda.current_stream().cuda_stream
     gen = torch.Generator(device="cuda").manual_seed(0)
+    if args.only:
+        names = [w for w in args.only.split(",") if w]
+        print(json.dumps({"only": names, "extra": extra(torch, np, capi, L, stream, gen, names)}), flush=True)
+        return
 
     # ---- headline: TernGrad 2-bit encode + decode, N = 25,557,032 --------------------------
     n = N_TERNGRAD
@@ -180,6 +186,8 @@ def main():
     achieved = alg_bytes[dom] / kt[dom] / 1e9
     roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(dom),
+                "traffic_is": "not read in this run: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, scaled by a plain "
+                              "copy's readings, from profiles/terngrad_25M_pmc_fetch_write.txt",
                 "algorithmic_bytes_per_launch": alg_bytes[dom], "avg_launch_us": round(kt[dom] * 1e6, 2),
                 "kernel_us": {k: (round(v * 1e6, 2) if v else None) for k, v in kt.items()}}
     path_alg = 8.5 * n  # x once in, codes out; codes in, fp32 out
@@ -199,7 +207,7 @@ def main():
 
     del sets
     torch.cuda.empty_cache()
-    result["plain_streams"] = plain_streams(torch, capi, L, stream, n)
+    result["plain_streams"] = plain_streams(torch, stream, n)
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(np, n, args.cpu_seconds)
@@ -208,11 +216,14 @@ def main():
     print(json.dumps(result), flush=True)
 
 
-def plain_streams(torch, capi, L, stream, n):
-    """What the memory system gives the simplest kernels of the codecs' shapes (hpx_probe_stream), measured the way
-    the headline is: buffers rotate over distinct sets, HIP events on the launch stream around each kernel.  The
-    TernGrad step reads 4*n bytes once and writes 4*n bytes once, so read + write of 4*n bytes is the time below
-    which no encode+decode of this tensor can go on this part."""
+def plain_streams(torch, stream, n):
+    """What the memory system gives the simplest kernels of the codecs' shapes (bench_probe.hip, built beside this
+    file; not part of the product library), measured the way the headline is: buffers rotate over distinct sets,
+    events on the launch stream around each kernel.  The TernGrad step reads 4*n bytes once and writes 4*n bytes
+    once, so read + write of 4*n bytes is the time below which no encode+decode of this tensor can go on this part."""
+    import __graft_entry__
+    probe = C.CDLL(__graft_entry__.BENCH_PROBE)
+    probe.bench_probe_stream.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]
     names = {0: "read", 1: "write_streaming", 2: "write_plain", 3: "read_read_write"}
     out = {}
     for label, elems, nsets in (("headline_tensor", n, 6), ("440MB", 110_000_000, 3)):
@@ -225,12 +236,20 @@ def plain_streams(torch, capi, L, stream, n):
 
             def f():
                 i[0] += 1
-                rc = L.hpx_probe_stream(kind, a[i[0] % nsets].data_ptr(), b.data_ptr(), nbytes, stream)
-                assert rc == 0, capi.last_error()
+                rc = probe.bench_probe_stream(kind, a[i[0] % nsets].data_ptr(), b.data_ptr(), nbytes, stream)
+                assert rc == 0, rc
 
             for _ in range(2 * nsets):   # untimed: clocks up, the zero fill's dirty lines out of the caches
                 f()
-            kt = kernel_times(torch, capi, f, ["probe_stream_kernel"], reps=24)["probe_stream_kernel"]
+            reps = 24
+            evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+            torch.cuda.synchronize()
+            for e0, e1 in evs:           # the launches go out on torch's current stream, which `stream` is
+                e0.record()
+                f()
+                e1.record()
+            torch.cuda.synchronize()
+            kt = sum(e0.elapsed_time(e1) for e0, e1 in evs) / reps * 1e-3
             traffic = nbytes * (3 if kind == 3 else 1)
             res[name] = {"us": round(kt * 1e6, 2), "GBps": round(traffic / kt / 1e9, 1),
                          "frac_of_hbm_peak": round(traffic / kt / 1e9 / HBM_PEAK_GBS, 4)}
@@ -282,15 +301,36 @@ def cpu_baseline(np, n, budget_s):
     return res
 
 
-def extra(torch, np, capi, L, stream, gen):
-    """Other codecs of the path at their configuration sizes (GPU only, short runs)."""
-    res = {}
-    # ---- TBQ fused bucket: 110M elements in 200 tensors, thr = 2 sigma ----------------------
+def kernel_roofline(kt, alg_bytes):
+    """The roofline block of a side measurement: its dominant kernel (longest average launch among those with
+    algorithmic bytes) priced against the HBM peak, as the headline's is."""
+    cand = {k: v for k, v in kt.items() if v and k in alg_bytes}
+    if not cand:
+        return None
+    dom = max(cand, key=cand.get)
+    ach = alg_bytes[dom] / cand[dom] / 1e9
+    return {"bound": "hbm", "kernel": dom, "avg_launch_us": round(cand[dom] * 1e6, 2), "algorithmic_bytes": alg_bytes[dom],
+            "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4)}
+
+
+def bucket_sizes(np):
+    """The 200 tensor sizes of the fused-bucket configuration (110 M elements, log-uniform in [768, 3e7])."""
     rng = np.random.default_rng(0)
     sizes = np.exp(rng.uniform(np.log(768), np.log(3e7), 200))
     sizes = np.clip(np.floor(sizes * 110e6 / sizes.sum()), 768, 3e7).astype(np.int64)
     sizes[np.argmax(sizes)] += 110_000_000 - sizes.sum()
-    tot = int(sizes.sum())
+    return [int(x) for x in sizes]
+
+
+# MFMA busy cycles of the PowerSGD kernels from a counter run of `bench.py --only powersgd`
+# (profiles/powersgd_mfma_busy.txt): SQ_VALU_MFMA_BUSY_CYCLES / SQ_BUSY_CYCLES per kernel, not read in this run.
+MEASURED_MFMA_BUSY = None
+
+
+def x_tbq(torch, np, capi, L, stream, gen, res):
+    # ---- TBQ fused bucket: 110M elements in 200 tensors, thr = 2 sigma ----------------------
+    sizes = bucket_sizes(np)
+    tot = sum(sizes)
     gs = [torch.randn(int(s), device="cuda", generator=gen) * 5e-3 for s in sizes]
     rs = [torch.zeros(int(s), device="cuda") for s in sizes]
     ps = [torch.zeros((int(s) + 3) // 4, dtype=torch.uint8, device="cuda") for s in sizes]
@@ -312,7 +352,8 @@ def extra(torch, np, capi, L, stream, gen):
     res["tbq_bucket_110M_200_tensors"] = {
         "ms_per_step": round(sec * 1e3, 4), "GBps_of_gradient": round(4.0 * tot / sec / 1e9, 1),
         "algorithmic_bytes": 16.5 * tot, "frac_of_hbm_peak": round(16.5 * tot / sec / 1e9 / HBM_PEAK_GBS, 4),
-        "kernel_us_per_launch": {k: round(v * 1e6, 1) for k, v in kt.items() if v}}
+        "kernel_us_per_launch": {k: round(v * 1e6, 1) for k, v in kt.items() if v},
+        "roofline": kernel_roofline(kt, {"tbq_encode_kernel": 12.25 * tot, "tbq_decode_kernel": 4.25 * tot})}
     # the root's gather-decode: 7 gathered messages per tensor accumulate into the tensor (hp_cuda.cpp:241-259)
     slots = 7
     msgs7 = [[torch.randint(0, 255, ((int(s) + 3) // 4,), dtype=torch.uint8, device="cuda", generator=gen) & 0xA5
@@ -325,14 +366,20 @@ def extra(torch, np, capi, L, stream, gen):
                 capi.i32_array([int(s) for s in sizes] * slots), capi.ptr_array([m_.data_ptr() for m_ in ins7]),
                 capi.f32_array([1e-2] * (slots * len(sizes))), capi.i32_array([1] * (slots * len(sizes))), stream)
     sec = timed(torch, root, 10, 2)
+    kt = kernel_times(torch, capi, root, ["tbq_decode_multi_kernel"], reps=5)
     alg = (8.0 + 0.25 * slots) * tot
     res["tbq_root_decode_add_7_messages_per_tensor"] = {
         "ms": round(sec * 1e3, 4), "algorithmic_bytes": alg, "frac_of_hbm_peak": round(alg / sec / 1e9 / HBM_PEAK_GBS, 4),
-        "bytes_if_applied_one_message_at_a_time": 8.25 * slots * tot}
-    del gs, rs, ps, os_, msgs7, outs7, ins7
-    torch.cuda.empty_cache()
+        "bytes_if_applied_one_message_at_a_time": 8.25 * slots * tot,
+        "roofline": {"bound": "hbm", "kernel": "tbq_decode_multi_kernel (all launches of the call)", "avg_launch_us": round(sec * 1e6, 2),
+                     "algorithmic_bytes": alg, "achieved": round(alg / sec / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(alg / sec / 1e9 / HBM_PEAK_GBS, 4),
+                     "kernel_us_per_launch": round(kt["tbq_decode_multi_kernel"] * 1e6, 1) if kt["tbq_decode_multi_kernel"] else None}}
 
-    # the same for TernGrad: 7 gathered 2-bit messages of the 25.56 M-element gradient accumulate into it
+
+def x_terngrad_root(torch, np, capi, L, stream, gen, res):
+    # 7 gathered 2-bit messages of the 25.56 M-element gradient accumulate into it (the root's gather-decode)
+    slots = 7
     n = N_TERNGRAD
     x = outlier_gradient(torch, n, gen)
     nbytes = 10 + (n + 3) // 4
@@ -345,13 +392,15 @@ def extra(torch, np, capi, L, stream, gen):
     troot = Call(L.hpx_terngrad_decode, slots, capi.ptr_array([acc.data_ptr()] * slots), capi.i32_array([n] * slots),
                  capi.ptr_array([m_.data_ptr() for m_ in msgs]), capi.i32_array([nbytes] * slots), capi.i32_array([1] * slots), stream)
     sec = timed(torch, troot, 30, 5)
+    kt = kernel_times(torch, capi, troot, ["terngrad_decode_multi_kernel"], reps=10)
     alg = (8.0 + 0.25 * slots) * n
     res["terngrad_root_decode_add_7_messages_25M"] = {
         "ms": round(sec * 1e3, 4), "algorithmic_bytes": alg, "frac_of_hbm_peak": round(alg / sec / 1e9 / HBM_PEAK_GBS, 4),
-        "bytes_if_applied_one_message_at_a_time": 8.25 * slots * n}
-    del x, msgs, acc
-    torch.cuda.empty_cache()
+        "bytes_if_applied_one_message_at_a_time": 8.25 * slots * n,
+        "roofline": kernel_roofline(kt, {"terngrad_decode_multi_kernel": alg})}
 
+
+def x_terngrad_resnet50(torch, np, capi, L, stream, gen, res):
     # ---- TernGrad over ResNet-50's own 161 parameter tensors (the same 25,557,032 elements, one call each way) ----
     r50 = [64 * 3 * 7 * 7, 64, 64]
     inp = 64
@@ -378,16 +427,24 @@ def extra(torch, np, capi, L, stream, gen):
         dec()
 
     sec = timed(torch, r50_step, 50, 10)
+    kt = kernel_times(torch, capi, r50_step, ["terngrad_resident_multi_kernel", "terngrad_decode_kernel"], reps=10)
     L.hpx_set_option(b"terngrad_resident_bucket", 0)          # the same call as a min/max launch and a quantise launch
     sec_tiled = timed(torch, r50_step, 50, 10)
     L.hpx_set_option(b"terngrad_resident_bucket", 1)
+    msg_bytes = sum(10 + (m_ + 3) // 4 for m_ in r50)
     res["terngrad_resnet50_161_tensors"] = {
         "ms_per_step": round(sec * 1e3, 4), "tensors": k_, "launches_per_step": 2,
         "algorithmic_bytes": 8.5 * N_TERNGRAD, "frac_of_hbm_peak": round(8.5 * N_TERNGRAD / sec / 1e9 / HBM_PEAK_GBS, 4),
-        "ms_per_step_with_the_two_launch_encode": round(sec_tiled * 1e3, 4)}
-    del xs, ms_, ds_
-    torch.cuda.empty_cache()
+        "ms_per_step_with_the_two_launch_encode": round(sec_tiled * 1e3, 4),
+        "roofline": kernel_roofline(kt, {"terngrad_resident_multi_kernel": 4.0 * N_TERNGRAD + msg_bytes,
+                                         "terngrad_decode_kernel": 4.0 * N_TERNGRAD + msg_bytes})}
 
+
+GD_KERNELS = ["gd_sample_kernel", "gd_select_kernel", "gd_threshold_kernel", "gd_stream_kernel", "gd_scan_kernel",
+              "gd_expand_kernel", "gd_sort_count_kernel", "gd_sort_pass_kernel", "gd_gather_kernel"]
+
+
+def x_dgc(torch, np, capi, L, stream, gen, res):
     # ---- DGC / GradDrop top-0.1 %: 138,357,544 elements --------------------------------------
     n = N_DGC
     u = torch.rand(n, device="cuda", generator=gen) - 0.5
@@ -397,9 +454,6 @@ def extra(torch, np, capi, L, stream, gen):
     r = r0.clone()
     out = torch.zeros(4 + 8 * int(np.ceil(n * (1 - 0.999))), dtype=torch.uint8, device="cuda")
     scrub = torch.empty(160_000_000, device="cuda")  # 640 MB, larger than L2 + Infinity Cache
-    sort_kernels = ["gd_sort_count_kernel", "gd_sort_pass_kernel", "gd_gather_kernel"]
-    all_kernels = ["gd_sample_kernel", "gd_select_kernel", "gd_threshold_kernel", "gd_stream_kernel", "gd_scan_kernel",
-                   "gd_expand_kernel"] + sort_kernels
     # Whether the sampled threshold lets through more than the `expected` entries (and the call has to sort and
     # cut) depends on the sample, i.e. on the seed: time several seeds and report each.
     per_seed = []
@@ -413,13 +467,13 @@ def extra(torch, np, capi, L, stream, gen):
             scrub.sum()                      # push the copy's dirty lines out of the caches: inputs are in HBM when the clock starts
             torch.cuda.synchronize()
             t0 = time.perf_counter()
-            gd()
+            gd()                             # returns once the counts are known; the tail of the work is still queued
             torch.cuda.synchronize()
             times.append(time.perf_counter() - t0)
         k = (int(out[:4].cpu().numpy().view(np.int32)[0]) - 4) // 8
         r.copy_(r0)
         scrub.sum()
-        kts = kernel_times(torch, capi, gd, all_kernels, reps=1)
+        kts = kernel_times(torch, capi, gd, GD_KERNELS, reps=1)
         cut = kts["gd_gather_kernel"] is not None
         per_seed.append({"seed": seed, "encode_ms": round(float(np.median(times[2:])) * 1e3, 4), "selected": k, "cut": cut})
         if kt is None or (cut and kt["gd_gather_kernel"] is None):
@@ -434,7 +488,8 @@ def extra(torch, np, capi, L, stream, gen):
         "encode_GBps_of_gradient": round(4.0 * n / sec / 1e9, 1),
         "algorithmic_bytes": 12.0 * n + 8 * k + 4, "frac_of_hbm_peak": round((12.0 * n + 8 * k + 4) / sec / 1e9 / HBM_PEAK_GBS, 4),
         "stream_kernel_frac_of_hbm_peak": round(12.0 * n / kt["gd_stream_kernel"] / 1e9 / HBM_PEAK_GBS, 4) if kt["gd_stream_kernel"] else None,
-        "decode_add_ms": round(sec_dec * 1e3, 4), "kernel_us_per_launch": {k_: round(v * 1e6, 1) for k_, v in kt.items() if v}}
+        "decode_add_ms": round(sec_dec * 1e3, 4), "kernel_us_per_launch": {k_: round(v * 1e6, 1) for k_, v in kt.items() if v},
+        "roofline": kernel_roofline(kt, {"gd_stream_kernel": 12.0 * n})}
     # the same sparsifier without residual (dgc_body.h): reads the gradient once, 4 B/elt
     del r, r0, dout
     g0 = g.clone()
@@ -450,13 +505,77 @@ def extra(torch, np, capi, L, stream, gen):
         torch.cuda.synchronize()
         times.append(time.perf_counter() - t0)
     sec_nr = float(np.median(times[2:]))
+    g.copy_(g0)
+    scrub.sum()
+    kt = kernel_times(torch, capi, dgc, GD_KERNELS, reps=1)
     res["dgc_without_residual_138M"] = {
         "encode_ms": round(sec_nr * 1e3, 4), "algorithmic_bytes": 4.0 * n,
         "frac_of_hbm_peak": round(4.0 * n / sec_nr / 1e9 / HBM_PEAK_GBS, 4),
-        "selected": (int(out[:4].cpu().numpy().view(np.int32)[0]) - 4) // 8}
-    del g, g0, out, scrub
-    torch.cuda.empty_cache()
+        "selected": (int(out[:4].cpu().numpy().view(np.int32)[0]) - 4) // 8,
+        "roofline": kernel_roofline(kt, {"gd_stream_kernel": 4.0 * n})}
 
+
+def x_dgc_bucket(torch, np, capi, L, stream, gen, res):
+    # ---- GradDrop over the 200-tensor bucket (110 M elements): one call against one call per tensor -------------
+    sizes = bucket_sizes(np)
+    tot = sum(sizes)
+    gs = [torch.randn(s, device="cuda", generator=gen) * 5e-3 for s in sizes]
+    r0 = [torch.randn(s, device="cuda", generator=gen) * 1e-4 for s in sizes]
+    rs = [t.clone() for t in r0]
+    outs = [torch.zeros(4 + 8 * int(np.ceil(s * 0.001)) + 64, dtype=torch.uint8, device="cuda") for s in sizes]
+
+    def call(idx):
+        return Call(L.hpx_gd_encode, len(idx), capi.ptr_array([gs[i].data_ptr() for i in idx]), capi.i32_array([sizes[i] for i in idx]),
+                    capi.ptr_array([rs[i].data_ptr() for i in idx]), capi.ptr_array([outs[i].data_ptr() for i in idx]),
+                    capi.f64_array([0.01] * len(idx)), capi.f64_array([0.999] * len(idx)), capi.u64_array([7 + i for i in idx]), stream)
+
+    whole = call(list(range(len(sizes))))
+    singles = [call([i]) for i in range(len(sizes))]
+
+    def one_by_one():
+        for c_ in singles:
+            c_()
+
+    def run(f, reps):
+        ts = []
+        for it in range(reps):
+            for a, b in zip(rs, r0):
+                a.copy_(b)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            f()
+            torch.cuda.synchronize()
+            ts.append(time.perf_counter() - t0)
+        return float(np.median(ts[1:]))
+
+    sec = run(whole, 6)
+    sec_loop = run(one_by_one, 3)
+    for a, b in zip(rs, r0):
+        a.copy_(b)
+    torch.cuda.synchronize()
+    L.hpx_profile_reset()
+    L.hpx_profile_enable(1)
+    whole()
+    torch.cuda.synchronize()
+    L.hpx_profile_enable(0)
+    per_call = {k_: capi.profile_query(k_) for k_ in GD_KERNELS}      # (total ms, launches) of the one call
+    L.hpx_profile_reset()
+    kt = {k_: (ms_ / n_) * 1e-3 if n_ else None for k_, (ms_, n_) in per_call.items()}
+    stream_s = per_call["gd_stream_kernel"][0] * 1e-3
+    cut = sum(1 for o, s in zip(outs, sizes) if (int(o[:4].cpu().numpy().view(np.int32)[0]) - 4) // 8 == int(np.ceil(s * 0.001)))
+    res["dgc_bucket_110M_200_tensors"] = {
+        "encode_ms_one_call": round(sec * 1e3, 4), "encode_ms_one_call_per_tensor": round(sec_loop * 1e3, 4),
+        "tensors": len(sizes), "tensors_filled_to_expected": cut,
+        "algorithmic_bytes": 12.0 * tot, "frac_of_hbm_peak": round(12.0 * tot / sec / 1e9 / HBM_PEAK_GBS, 4),
+        "kernel_us_per_launch": {k_: round(v * 1e6, 1) for k_, v in kt.items() if v},
+        "launches_per_call": {k_: n_ for k_, (ms_, n_) in per_call.items() if n_},
+        # the stream pass runs once per table of 128 tensors: both launches of the call together against all its bytes
+        "roofline": {"bound": "hbm", "kernel": "gd_stream_kernel (both launches of the call)", "avg_launch_us": round(stream_s * 1e6, 2),
+                     "algorithmic_bytes": 12.0 * tot, "achieved": round(12.0 * tot / stream_s / 1e9, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(12.0 * tot / stream_s / 1e9 / HBM_PEAK_GBS, 4)}}
+
+
+def x_powersgd(torch, np, capi, L, stream, gen, res):
     # ---- PowerSGD rank 4 over the 36-matrix layer set ------------------------------------------
     shapes = [(4096, 4096)] * 12 + [(1024, 4096)] * 12 + [(4096, 1024)] * 12
     rk = 4
@@ -478,20 +597,27 @@ def extra(torch, np, capi, L, stream, gen):
         dc()
 
     sec = timed(torch, psgd_step, 10, 2)
-    kt = kernel_times(torch, capi, psgd_step, ["psgd_encode1_kernel", "psgd_orth_kernel", "psgd_mtp_kernel",
-                                               "psgd_qreduce_kernel", "psgd_decode_kernel"], reps=3)
+    names = ["psgd_encode1_kernel", "psgd_orth_kernel", "psgd_mtp_kernel", "psgd_qreduce_kernel", "psgd_decode_kernel"]
+    kt = kernel_times(torch, capi, psgd_step, names, reps=3)
     elems = sum(a * b for a, b in shapes)
     flops = 24.0 * elems
+    # per kernel: 2 * n*m*r flops each for P = MQ, Q = M^T P and M = P Q^T
+    kflops = {"psgd_encode1_kernel": 8.0 * elems, "psgd_mtp_kernel": 8.0 * elems, "psgd_decode_kernel": 8.0 * elems}
     res["powersgd_rank4_36_matrices"] = {
         "ms_per_iteration": round(sec * 1e3, 4), "GBps_of_gradient": round(4.0 * elems / sec / 1e9, 1),
         "algorithmic_bytes": 16.0 * elems, "frac_of_hbm_peak": round(16.0 * elems / sec / 1e9 / HBM_PEAK_GBS, 4),
         "bytes_moved_by_three_phase_api": 32.0 * elems,
         "frac_of_hbm_peak_three_phase_bytes": round(32.0 * elems / sec / 1e9 / HBM_PEAK_GBS, 4),
         "mfma_frac_of_fp32_peak": round(flops / sec / 1e12 / FP32_MFMA_PEAK_TF, 5),
-        "kernel_us_per_launch": {k_: round(v * 1e6, 1) for k_, v in kt.items() if v}}
-    del G, R
-    torch.cuda.empty_cache()
+        "mfma_frac_of_fp32_peak_is": "flops / wall time / 157.3 TFLOP/s",
+        "mfma_frac_of_fp32_peak_per_kernel": {k_: round(kflops[k_] / kt[k_] / 1e12 / FP32_MFMA_PEAK_TF, 5) for k_ in kflops if kt.get(k_)},
+        "mfma_busy_from_counters": MEASURED_MFMA_BUSY,
+        "kernel_us_per_launch": {k_: round(v * 1e6, 1) for k_, v in kt.items() if v},
+        "roofline": kernel_roofline(kt, {"psgd_encode1_kernel": 12.0 * elems, "psgd_mtp_kernel": 4.0 * elems,
+                                         "psgd_decode_kernel": 16.0 * elems})}
 
+
+def x_scheduler(torch, np, capi, L, stream, gen, res):
     # ---- the scheduler around the path: one COMP task, submit -> name in the finished queue ------------
     # (TernGrad 2-bit, 25.56 M elements; includes the 6.4 MB device-to-host copy of the message into a
     # pinned C buffer and both thread hand-overs; the reference's worker polls its queue every 500 us)
@@ -523,9 +649,7 @@ def extra(torch, np, capi, L, stream, gen):
     # 200 COMP tasks at once (the TBQ bucket, 110 M elements): the worker batches what is queued into
     # multi-tensor encodes; 27.5 MB of messages go to pinned C buffers on the data stream
     if hp.init("tbq", {"threshold": 1e-2}, torch.cuda.current_device(), 0, 2):
-        rng = np.random.default_rng(0)
-        sizes = np.exp(rng.uniform(np.log(768), np.log(3e7), 200))
-        sizes = np.clip(np.floor(sizes * (110e6 / sizes.sum())), 768, 3e7).astype(np.int64)
+        sizes = bucket_sizes(np)
         gs = [torch.randn(int(n_), device="cuda", generator=gen) * 5e-3 for n_ in sizes]
         rs = [torch.zeros(int(n_), device="cuda") for n_ in sizes]
         Bs = [torch.zeros((int(n_) + 3) // 4, dtype=torch.uint8, device="cuda") for n_ in sizes]
@@ -547,8 +671,24 @@ def extra(torch, np, capi, L, stream, gen):
         msg_bytes = int(sum((int(n_) + 3) // 4 for n_ in sizes))
         res["scheduler_tbq_bucket_200_comp_tasks"] = {
             "submit_all_to_all_finished_ms_median": round(float(np.median(lat)) * 1e3, 4),
-            "elements": int(sizes.sum()), "message_bytes_to_host": msg_bytes,
-            "GBps_of_gradient": round(4.0 * float(sizes.sum()) / float(np.median(lat)) / 1e9, 1), "errors": hp.error_count()}
+            "elements": int(sum(sizes)), "message_bytes_to_host": msg_bytes,
+            "GBps_of_gradient": round(4.0 * float(sum(sizes)) / float(np.median(lat)) / 1e9, 1), "errors": hp.error_count()}
+
+
+EXTRAS = {"tbq": x_tbq, "terngrad_root": x_terngrad_root, "terngrad_resnet50": x_terngrad_resnet50, "dgc": x_dgc,
+          "dgc_bucket": x_dgc_bucket, "powersgd": x_powersgd, "scheduler": x_scheduler}
+
+
+def extra(torch, np, capi, L, stream, gen, only=None):
+    """Other codecs of the path at their configuration sizes (GPU only, short runs).  Every entry carries the same
+    kind of roofline block as the headline: its dominant kernel, that kernel's average launch time (HIP events on
+    the launch stream), its algorithmic bytes and the fraction of the HBM peak."""
+    res = {}
+    for name, fn in EXTRAS.items():
+        if only and name not in only:
+            continue
+        fn(torch, np, capi, L, stream, gen, res)
+        torch.cuda.empty_cache()
     return res
 
 

@@ -91,17 +91,6 @@ int hpx_profile_enable(int on);
 int hpx_profile_reset(void);
 int hpx_profile_query(const char* kernel, double* total_ms, int64_t* launches);
 
-/* Plain streaming kernels of known traffic, for pricing the codecs against what
- * the memory system gives the simplest possible kernel of the same shape
- * (16 KiB per workgroup, 128-bit accesses, launch order = address order):
- *   kind 0  read `bytes` of a            (non-temporal loads)
- *   kind 1  write `bytes` of a           (non-temporal stores)
- *   kind 2  write `bytes` of a           (plain stores)
- *   kind 3  a = a + b over `bytes` each  (read, read, write in place; non-temporal)
- * a and b are device pointers, 16-byte aligned; bytes is rounded down to a
- * multiple of 16 KiB.  No counterpart in the reference. */
-int hpx_probe_stream(int kind, void* a, const void* b, int64_t bytes, hpx_stream_t stream);
-
 /* ---- TBQ: threshold quantisation with residual feedback ------------------ */
 
 /* Replaces hp_cuda_tbq (hp_cuda.cpp:52-61, hp_cuda_kernel.cu:120-158; body

@@ -20,7 +20,6 @@ SYMBOLS = (
     "hpx_profile_enable",
     "hpx_profile_reset",
     "hpx_profile_query",
-    "hpx_probe_stream",
     "hpx_tbq_encode",
     "hpx_tbq_decode",
     "hpx_terngrad_encode",
@@ -88,7 +87,6 @@ def load():
     L.hpx_release_workspaces.restype = C.c_int
     L.hpx_profile_enable.argtypes = [C.c_int]
     L.hpx_profile_query.argtypes = [C.c_char_p, C.POINTER(C.c_double), C.POINTER(C.c_int64)]
-    L.hpx_probe_stream.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]
     L.hpx_set_option.argtypes = [C.c_char_p, C.c_int64]
     L.hpx_get_option.argtypes = [C.c_char_p, C.POINTER(C.c_int64)]
     L.hpx_tbq_encode.argtypes = [i32, pp, p, pp, pp, p, p]

@@ -118,7 +118,7 @@ struct GdSeg {
 static_assert(sizeof(GdSeg) == 64, "segment record");
 // What the scan launch reports per tensor in pinned host memory.
 constexpr int kReportWords = 4;  // count of candidates, threshold bits, bits of the largest |r|, unused
-constexpr uint32_t kNotReported = 0xFFFFFFFFu;  // a count is < 2^31
+constexpr uint32_t kNotReported = 0xFFFFFFFFu;  // a count is < 2^31; as fp32 bits this is a NaN, which no threshold or |r| is
 template <int CAP>
 struct GdArgs {
   int32_t nseg;
@@ -431,12 +431,12 @@ __global__ __launch_bounds__(kSelThreads) void gd_scan_kernel(const GdArgs<CAP> 
     if (2 * t + 1 < nchunks) chunk_off[2 * t + 1] = ex + a0;
     if (t == kWave - 1) {
       st->total = inc2;
-      // Pinned host words the host polls (no copy command, no wait for the stream): threshold and largest
-      // |r| first, the count - whose arrival the host waits for - last.
+      // Pinned host words the host polls (no copy command, no wait for the stream).  The host waits for each
+      // of the three words to change, so plain system-scope stores do (a release would write the whole L2 back).
       uint32_t* rep = a.report + size_t(s) * kReportWords;
+      __hip_atomic_store(rep + 0, inc2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
       __hip_atomic_store(rep + 1, st->thr_bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
       __hip_atomic_store(rep + 2, mm, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-      __hip_atomic_store(rep + 0, inc2, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
     }
   }
 }
@@ -888,7 +888,8 @@ int wait_reports(volatile uint32_t* report, int count, hipStream_t st) {
   for (int t = 0; t < count; t++) {
     volatile uint32_t* word = report + size_t(t) * kReportWords;
     uint32_t spins = 0;
-    while (*word == kNotReported) {
+    auto pending = [word]() { return word[0] == kNotReported || word[1] == kNotReported || word[2] == kNotReported; };
+    while (pending()) {
       _mm_pause();
       if ((++spins & 511u) == 0) {
         const hipError_t e = hipStreamQuery(st);
@@ -897,7 +898,7 @@ int wait_reports(volatile uint32_t* report, int count, hipStream_t st) {
           hpx::set_error("sparsifier encode: the stream failed: %s", hipGetErrorString(e));
           return HPX_ERR_HIP;
         }
-        if (*word == kNotReported) {  // everything has run and still no report
+        if (pending()) {  // everything has run and still no report
           hpx::set_error("sparsifier encode: tensor %d was not reported by the scan launch", t);
           return HPX_ERR_HIP;
         }
@@ -970,7 +971,8 @@ int gd_encode_batch(int count, float* const* grads, const int32_t* Ns, float* co
   const int total = int(plans.size());
   for (int first = 0; first < total; first += kMaxPerWait) {
     const int batch = total - first < kMaxPerWait ? total - first : kMaxPerWait;
-    for (int t = 0; t < batch; t++) report[size_t(t) * kReportWords] = kNotReported;
+    for (int t = 0; t < batch; t++)
+      for (int w = 0; w < 3; w++) report[size_t(t) * kReportWords + w] = kNotReported;
     __atomic_thread_fence(__ATOMIC_RELEASE);
     for (int k = 0; k < batch; k += kCapLarge) {
       const int m = batch - k < kCapLarge ? batch - k : kCapLarge;

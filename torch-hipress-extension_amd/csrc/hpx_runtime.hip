@@ -313,42 +313,6 @@ int copy_ranges(int count, uint8_t* const* dst, const uint8_t* const* src, const
   return HPX_OK;
 }
 
-// ---- plain streams of known traffic (hpx_probe_stream) ---------------------------
-namespace {
-constexpr int kProbeThreads = 256;
-constexpr int kProbeIters = 4;  // 16 KiB per workgroup
-template <int KIND>
-__global__ __launch_bounds__(kProbeThreads) void probe_stream_kernel(float* __restrict__ a, const float* __restrict__ b) {
-  const uint32_t lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-  const size_t g0 = size_t(blockIdx.x) * (kProbeThreads * kProbeIters) + wave * (kWave * kProbeIters) + lane;  // float4 units
-  if (KIND == 0) {
-    float4 v[kProbeIters];
-#pragma unroll
-    for (int k = 0; k < kProbeIters; k++) v[k] = ld4_stream(a + (g0 + k * kWave) * 4);
-    float s = 0.f;
-#pragma unroll
-    for (int k = 0; k < kProbeIters; k++) s += v[k].x + v[k].y + v[k].z + v[k].w;
-    if (s == 1.2345e38f) a[0] = s;  // keeps the loads; never true for finite data of ordinary size
-  } else if (KIND == 1 || KIND == 2) {
-#pragma unroll
-    for (int k = 0; k < kProbeIters; k++) {
-      const float4 v = make_float4(1.f, 2.f, 3.f, float(k));
-      if (KIND == 1) st4_stream(a + (g0 + k * kWave) * 4, v); else st4(a + (g0 + k * kWave) * 4, v);
-    }
-  } else {
-    float4 x[kProbeIters], y[kProbeIters];
-#pragma unroll
-    for (int k = 0; k < kProbeIters; k++) {
-      x[k] = ld4_stream(a + (g0 + k * kWave) * 4);
-      y[k] = ld4_stream(b + (g0 + k * kWave) * 4);
-    }
-#pragma unroll
-    for (int k = 0; k < kProbeIters; k++)
-      st4_stream(a + (g0 + k * kWave) * 4, make_float4(x[k].x + y[k].x, x[k].y + y[k].y, x[k].z + y[k].z, x[k].w + y[k].w));
-  }
-}
-}  // namespace
-
 int reject_capture(hipStream_t stream, const char* who) {
   hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
   if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
@@ -411,28 +375,6 @@ HPX_API int hpx_get_option(const char* name, int64_t* value) {
   const int i = hpx::option_index(name);
   HPX_ARG(i >= 0, "hpx_get_option: unknown option '%s'", name);
   *value = hpx::g_opt[i].load();
-  return HPX_OK;
-}
-
-HPX_API int hpx_probe_stream(int kind, void* a, const void* b, int64_t bytes, hpx_stream_t stream) {
-  hpx::clear_error();
-  HPX_ARG(kind >= 0 && kind <= 3, "hpx_probe_stream: kind %d", kind);
-  HPX_ARG(a && (kind != 3 || b), "hpx_probe_stream: null pointer");
-  HPX_ARG(((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15) == 0, "hpx_probe_stream: pointers must be 16-byte aligned");
-  constexpr int64_t kTile = int64_t(hpx::kProbeThreads) * hpx::kProbeIters * 16;
-  const int64_t tiles = bytes / kTile;
-  HPX_ARG(tiles > 0 && tiles <= INT32_MAX, "hpx_probe_stream: %lld bytes", static_cast<long long>(bytes));
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  float* fa = static_cast<float*>(a);
-  const float* fb = static_cast<const float*>(b);
-  const dim3 grid(static_cast<uint32_t>(tiles)), block(hpx::kProbeThreads);
-  switch (kind) {
-    case 0: HPX_LAUNCH("probe_stream_kernel", hpx::probe_stream_kernel<0>, grid, block, st, fa, fb); break;
-    case 1: HPX_LAUNCH("probe_stream_kernel", hpx::probe_stream_kernel<1>, grid, block, st, fa, fb); break;
-    case 2: HPX_LAUNCH("probe_stream_kernel", hpx::probe_stream_kernel<2>, grid, block, st, fa, fb); break;
-    default: HPX_LAUNCH("probe_stream_kernel", hpx::probe_stream_kernel<3>, grid, block, st, fa, fb); break;
-  }
-  HPX_HIP(hipGetLastError());
   return HPX_OK;
 }
 
