@@ -322,9 +322,13 @@ def bucket_sizes(np):
     return [int(x) for x in sizes]
 
 
-# MFMA busy cycles of the PowerSGD kernels from a counter run of `bench.py --only powersgd`
-# (profiles/powersgd_mfma_busy.txt): SQ_VALU_MFMA_BUSY_CYCLES / SQ_BUSY_CYCLES per kernel, not read in this run.
-MEASURED_MFMA_BUSY = None
+# MFMA utilisation of the PowerSGD kernels from a counter run of `bench.py --only powersgd`
+# (profiles/powersgd_mfma_busy.txt): matrix-pipe busy cycles over the cycles on offer, per kernel.
+MEASURED_MFMA_BUSY = {
+    "from": "profiles/powersgd_mfma_busy.txt (rocprofv3 --pmc run of `bench.py --only powersgd`), not read in this run",
+    "busy_is": "SQ_VALU_MFMA_BUSY_CYCLES / (GRBM_GUI_ACTIVE / 8 XCDs * 1024 SIMDs)",
+    "psgd_encode1_kernel": 0.0265, "psgd_mtp_kernel": 0.0749, "psgd_decode_kernel": 0.0195,
+    "SQ_INSTS_MFMA_per_launch": 4718592, "SQ_VALU_MFMA_BUSY_CYCLES_per_launch": 37748736}
 
 
 def x_tbq(torch, np, capi, L, stream, gen, res):
