@@ -268,6 +268,38 @@ int hpx_dgc_decode(int count, const uint8_t* const* ins, const int32_t* in_sizes
                    float* const* outs, const int32_t* out_sizes,
                    const int32_t* is_add_tos, hpx_stream_t stream);
 
+/* ---- ECQ: error-compensated quantiser with a history -----------------------
+ * The reference holds this codec as a body without a driver or a caller
+ * (ecq_body / ecq_r_body, ecq_body.h:157-286 / :342-423); these two entry points
+ * are the drivers it would have.  The body keeps its |G + alpha*H| scratch at the
+ * start of the output buffer and writes the packed bytes over it, which is only
+ * well defined under its serial policy; that serial behaviour is what is
+ * reproduced, bit for bit, quirks included:
+ *   message  [0:4] int32 10 + M, [4:8] max|G + alpha*H| (fp32), [8] bitwidth,
+ *            [9] unused slots of the last byte, [10:] M = ceil(N/(8/b)) bytes of
+ *            b-bit codes LSB-first, code = uint8((|G + alpha*H| + max) / gap + u),
+ *            gap = max / (2^(b-1) - 1), u from the reference's LCG seeded with
+ *            seeds[t] + byte index (NULL: the wall clock, ecq_body.h:253-255);
+ *   history  H = beta*H + (unrounded - code) * gap;
+ *   quirks   the quantise loop covers M - 1 bytes: the LAST payload byte is not a
+ *            code byte (it holds one byte of the scratch, or stays as the caller
+ *            left it when N <= 2) and the history of its elements is not updated;
+ *            for 4- and 8-bit codes scratch elements 2 (and 3) are read after a
+ *            payload byte has been stored into them; codes come out of an absolute
+ *            value, so decoded values are >= 0 (the sign is lost); max < 1e-6
+ *            gives zero bytes and H *= beta.
+ * outs[t] needs 10 + M bytes (the reference needs 4*N for its scratch).
+ * bitwidths must be 2, 4 or 8 (-1 otherwise; the reference aborts).
+ * Encode only enqueues work; decode reads every header first (one wait on the
+ * stream, as the reference copies the header to the host) and returns -1 if an
+ * output is smaller than its message's element count (the reference aborts).
+ * out[x] = code*gap - max, added to the existing value when is_add_tos[t] != 0. */
+int hpx_ecq_encode(int count, const float* const* Gs, const int32_t* Ns, float* const* Hs, uint8_t* const* outs,
+                   const int32_t* out_sizes, const double* alphas, const double* betas, const int32_t* bitwidths,
+                   const uint64_t* seeds, hpx_stream_t stream);
+int hpx_ecq_decode(int count, const uint8_t* const* ins, const int32_t* in_sizes, float* const* outs,
+                   const int32_t* out_sizes, const int32_t* is_add_tos, hpx_stream_t stream);
+
 /* ---- PowerSGD: rank-r factorisation with error feedback ------------------- */
 /* The reference bodies operate on torch tensors (powersgd_body.h); here every
  * matrix is a row-major fp32 device array: M is n x m, Q is m x r, P is n x r,

@@ -48,6 +48,8 @@ def lib():
         L.orc_gd_decode.argtypes = [u8p, C.c_int32, f32p, C.c_int32, C.c_int]
         L.orc_dgc_encode.argtypes = [f32p, C.c_int32, u8p, C.c_double, C.c_double, C.c_uint64, i32p]
         L.orc_dgc_decode.argtypes = [u8p, C.c_int32, f32p, C.c_int]
+        L.orc_ecq_encode.argtypes = [f32p, C.c_int32, f32p, u8p, C.c_double, C.c_double, C.c_int32, C.c_uint64, i32p]
+        L.orc_ecq_decode.argtypes = [u8p, f32p, C.c_int32, C.c_int]
         L.orc_max_threads.restype = C.c_int
         L.orc_set_threads.argtypes = [C.c_int]
         L.orc_set_threads.restype = None
@@ -186,3 +188,29 @@ def dgc_encode(g, sample_rate, s_percent, seed=0):
 
 def dgc_decode(msg, out, is_add_to=0, in_size=None):
     return lib().orc_dgc_decode(_u8(msg), msg.size if in_size is None else in_size, _f32(out), int(is_add_to))
+
+
+# ---- ECQ (ecq_body.h), the reference's serial-policy behaviour ------------------
+def ecq_packed_size(n, bitwidth):
+    dpb = 8 // bitwidth
+    return 10 + (n + dpb - 1) // dpb
+
+
+def ecq_encode(g, h, alpha, beta, bitwidth, seed=0):
+    """Returns (rc, message of 10 + M bytes, last_byte_defined).  `h` (the history) is updated in place.
+    When last_byte_defined is False the last payload byte is not part of the result (the reference leaves
+    whatever the caller's buffer held there)."""
+    n = g.size
+    if bitwidth not in (2, 4, 8):
+        work = np.zeros(16, np.uint8)
+        defined = C.c_int32()
+        return lib().orc_ecq_encode(_f32(g), n, _f32(h), _u8(work), alpha, beta, bitwidth, seed, C.byref(defined)), None, False
+    m = ecq_packed_size(n, bitwidth)
+    work = np.zeros(max(4 * n, m) + 16, np.uint8)
+    defined = C.c_int32()
+    rc = lib().orc_ecq_encode(_f32(g), n, _f32(h), _u8(work), alpha, beta, bitwidth, seed, C.byref(defined))
+    return rc, work[:m].copy(), bool(defined.value)
+
+
+def ecq_decode(msg, out, is_add_to=0):
+    return lib().orc_ecq_decode(_u8(msg), _f32(out), out.size, int(is_add_to))

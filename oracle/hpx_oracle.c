@@ -533,3 +533,109 @@ ORC_API void orc_set_threads(int n) {
     (void)n;
 #endif
 }
+
+/* ------------------------------------------------------------------ ECQ -- */
+/* ecq_body, ecq_body.h:157-286, as the reference's SERIAL policy (thrust::host)
+ * executes it, literally: the |G + alpha*H| scratch `GH` is a float view of the
+ * output buffer from byte 0 (:180), the packed bytes are written into the same
+ * buffer from byte 10 (:171) while later elements are still to be read, and the
+ * quantise loop covers M - 1 bytes only (:222, :240).  Under the serial order
+ * this is deterministic, and it is what this function reproduces:
+ *   - GH[x] = float(fabs(double(G[x]) + alpha * double(H[x])))            (:58)
+ *   - max_GH = the largest GH (:191-203); out_true_size = 10 + M
+ *   - max_GH < 1e-6: bytes 0 .. M-2 of the payload are 0 and H *= beta     (:207-226)
+ *   - else gap = max_GH / s with s = 2^(b-1) - 1, gap_inverse = float(1.0 / gap);
+ *     byte x < M - 1: srand(seed + x); per element f = (GH[j] + max_GH) * gap_inverse,
+ *     t = uint8(f + draw), q |= t << (b * slot), H[j] = float(beta * H[j] + (f - t) * gap)
+ *     (:105-131); a byte written at 10 + x lands in GH[(10 + x) / 4]: for 4- and
+ *     8-bit codes that element (index 2, for 8 bits also 3) has not been read yet
+ *     and is read with the overwritten byte(s)
+ *   - the LAST payload byte is never written by the loop: it keeps what the scratch
+ *     left there, byte (9 + M) % 4 of GH[(9 + M) / 4], provided that element exists
+ *     (9 + M < 4 N); otherwise it is whatever the caller's buffer held.  The history
+ *     of the last byte's elements is left as it was.
+ *   - header: int32 10 + M, float max_GH, bitwidth, unused slots of the last byte (:262-272)
+ * `work` must hold max(4 N, 10 + M) bytes; it is the reference's out_uint8_t.
+ * Returns -1 for a bitwidth other than 2, 4, 8 (the reference aborts there, :172-175).
+ * *last_byte_defined tells whether the last payload byte is part of the result.
+ * PARITY UNPINNED against a build of the reference (its CHECK_EQ needs glog, and
+ * the body has neither driver nor caller); pinned by a hand-derived message and by
+ * an independent byte-buffer model in the tests. */
+/* static_cast<uint8_t>(float) as the reference's x86-64 build performs it: a truncating conversion to int32
+ * (cvttss2si: NaN and values outside int32 give 0x80000000) of which the low byte is kept.  For values in
+ * [0, 256) this is the C++ conversion; outside it C++ leaves the result undefined, and the reference does get
+ * there: with 4- and 8-bit codes scratch elements 2 and 3 are read back with payload bytes stored into them. */
+static inline uint8_t u8_of_float_x86(float v) {
+    int32_t i = (v >= -2147483648.0f && v < 2147483648.0f) ? (int32_t)v : INT32_MIN;
+    return (uint8_t)((uint32_t)i & 0xFFu);
+}
+
+ORC_API int orc_ecq_encode(const float *G, int32_t N, float *H, uint8_t *work, double alpha, double beta,
+                           int32_t bitwidth, uint64_t seed, int32_t *last_byte_defined) {
+    if (bitwidth != 2 && bitwidth != 4 && bitwidth != 8) return -1;
+    uint8_t *Q = work + 10;
+    uint8_t s = (uint8_t)((1 << (bitwidth - 1)) - 1);
+    uint8_t dpb = (uint8_t)(8 / bitwidth);
+    int32_t M = (int32_t)ceil(N * 1.0 / dpb);
+    float *GH = (float *)work;
+    for (int32_t x = 0; x < N; x++) GH[x] = (float)fabs((double)G[x] + alpha * (double)H[x]);
+    float max_GH = GH[0];
+    for (int32_t x = 1; x < N; x++)
+        if (GH[x] > max_GH) max_GH = GH[x];
+    int32_t out_true_size = 4 + 4 + 1 + 1 + M;
+    if (max_GH < 1e-6) {
+        for (int32_t x = 0; x < M - 1; x++) Q[x] = 0;
+        for (int32_t x = 0; x < N; x++) H[x] = (float)((double)H[x] * beta);
+    } else {
+        float gap = max_GH / s;
+        float gap_inverse = (float)(1.0 / (double)gap);
+        for (int32_t x = 0; x < M - 1; x++) {
+            uint8_t q = 0;
+            int32_t head = x * dpb, tail = head + dpb;
+            uint32_t st;
+            lcg_srand(&st, (uint32_t)(seed + (uint64_t)x));
+            for (int32_t j = head; j < tail; j++) {
+                float f = (GH[j] + max_GH) * gap_inverse;
+                uint8_t t = u8_of_float_x86(f + lcg_real01(&st));
+                q = (uint8_t)(q | (t << (bitwidth * (j - head))));
+                H[j] = (float)(beta * (double)H[j] + (double)((f - t) * gap));
+            }
+            Q[x] = q;
+        }
+    }
+    *last_byte_defined = (int64_t)9 + M < (int64_t)4 * N;
+    uint8_t header[10];
+    memcpy(header, &out_true_size, 4);
+    memcpy(header + 4, &max_GH, 4);
+    header[8] = (uint8_t)bitwidth;
+    header[9] = (uint8_t)(M * dpb - N);
+    memcpy(work, header, 10);
+    return 0;
+}
+
+/* ecq_r_body, ecq_body.h:342-423 for ONE message: M = header size - 10,
+ * N = M * dpb - unused, gap = max / s, out[x] = code * gap - max (write, :302) or
+ * out[x] += code * gap - max (add, :332).  -1 if the output is smaller than N (the
+ * reference aborts there, :386-390) or the width byte is not 2, 4 or 8. */
+ORC_API int orc_ecq_decode(const uint8_t *in, float *out, int32_t out_size, int is_add_to) {
+    int32_t in_size_used;
+    float max_abs_G;
+    memcpy(&in_size_used, in, 4);
+    memcpy(&max_abs_G, in + 4, 4);
+    uint8_t bitwidth = in[8], unused = in[9];
+    if (bitwidth != 2 && bitwidth != 4 && bitwidth != 8) return -1;
+    const uint8_t *Q = in + 10;
+    int32_t M = in_size_used - 10;
+    uint8_t dpb = (uint8_t)(8 / bitwidth);
+    int32_t N = M * dpb - unused;
+    uint8_t s = (uint8_t)((1 << (bitwidth - 1)) - 1);
+    float gap = max_abs_G / s;
+    if (out_size < N) return -1;
+    uint8_t mask = (uint8_t)((1 << bitwidth) - 1);
+    for (int32_t x = 0; x < N; x++) {
+        uint8_t qval = (uint8_t)((Q[x / dpb] >> ((x % dpb) * bitwidth)) & mask);
+        if (is_add_to) out[x] += qval * gap - max_abs_G;
+        else out[x] = qval * gap - max_abs_G;
+    }
+    return 0;
+}

@@ -32,6 +32,8 @@ SYMBOLS = (
     "hpx_gd_decode",
     "hpx_dgc_encode",
     "hpx_dgc_decode",
+    "hpx_ecq_encode",
+    "hpx_ecq_decode",
     "hpx_powersgd_encode1",
     "hpx_powersgd_encode2",
     "hpx_powersgd_decode",
@@ -103,6 +105,8 @@ def load():
     L.hpx_gd_decode.argtypes = [i32, pp, p, pp, p, p, p]
     L.hpx_dgc_encode.argtypes = [i32, pp, p, pp, p, p, p, p]
     L.hpx_dgc_decode.argtypes = [i32, pp, p, pp, p, p, p]
+    L.hpx_ecq_encode.argtypes = [i32, pp, p, pp, pp, p, p, p, p, p, p]
+    L.hpx_ecq_decode.argtypes = [i32, pp, p, pp, p, p, p]
     L.hpx_powersgd_encode1.argtypes = [i32, pp, p, pp, pp, pp, pp, p, p, p, p]
     L.hpx_powersgd_encode2.argtypes = [i32, pp, pp, pp, p, p, p, p]
     L.hpx_powersgd_decode.argtypes = [i32, pp, pp, pp, pp, pp, p, p, p, p, p]
