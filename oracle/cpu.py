@@ -50,6 +50,8 @@ def lib():
         L.orc_dgc_decode.argtypes = [u8p, C.c_int32, f32p, C.c_int]
         L.orc_ecq_encode.argtypes = [f32p, C.c_int32, f32p, u8p, C.c_double, C.c_double, C.c_int32, C.c_uint64, i32p]
         L.orc_ecq_decode.argtypes = [u8p, f32p, C.c_int32, C.c_int]
+        L.orc_set_fused_multiply_add.argtypes = [C.c_int]
+        L.orc_set_fused_multiply_add.restype = None
         L.orc_max_threads.restype = C.c_int
         L.orc_set_threads.argtypes = [C.c_int]
         L.orc_set_threads.restype = None
@@ -65,6 +67,12 @@ def _f32(a):
 def _u8(a):
     assert a.dtype == np.uint8 and a.flags.c_contiguous
     return a.ctypes.data_as(C.POINTER(C.c_uint8))
+
+
+def set_fused_multiply_add(on):
+    """Lets the TernGrad oracle fuse `(x - min) * gi + u` and `q * gap + min` as a CUDA build of the reference
+    may (for measuring that difference only; parity is held to the unfused CPU arithmetic)."""
+    lib().orc_set_fused_multiply_add(int(bool(on)))
 
 
 def set_threads(n):

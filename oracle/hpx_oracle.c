@@ -221,6 +221,14 @@ static void first_minmax(const float *x, int32_t n, float *mn, float *mx) {
     *mx = x[imax];
 }
 
+/* The reference's CPU build rounds the multiply and the add of `(x - min) * gap_inverse + u`
+ * (terngrad_body.h:92-93) and of `qval * gap + min` (:127, :158) separately, and that is what parity is
+ * held to.  A CUDA build of the same source (nvcc contracts to FMA by default) may fuse them.  With this
+ * switch on, the oracle fuses exactly those two expressions, so that the size of that difference can be
+ * measured on the CPU (tests/test_oracle_tbq_terngrad.py); nothing else uses it. */
+static int g_fuse_multiply_add = 0;
+ORC_API void orc_set_fused_multiply_add(int on) { g_fuse_multiply_add = on != 0; }
+
 /* terngrad_body, terngrad_body.h:162-307 for ONE tensor.
  *   header  :219-224   [0]=bitwidth [1]=tail [2:6]=min [6:10]=max
  *   scalars :204-206   gap (fp32), gap_inverse = float(1./(double(gap)+1e-8))
@@ -257,8 +265,9 @@ ORC_API int orc_terngrad_encode(const float *x, int32_t n, uint8_t *out,
             uint32_t st;
             lcg_srand(&st, (uint32_t)(seed + (uint64_t)(int64_t)i));
             for (int j = 0; j < dpb; j++) {
-                float th = (x[((int64_t)i << dlg2) + j] - mn) * gi;
-                th += lcg_real01(&st);
+                float d = x[((int64_t)i << dlg2) + j] - mn;
+                float u = lcg_real01(&st);
+                float th = g_fuse_multiply_add ? fmaf(d, gi, u) : d * gi + u;
                 uint8_t t = (uint8_t)(int32_t)th;
                 q |= (uint8_t)(t << (bitwidth * j));
             }
@@ -309,8 +318,8 @@ ORC_API int orc_terngrad_decode(float *out, const uint8_t *in, int32_t in_size,
     for (int32_t i = 0; i < cnt; i++) {
         uint8_t off = i & ((1 << dlg2) - 1);
         uint8_t q = (in[(i >> dlg2) + 10] >> (off * bitwidth)) & mask;
-        float prod = q * gap;
-        out[i] = is_add_to ? (float)(prod + mn + out[i]) : (float)(prod + mn);
+        float v = g_fuse_multiply_add ? fmaf((float)q, gap, mn) : q * gap + mn;
+        out[i] = is_add_to ? (float)(v + out[i]) : v;
     }
     return 0;
 }
