@@ -29,6 +29,7 @@
 //     a zero extreme; it is recovered from the first zero of the tensor.
 #include <cstdlib>
 #include <mutex>
+#include <type_traits>
 #include <unordered_map>
 #include <vector>
 
@@ -140,6 +141,31 @@ __device__ __forceinline__ void acc3(float v, float& mn, float& mx, float& am) {
   am = a < am ? a : am;
 }
 
+// Three-operand minimum / maximum: one instruction for two elements, where the comparison-and-select
+// form above costs the compiler three issue slots per element (compare, a wait for the condition, select).
+// A NaN operand is ignored, as the comparisons ignore it; which zero wins among +0 and -0 does not matter,
+// because the sign of a zero extreme is settled from the first zero of the tensor.
+__device__ __forceinline__ float vmin3(float a, float b, float c) {
+  float r;
+  __asm__("v_min3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+__device__ __forceinline__ float vmax3(float a, float b, float c) {
+  float r;
+  __asm__("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+__device__ __forceinline__ float vmin3_abs(float a, float b, float c) {  // min(a, |b|, |c|)
+  float r;
+  __asm__("v_min3_f32 %0, %1, |%2|, |%3|" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+// min, max and min |x| over four elements: six instructions.
+__device__ __forceinline__ void acc3x4(const float4& v, float& mn, float& mx, float& am) {
+  mn = vmin3(mn, v.x, v.y); mx = vmax3(mx, v.x, v.y); am = vmin3_abs(am, v.x, v.y);
+  mn = vmin3(mn, v.z, v.w); mx = vmax3(mx, v.z, v.w); am = vmin3_abs(am, v.z, v.w);
+}
+
 // Order-preserving map of a float onto unsigned integers, and back.
 __device__ __forceinline__ uint32_t okey(float f) {
   const uint32_t b = __float_as_uint(f);
@@ -176,10 +202,7 @@ __global__ __launch_bounds__(kThreads) void terngrad_minmax_kernel(const EncArgs
 #pragma unroll
     for (int k = 0; k < kRedIters; k++) v[k] = ld4(xp + size_t(e0) + size_t(k * kThreads + threadIdx.x) * 4);
 #pragma unroll
-    for (int k = 0; k < kRedIters; k++) {
-      acc3(v[k].x, mn, mx, am); acc3(v[k].y, mn, mx, am);
-      acc3(v[k].z, mn, mx, am); acc3(v[k].w, mn, mx, am);
-    }
+    for (int k = 0; k < kRedIters; k++) acc3x4(v[k], mn, mx, am);
   } else {
     for (uint32_t e = e0 + threadIdx.x; e < n; e += kThreads) acc3(xp[e], mn, mx, am);
   }
@@ -437,7 +460,9 @@ constexpr int kResLdsGroups = 8;   // float4 per lane of the tensor held in LDS 
 constexpr int kResLdsTotalGroups = 9;  // ... and what the workgroup may use altogether (144 KiB): the rest holds prepared draws
 struct ResArgs {
   EncSeg seg;
-  uint32_t chunk_units;  // units per workgroup, a multiple of kResThreads
+  uint32_t chunk_units;  // units per workgroup, a multiple of kWave
+  uint32_t reg_rows;     // rows of 64 units a wave holds in registers: all the kernel has room for when the share
+                         // fills them, otherwise just enough of them, so that a smaller share still spreads over all waves
   uint32_t lds_rows;     // rows of kResThreads units kept in LDS
   uint32_t pre_rows;     // register rows whose random addends are prepared during pass 1: 0 or res_pre_rows(bits)
   uint32_t gen;          // generation of this launch, counted from 1: the tag of its records
@@ -502,76 +527,91 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
   // input per wave: measurably faster than rows spread over the workgroup's
   // share); the LDS rows follow all register rows.
   constexpr uint32_t rs = kWave;
-  const uint32_t u0 = wg_u0 + (threadIdx.x / kWave) * (KU * kWave) + (threadIdx.x & (kWave - 1));
+  const uint32_t R = a.reg_rows;  // KU whenever there are LDS rows
+  const uint32_t u0 = wg_u0 + (threadIdx.x / kWave) * (R * kWave) + (threadIdx.x & (kWave - 1));
   const uint32_t l0 = wg_u0 + KU * kResThreads + threadIdx.x;
   constexpr uint32_t stride_bytes = rs * BPU;
   const float qnan = __builtin_nanf("");  // compares false both ways: ignored by min and max
 
   // ---- pass 1: load the share, reduce ------------------------------------------
+  // All loads of the lane are requested at once: the first LDS row, then its register rows.  While
+  // they are in flight and the ALUs idle, the random addends of the first PRE register rows, which
+  // depend on position and seed only, go into the LDS the tensor does not need; pass 2 (ALU-bound:
+  // nothing left to overlap with) then skips 6 of its 11 operations per element for those rows.
+  // Then each register row is reduced as it arrives (min, max and min |x| of every element; the
+  // index of the first zero is only worked out by lanes that met one), so that only the last
+  // rows' work is left when the last byte has landed.  This is one straight block per case - a
+  // workgroup whose register rows are all whole, and the others - because behind a join of the
+  // two the compiler no longer knows the order of the loads and waits for all of them at once.
   float4 v[KU][H];
-  if (wg_u0 + uint32_t(KU * kResThreads) <= wg_end) {
+  float4 t0[H];
+  float4* s_pre = s_rows + size_t(a.lds_rows) * H * kResThreads;
+  float mn = __builtin_inff(), mx = -__builtin_inff(), am = __builtin_inff();
+  const bool whole_rows = wg_u0 + uint32_t(KU * kResThreads) <= wg_end;
+  auto pass1 = [&](auto whole) {
+    if (a.lds_rows > 0) {
 #pragma unroll
-    for (int k = 0; k < KU; k++)
-#pragma unroll
-      for (int h = 0; h < H; h++) v[k][h] = ld4_stream(xp + size_t(u0 + k * rs) * UNIT + h * 4);
-  } else {
+      for (int h = 0; h < H; h++)
+        t0[h] = l0 < wg_end ? ld4_stream(xp + size_t(l0) * UNIT + h * 4) : make_float4(qnan, qnan, qnan, qnan);
+    }
 #pragma unroll
     for (int k = 0; k < KU; k++) {
       const uint32_t u = u0 + k * rs;
 #pragma unroll
       for (int h = 0; h < H; h++)
-        v[k][h] = u < wg_end ? ld4_stream(xp + size_t(u) * UNIT + h * 4) : make_float4(qnan, qnan, qnan, qnan);
+        v[k][h] = (decltype(whole)::value || (uint32_t(k) < R && u < wg_end)) ? ld4_stream(xp + size_t(u) * UNIT + h * 4)
+                                                         : make_float4(qnan, qnan, qnan, qnan);
     }
-  }
-  // While the loads are in flight and the ALUs idle: the random addends of the first pre_rows
-  // register rows, which depend on position and seed only, go into the LDS the tensor does not
-  // need; pass 2 (ALU-bound: nothing left to overlap with) then skips 6 of its 11 operations
-  // per element for those rows.
-  float4* s_pre = s_rows + size_t(a.lds_rows) * H * kResThreads;
-  if (RANDOM && PRE > 0) {
-    uint32_t d[UNIT];
-    const uint32_t x0 = a.seg.seed + u0 * BPU;
+    if (RANDOM && PRE > 0) {
+      uint32_t d[UNIT];
+      const uint32_t x0 = a.seg.seed + u0 * BPU;
 #pragma unroll
-    for (int q = 0; q < UNIT; q++) {
-      const int jb = q / DPB, j = q % DPB;
-      d[q] = lcg_mul(j + 2) * (x0 + jb) + lcg_add(j + 2);
+      for (int q = 0; q < UNIT; q++) {
+        const int jb = q / DPB, j = q % DPB;
+        d[q] = lcg_mul(j + 2) * (x0 + jb) + lcg_add(j + 2);
+      }
+      for (uint32_t k = 0; k < uint32_t(PRE); k++) {
+#pragma unroll
+        for (int h = 0; h < H; h++)
+          s_pre[(k * H + h) * kResThreads + threadIdx.x] =
+              make_float4(u01_scaled(d[4 * h]), u01_scaled(d[4 * h + 1]), u01_scaled(d[4 * h + 2]), u01_scaled(d[4 * h + 3]));
+#pragma unroll
+        for (int q = 0; q < UNIT; q++) d[q] += lcg_mul(q % DPB + 2) * stride_bytes;
+      }
     }
-    for (uint32_t k = 0; k < uint32_t(PRE); k++) {
+    if (a.lds_rows > 0) {
 #pragma unroll
-      for (int h = 0; h < H; h++)
-        s_pre[(k * H + h) * kResThreads + threadIdx.x] =
-            make_float4(u01_scaled(d[4 * h]), u01_scaled(d[4 * h + 1]), u01_scaled(d[4 * h + 2]), u01_scaled(d[4 * h + 3]));
-#pragma unroll
-      for (int q = 0; q < UNIT; q++) d[q] += lcg_mul(q % DPB + 2) * stride_bytes;
+      for (int h = 0; h < H; h++) {
+        s_rows[h * kResThreads + threadIdx.x] = t0[h];
+        acc3x4(t0[h], mn, mx, am);
+      }
     }
-  }
-  float mn = __builtin_inff(), mx = -__builtin_inff();
-  uint32_t fz = 0xFFFFFFFFu;
-  for (uint32_t r = 0; r < a.lds_rows; r++) {
+#pragma unroll
+    for (int k = 0; k < KU; k++)
+#pragma unroll
+      for (int h = 0; h < H; h++) acc3x4(v[k][h], mn, mx, am);
+  };
+  if (whole_rows) pass1(std::true_type{}); else pass1(std::false_type{});
+  for (uint32_t r = 1; r < a.lds_rows; r++) {
     const uint32_t u = l0 + r * kResThreads;
 #pragma unroll
     for (int h = 0; h < H; h++) {
       const float4 f = u < wg_end ? ld4_stream(xp + size_t(u) * UNIT + h * 4) : make_float4(qnan, qnan, qnan, qnan);
       s_rows[(r * H + h) * kResThreads + threadIdx.x] = f;
-      acc_zero4(f, u * UNIT + h * 4, mn, mx, fz);
+      acc3x4(f, mn, mx, am);
     }
   }
-  // Register rows: min, max and min |x| per element; the index of the first zero is
-  // only worked out by lanes that met one.
-  float am = __builtin_inff();
-#pragma unroll
-  for (int k = 0; k < KU; k++)
-#pragma unroll
-    for (int h = 0; h < H; h++) {
-      acc3(v[k][h].x, mn, mx, am); acc3(v[k][h].y, mn, mx, am);
-      acc3(v[k][h].z, mn, mx, am); acc3(v[k][h].w, mn, mx, am);
-    }
+  uint32_t fz = 0xFFFFFFFFu;
   if (am == 0.0f) {
     float d0 = 0.f, d1 = 0.f;
 #pragma unroll
     for (int k = 0; k < KU; k++)
 #pragma unroll
       for (int h = 0; h < H; h++) acc_zero4(v[k][h], (u0 + k * rs) * UNIT + h * 4, d0, d1, fz);
+    for (uint32_t r = 0; r < a.lds_rows; r++)  // this lane's own LDS rows, read back
+#pragma unroll
+      for (int h = 0; h < H; h++)
+        acc_zero4(s_rows[(r * H + h) * kResThreads + threadIdx.x], (l0 + r * kResThreads) * UNIT + h * 4, d0, d1, fz);
   }
   if (blockIdx.x == 0 && threadIdx.x == 0)
     for (uint32_t e = full_units * UNIT; e < n; e++) acc_zero(xp[e], e, mn, mx, fz);
@@ -634,23 +674,28 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
       draw[q] = lcg_mul(j + 2) * (x0 + jb) + lcg_add(j + 2);
     }
   }
+  // A workgroup whose register rows are all whole (every one but the last with a share) stores
+  // without a bounds check per row: the checks cost a branch each.
+  auto register_rows = [&](auto whole) {
 #pragma unroll
-  for (int k = 0; k < KU; k++) {
-    const uint32_t u = u0 + k * rs;
-    uint32_t packed;
-    if (RANDOM && k < PRE) {
-      float4 sc[H];
+    for (int k = 0; k < KU; k++) {
+      const uint32_t u = u0 + k * rs;
+      uint32_t packed;
+      if (RANDOM && k < PRE) {
+        float4 sc[H];
 #pragma unroll
-      for (int h = 0; h < H; h++) sc[h] = s_pre[(k * H + h) * kResThreads + threadIdx.x];
-      packed = quant_unit_prepared<B>(v[k], sc, mn, gi);
-    } else {
-      packed = quant_unit<B, RANDOM>(v[k], mn, gi, draw, stride_bytes);
+        for (int h = 0; h < H; h++) sc[h] = s_pre[(k * H + h) * kResThreads + threadIdx.x];
+        packed = quant_unit_prepared<B>(v[k], sc, mn, gi);
+      } else {
+        packed = quant_unit<B, RANDOM>(v[k], mn, gi, draw, stride_bytes);
+      }
+      if (decltype(whole)::value || (uint32_t(k) < R && u < wg_end)) {
+#pragma unroll
+        for (int jb = 0; jb < BPU; jb++) pay[size_t(u) * BPU + jb] = uint8_t(packed >> (8 * jb));
+      }
     }
-    if (u < wg_end) {
-#pragma unroll
-      for (int jb = 0; jb < BPU; jb++) pay[size_t(u) * BPU + jb] = uint8_t(packed >> (8 * jb));
-    }
-  }
+  };
+  if (whole_rows) register_rows(std::true_type{}); else register_rows(std::false_type{});
   if (RANDOM) {
     uint32_t x0 = a.seg.seed + l0 * BPU;
     // Keeps the compiler from preparing these draws before the register rows are
@@ -1418,7 +1463,10 @@ bool resident_plan(int32_t n, int bits, bool random, const hpx::Workspace* ws, R
   if (rows < 1) rows = 1;
   const int reg_rows = res_reg_groups(bits, random) / h, lds_rows_max = kResLdsGroups / h;
   if (rows > reg_rows + lds_rows_max) return false;
-  ra.chunk_units = static_cast<uint32_t>(rows * kResThreads);
+  // The share itself is only rounded up to whole waves' worth of units, so that every CU has one (rounded to
+  // whole rows, the headline tensor's 24.4 rows per workgroup became 25 rows for 250 workgroups and none for six).
+  ra.chunk_units = static_cast<uint32_t>((per_wg + kWave - 1) / kWave * kWave);
+  ra.reg_rows = static_cast<uint32_t>(rows < reg_rows ? rows : reg_rows);
   ra.lds_rows = rows > reg_rows ? static_cast<uint32_t>(rows - reg_rows) : 0u;
   const int spare_rows = (kResLdsTotalGroups - int(ra.lds_rows) * h) / h;
   ra.pre_rows = (random && spare_rows >= res_pre_rows(bits)) ? static_cast<uint32_t>(res_pre_rows(bits)) : 0u;
