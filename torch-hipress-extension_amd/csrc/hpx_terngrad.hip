@@ -310,25 +310,38 @@ __device__ __forceinline__ uint32_t quant_one(float x, float mn, float gi, uint3
   return static_cast<uint32_t>(t) & 0xFFu;
 }
 
+// The codes of one unit as its packed bytes.  Within a byte codes are OR-ed without masking
+// (terngrad_body.h:95): a code that reaches 1<<B spills into the next slot of the SAME byte.  Shifting
+// distributes over OR, so the byte is built from its last slot down, one shift-and-or per slot.
+template <int B, int UNIT>
+__device__ __forceinline__ uint32_t pack_codes(const uint32_t (&t)[UNIT]) {
+  constexpr int DPB = 8 / B;
+  uint32_t packed = 0;
+#pragma unroll
+  for (int jb = 0; jb < UNIT / DPB; jb++) {
+    uint32_t p = t[jb * DPB + DPB - 1];
+#pragma unroll
+    for (int j = DPB - 2; j >= 0; j--) p = (p << B) | t[jb * DPB + j];
+    packed |= (UNIT / DPB > 1 ? (p & 0xFFu) : p) << (8 * jb);  // a single byte is cut by its store
+  }
+  return packed;
+}
+
 // Quantises one unit held in registers and returns its BPU packed bytes; advances
 // the lane's draws by `stride_bytes` output bytes.
 template <int B, bool RANDOM, int UNIT = (8 / B > 4 ? 8 / B : 4)>
 __device__ __forceinline__ uint32_t quant_unit(const float4 (&v)[UNIT / 4], float mn, float gi, uint32_t (&draw)[UNIT],
                                                uint32_t stride_bytes) {
   constexpr int DPB = 8 / B;
-  uint32_t packed = 0;
+  uint32_t t[UNIT];
 #pragma unroll
   for (int q = 0; q < UNIT; q++) {
     const float4 f = v[q / 4];
     const float x = (q & 3) == 0 ? f.x : (q & 3) == 1 ? f.y : (q & 3) == 2 ? f.z : f.w;
-    const uint32_t t = quant_one<B, RANDOM>(x, mn, gi, RANDOM ? draw[q] : 0u);
-    // Within a byte codes are OR-ed without masking (terngrad_body.h:95):
-    // a code that reaches 1<<B spills into the next slot of the SAME byte.
-    const int jb = q / DPB, j = q % DPB;
-    packed |= ((t << (B * j)) & 0xFFu) << (8 * jb);
-    if (RANDOM) draw[q] += lcg_mul(j + 2) * stride_bytes;
+    t[q] = quant_one<B, RANDOM>(x, mn, gi, RANDOM ? draw[q] : 0u);
+    if (RANDOM) draw[q] += lcg_mul(q % DPB + 2) * stride_bytes;
   }
-  return packed;
+  return pack_codes<B, UNIT>(t);
 }
 
 // Unit u of a tensor whose end may fall inside it: element-wise from memory.
@@ -455,6 +468,9 @@ constexpr int kResRegGroups = 24;  // float4 per lane held in registers ...
 // ... except at 1 bit with stochastic rounding, whose eight draws per lane need the room.
 // Rows of prepared random addends when the LDS has room for them (8 float4 per lane).
 constexpr int res_pre_rows(int bits) { return bits == 1 ? 4 : 8; }
+// Further rows whose addends are prepared into registers, after those that go into LDS: pass 2 takes the
+// prepared rows first and gives registers back as it goes, so a few float4 per lane are free until then.
+constexpr int res_pre_reg_rows(int bits, int pre) { return (pre > 0 && bits != 1) ? 0 : 0; }
 constexpr int res_reg_groups(int bits, bool random) { return (bits == 1 && random) ? 14 : kResRegGroups; }
 constexpr int kResLdsGroups = 8;   // float4 per lane of the tensor held in LDS (128 KiB per workgroup)
 constexpr int kResLdsTotalGroups = 9;  // ... and what the workgroup may use altogether (144 KiB): the rest holds prepared draws
@@ -485,8 +501,7 @@ __device__ __forceinline__ void acc_zero4(float4 v, uint32_t idx, float& mn, flo
 template <int B, int UNIT = (8 / B > 4 ? 8 / B : 4)>
 __device__ __forceinline__ uint32_t quant_unit_prepared(const float4 (&v)[UNIT / 4], const float4 (&s)[UNIT / 4], float mn,
                                                         float gi) {
-  constexpr int DPB = 8 / B;
-  uint32_t packed = 0;
+  uint32_t t[UNIT];
 #pragma unroll
   for (int q = 0; q < UNIT; q++) {
     const float4 f = v[q / 4], g = s[q / 4];
@@ -494,11 +509,9 @@ __device__ __forceinline__ uint32_t quant_unit_prepared(const float4 (&v)[UNIT /
     const float sc = (q & 3) == 0 ? g.x : (q & 3) == 1 ? g.y : (q & 3) == 2 ? g.z : g.w;
     float th = (x - mn) * gi;
     th = __builtin_fmaf(sc, 0x1p-32f, th);
-    const uint32_t t = static_cast<uint32_t>(static_cast<int32_t>(th)) & 0xFFu;
-    const int jb = q / DPB, j = q % DPB;
-    packed |= ((t << (B * j)) & 0xFFu) << (8 * jb);
+    t[q] = static_cast<uint32_t>(static_cast<int32_t>(th)) & 0xFFu;
   }
-  return packed;
+  return pack_codes<B, UNIT>(t);
 }
 
 // PRE: register rows whose random addends are prepared during pass 1 (a compile-time count, so that pass 2
@@ -545,6 +558,8 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
   // two the compiler no longer knows the order of the loads and waits for all of them at once.
   float4 v[KU][H];
   float4 t0[H];
+  constexpr int PREG = res_pre_reg_rows(B, PRE);
+  float4 pre_reg[PREG > 0 ? PREG : 1][H];
   float4* s_pre = s_rows + size_t(a.lds_rows) * H * kResThreads;
   float mn = __builtin_inff(), mx = -__builtin_inff(), am = __builtin_inff();
   const bool whole_rows = wg_u0 + uint32_t(KU * kResThreads) <= wg_end;
@@ -574,6 +589,15 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
 #pragma unroll
         for (int h = 0; h < H; h++)
           s_pre[(k * H + h) * kResThreads + threadIdx.x] =
+              make_float4(u01_scaled(d[4 * h]), u01_scaled(d[4 * h + 1]), u01_scaled(d[4 * h + 2]), u01_scaled(d[4 * h + 3]));
+#pragma unroll
+        for (int q = 0; q < UNIT; q++) d[q] += lcg_mul(q % DPB + 2) * stride_bytes;
+      }
+#pragma unroll
+      for (int k = 0; k < PREG; k++) {
+#pragma unroll
+        for (int h = 0; h < H; h++)
+          pre_reg[k][h] =
               make_float4(u01_scaled(d[4 * h]), u01_scaled(d[4 * h + 1]), u01_scaled(d[4 * h + 2]), u01_scaled(d[4 * h + 3]));
 #pragma unroll
         for (int q = 0; q < UNIT; q++) d[q] += lcg_mul(q % DPB + 2) * stride_bytes;
@@ -667,7 +691,7 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
   uint8_t* __restrict__ pay = a.seg.out + 10;
   uint32_t draw[UNIT];
   if (RANDOM) {
-    const uint32_t x0 = a.seg.seed + u0 * BPU + uint32_t(PRE) * stride_bytes;  // first row that draws for itself
+    const uint32_t x0 = a.seg.seed + u0 * BPU + uint32_t(PRE + PREG) * stride_bytes;  // first row that draws for itself
 #pragma unroll
     for (int q = 0; q < UNIT; q++) {
       const int jb = q / DPB, j = q % DPB;
@@ -686,6 +710,8 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
 #pragma unroll
         for (int h = 0; h < H; h++) sc[h] = s_pre[(k * H + h) * kResThreads + threadIdx.x];
         packed = quant_unit_prepared<B>(v[k], sc, mn, gi);
+      } else if (RANDOM && k < PRE + PREG) {
+        packed = quant_unit_prepared<B>(v[k], pre_reg[k - PRE < 0 ? 0 : k - PRE], mn, gi);
       } else {
         packed = quant_unit<B, RANDOM>(v[k], mn, gi, draw, stride_bytes);
       }
@@ -772,7 +798,9 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_multi_kernel(co
   extern __shared__ float4 s_rows[];  // [wave][lds_rows][H][64], then the prepared draws [wave][PRE][H][64]
   __shared__ uint32_t s_ok;
 
-  const uint32_t wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  // The wave index is the same in every lane: taken from the first lane, it and all that is derived from it
+  // (piece, tensor, bounds) live in scalar registers.
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x & (kWave - 1);
   const int total = a.piece_start[a.nseg];
   const int my_piece = int(blockIdx.x) * kWaves + int(wave);
   const bool active = my_piece < total;           // wave-uniform
@@ -794,63 +822,78 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_multi_kernel(co
   float4* s_pre = s_rows + size_t(kWaves) * a.lds_rows * H * kWave + size_t(wave) * PRE * H * kWave;
 
   // ---- pass 1: load the piece, reduce ---------------------------------------------
+  // As in the single-tensor kernel: all loads at once (the first LDS row ahead of the register rows), the
+  // random addends of the first PRE rows while they are in flight, then every row reduced as it arrives,
+  // one straight block per case.
   float4 v[KU][H];
-  if (u_beg + uint32_t(KU * kWave) <= u_end) {
+  float4 t0[H];
+  float mn = __builtin_inff(), mx = -__builtin_inff(), am = __builtin_inff();
+  const bool whole_rows = u_beg + uint32_t(KU * kWave) <= u_end;
+  const uint32_t ul0 = u0 + uint32_t(KU) * kWave;  // this lane's unit in the first LDS row
+  auto pass1 = [&](auto whole) {
+    if (a.lds_rows > 0) {
 #pragma unroll
-    for (int k = 0; k < KU; k++)
-#pragma unroll
-      for (int h = 0; h < H; h++) v[k][h] = ld4_stream(xp + size_t(u0 + k * kWave) * UNIT + h * 4);
-  } else {
+      for (int h = 0; h < H; h++)
+        t0[h] = ul0 < u_end ? ld4_stream(xp + size_t(ul0) * UNIT + h * 4) : make_float4(qnan, qnan, qnan, qnan);
+    }
 #pragma unroll
     for (int k = 0; k < KU; k++) {
       const uint32_t u = u0 + k * kWave;
 #pragma unroll
       for (int h = 0; h < H; h++)
-        v[k][h] = u < u_end ? ld4_stream(xp + size_t(u) * UNIT + h * 4) : make_float4(qnan, qnan, qnan, qnan);
+        v[k][h] = (decltype(whole)::value || u < u_end) ? ld4_stream(xp + size_t(u) * UNIT + h * 4)
+                                                        : make_float4(qnan, qnan, qnan, qnan);
     }
-  }
-  if (RANDOM && PRE > 0) {  // random addends of the first PRE rows, while the loads are in flight
-    uint32_t d[UNIT];
-    const uint32_t x0 = sg.seed + u0 * BPU;
+    if (RANDOM && PRE > 0) {
+      uint32_t d[UNIT];
+      const uint32_t x0 = sg.seed + u0 * BPU;
 #pragma unroll
-    for (int q = 0; q < UNIT; q++) {
-      const int jb = q / DPB, j = q % DPB;
-      d[q] = lcg_mul(j + 2) * (x0 + jb) + lcg_add(j + 2);
+      for (int q = 0; q < UNIT; q++) {
+        const int jb = q / DPB, j = q % DPB;
+        d[q] = lcg_mul(j + 2) * (x0 + jb) + lcg_add(j + 2);
+      }
+      for (uint32_t k = 0; k < uint32_t(PRE); k++) {
+#pragma unroll
+        for (int h = 0; h < H; h++)
+          s_pre[(k * H + h) * kWave + lane] =
+              make_float4(u01_scaled(d[4 * h]), u01_scaled(d[4 * h + 1]), u01_scaled(d[4 * h + 2]), u01_scaled(d[4 * h + 3]));
+#pragma unroll
+        for (int q = 0; q < UNIT; q++) d[q] += lcg_mul(q % DPB + 2) * stride_bytes;
+      }
     }
-    for (uint32_t k = 0; k < uint32_t(PRE); k++) {
+    if (a.lds_rows > 0) {
 #pragma unroll
-      for (int h = 0; h < H; h++)
-        s_pre[(k * H + h) * kWave + lane] =
-            make_float4(u01_scaled(d[4 * h]), u01_scaled(d[4 * h + 1]), u01_scaled(d[4 * h + 2]), u01_scaled(d[4 * h + 3]));
-#pragma unroll
-      for (int q = 0; q < UNIT; q++) d[q] += lcg_mul(q % DPB + 2) * stride_bytes;
+      for (int h = 0; h < H; h++) {
+        s_mine[h * kWave + lane] = t0[h];
+        acc3x4(t0[h], mn, mx, am);
+      }
     }
-  }
-  float mn = __builtin_inff(), mx = -__builtin_inff();
-  uint32_t fz = 0xFFFFFFFFu;
-  for (uint32_t r = 0; r < a.lds_rows; r++) {
-    const uint32_t u = u0 + (uint32_t(KU) + r) * kWave;
+#pragma unroll
+    for (int k = 0; k < KU; k++)
+#pragma unroll
+      for (int h = 0; h < H; h++) acc3x4(v[k][h], mn, mx, am);
+  };
+  if (whole_rows) pass1(std::true_type{}); else pass1(std::false_type{});
+  for (uint32_t r = 1; r < a.lds_rows; r++) {
+    const uint32_t u = ul0 + r * kWave;
 #pragma unroll
     for (int h = 0; h < H; h++) {
       const float4 f = u < u_end ? ld4_stream(xp + size_t(u) * UNIT + h * 4) : make_float4(qnan, qnan, qnan, qnan);
       s_mine[(r * H + h) * kWave + lane] = f;
-      acc_zero4(f, u * UNIT + h * 4, mn, mx, fz);
+      acc3x4(f, mn, mx, am);
     }
   }
-  float am = __builtin_inff();
-#pragma unroll
-  for (int k = 0; k < KU; k++)
-#pragma unroll
-    for (int h = 0; h < H; h++) {
-      acc3(v[k][h].x, mn, mx, am); acc3(v[k][h].y, mn, mx, am);
-      acc3(v[k][h].z, mn, mx, am); acc3(v[k][h].w, mn, mx, am);
-    }
+  uint32_t fz = 0xFFFFFFFFu;
   if (am == 0.0f) {
     float d0 = 0.f, d1 = 0.f;
 #pragma unroll
     for (int k = 0; k < KU; k++)
 #pragma unroll
       for (int h = 0; h < H; h++) acc_zero4(v[k][h], (u0 + k * kWave) * UNIT + h * 4, d0, d1, fz);
+    for (uint32_t r = 0; r < a.lds_rows; r++)  // this lane's own LDS rows, read back
+#pragma unroll
+      for (int h = 0; h < H; h++)
+        acc_zero4(s_mine[(r * H + h) * kWave + lane], (ul0 + r * kWave) * UNIT + h * 4, d0, d1, fz);
   }
   if (ends_tensor && lane == 0)
     for (uint32_t e = full_units * UNIT; e < n; e++) acc_zero(xp[e], e, mn, mx, fz);
@@ -921,23 +964,26 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_multi_kernel(co
       draw[q] = lcg_mul(j + 2) * (x0 + jb) + lcg_add(j + 2);
     }
   }
+  auto register_rows = [&](auto whole) {
 #pragma unroll
-  for (int k = 0; k < KU; k++) {
-    const uint32_t u = u0 + k * kWave;
-    uint32_t packed;
-    if (RANDOM && k < PRE) {
-      float4 sc[H];
+    for (int k = 0; k < KU; k++) {
+      const uint32_t u = u0 + k * kWave;
+      uint32_t packed;
+      if (RANDOM && k < PRE) {
+        float4 sc[H];
 #pragma unroll
-      for (int h = 0; h < H; h++) sc[h] = s_pre[(k * H + h) * kWave + lane];
-      packed = quant_unit_prepared<B>(v[k], sc, mn, gi);
-    } else {
-      packed = quant_unit<B, RANDOM>(v[k], mn, gi, draw, stride_bytes);
+        for (int h = 0; h < H; h++) sc[h] = s_pre[(k * H + h) * kWave + lane];
+        packed = quant_unit_prepared<B>(v[k], sc, mn, gi);
+      } else {
+        packed = quant_unit<B, RANDOM>(v[k], mn, gi, draw, stride_bytes);
+      }
+      if (decltype(whole)::value || u < u_end) {
+#pragma unroll
+        for (int jb = 0; jb < BPU; jb++) pay[size_t(u) * BPU + jb] = uint8_t(packed >> (8 * jb));
+      }
     }
-    if (u < u_end) {
-#pragma unroll
-      for (int jb = 0; jb < BPU; jb++) pay[size_t(u) * BPU + jb] = uint8_t(packed >> (8 * jb));
-    }
-  }
+  };
+  if (whole_rows) register_rows(std::true_type{}); else register_rows(std::false_type{});
   // The LDS rows follow the register rows of the same wave, so the draws simply go on.
   for (uint32_t r = 0; r < a.lds_rows; r++) {
     const uint32_t u = u0 + (uint32_t(KU) + r) * kWave;
