@@ -316,6 +316,20 @@ def test_resident_capacity_edge(tg, oracle_cpu, b, n):
     assert_bits_equal(host(out), ref, f"message n={n} b={b}")
 
 
+@pytest.mark.parametrize("b,rnd,n", [(2, 1, 7_000_003), (2, 1, 13_631_489), (4, 0, 17_111_111), (2, 1, 24_000_001), (8, 1, 25_165_823),
+                                     (2, 1, 25_165_824), (2, 0, 25_231_361)])
+def test_resident_shares_between_one_row_and_the_register_rows(tg, oracle_cpu, resident_forced, b, rnd, n):
+    # shares of 7 ... 24 rows per workgroup, not whole rows, and one that ends a few units into the first LDS row:
+    # every wave holds a part of the share, the last waves a ragged one
+    rng = np.random.default_rng(n % 1000 + b)
+    x = rng.normal(0, 1e-2, n).astype(np.float32)
+    x[rng.integers(0, n, 1000)] = 0.0
+    out = tg.encode([dev(x)], [b], [rnd], [987654321])[0]
+    rc, ref = oracle_cpu.terngrad_encode(x, b, rnd, 987654321)
+    assert rc == 0
+    assert_bits_equal(host(out), ref, f"message n={n} b={b}")
+
+
 def test_resident_and_tiled_tensors_in_one_call(tg, oracle_cpu, resident_from_2m):
     rng = np.random.default_rng(77)
     sizes = [3_000_001, 1000, 2_500_000, 70001, 2_097_152, 2_097_151]
