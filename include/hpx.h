@@ -66,7 +66,7 @@ int hpx_release_stream(hpx_stream_t stream);
  *                             decoders use streaming stores (default 128 MiB)
  *   "terngrad_resident_min"   smallest tensor, in elements, that
  *                             hpx_terngrad_encode sends through its
- *                             single-launch resident kernel (default 10 * 2^20,
+ *                             single-launch resident kernel (default 5 * 2^20,
  *                             where it starts to beat the two-launch encode;
  *                             negative: never)
  *   "terngrad_barrier_ms"     bound on that kernel's grid-barrier wait

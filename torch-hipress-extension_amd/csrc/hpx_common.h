@@ -182,8 +182,9 @@ size_t stream_store_max_bytes();
 enum Option {
   kOptStreamStoreMaxBytes = 0,  // "stream_store_max_bytes", default kStreamStoreMaxBytes
   kOptTerngradResidentMin,      // "terngrad_resident_min": smallest tensor (elements) that takes the
-                                // single-launch resident encode; negative = never.  Default 10 * 2^20:
-                                // below about 10 M elements the two-launch encode is faster (2.2 M: 8.7 against 14.9 us).
+                                // single-launch resident encode; negative = never.  Default 5 * 2^20:
+                                // below about 4 M elements the two-launch encode is faster (2 M: 7.3 against 10.9 us;
+                                // 4 M: 11.0 against 11.3; 6 M: 13.7 against 12.1).
   kOptTerngradBarrierMs,        // "terngrad_barrier_ms": bound on the resident kernel's barrier wait.  Default 2000.
   kOptTerngradResidentBucket,   // "terngrad_resident_bucket": 1 = a call with several tensors that fit the chip together
                                 // and add up to terngrad_resident_min elements takes ONE resident launch.  Default 1.

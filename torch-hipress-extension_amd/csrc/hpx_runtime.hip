@@ -189,7 +189,7 @@ struct OptionDef {
 };
 const OptionDef kOptions[kOptCount] = {
     {"stream_store_max_bytes", "HPX_STREAM_STORE_MAX_BYTES", int64_t(kStreamStoreMaxBytes)},
-    {"terngrad_resident_min", "HPX_TERNGRAD_RESIDENT_MIN", int64_t(10) << 20},
+    {"terngrad_resident_min", "HPX_TERNGRAD_RESIDENT_MIN", int64_t(5) << 20},
     {"terngrad_barrier_ms", "HPX_TERNGRAD_BARRIER_MS", 2000},
     {"terngrad_resident_bucket", "HPX_TERNGRAD_RESIDENT_BUCKET", 1},
 };

@@ -160,6 +160,28 @@ __device__ __forceinline__ float vmin3_abs(float a, float b, float c) {  // min(
   __asm__("v_min3_f32 %0, %1, |%2|, |%3|" : "=v"(r) : "v"(a), "v"(b), "v"(c));
   return r;
 }
+// 16 bytes per lane from global memory straight into LDS, without passing through registers: lane i's
+// piece lands at lds_wave_base + 16 * i (the base must be the same in every lane); lanes that are switched
+// off leave their 16 bytes of LDS as they were.  The load counts as a vector-memory load (vmcnt) and returns
+// in order with the others; the address needs 4-byte alignment only.  Non-temporal, like ld4_stream.
+//
+// Written out as instructions, so that the compiler does not know of it: told of loads into LDS in flight,
+// it makes every LDS access wait for all of them, and every use of an ordinary load that follows them too
+// (it no longer trusts the order of returns), which serialises the whole pass.  Unaware of them, its counted
+// waits for the ordinary loads stay right as long as these loads are requested BEFORE those (returns are in
+// order, so a wait for "at most N younger loads outstanding" also covers everything older).  The caller
+// answers for the rest: wait_vector_loads() before anything reads the LDS the loads fill.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"  // m0 is reserved, and naming it is still how the compiler learns that it changes
+__device__ __forceinline__ void ld4_stream_to_lds(const float* p, float4* lds_wave_base) {
+  const uint32_t base = __builtin_amdgcn_readfirstlane(
+      static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)lds_wave_base)));
+  __asm__ volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt" ::"v"(p), "s"(base) : "memory", "m0");
+}
+#pragma clang diagnostic pop
+// Waits for every vector-memory load of the wave, LDS-bound ones included.
+__device__ __forceinline__ void wait_vector_loads() { __asm__ volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
 // min, max and min |x| over four elements: six instructions.
 __device__ __forceinline__ void acc3x4(const float4& v, float& mn, float& mx, float& am) {
   mn = vmin3(mn, v.x, v.y); mx = vmax3(mx, v.x, v.y); am = vmin3_abs(am, v.x, v.y);
@@ -547,7 +569,9 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
   const float qnan = __builtin_nanf("");  // compares false both ways: ignored by min and max
 
   // ---- pass 1: load the share, reduce ------------------------------------------
-  // All loads of the lane are requested at once: the first LDS row, then its register rows.  While
+  // All loads of the lane are requested at once: the LDS rows, which go straight into LDS and cost no
+  // registers on the way (lanes past the end of the share keep whatever their slot held: every later
+  // reader checks the bound), then its register rows.  While
   // they are in flight and the ALUs idle, the random addends of the first PRE register rows, which
   // depend on position and seed only, go into the LDS the tensor does not need; pass 2 (ALU-bound:
   // nothing left to overlap with) then skips 6 of its 11 operations per element for those rows.
@@ -557,18 +581,20 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
   // workgroup whose register rows are all whole, and the others - because behind a join of the
   // two the compiler no longer knows the order of the loads and waits for all of them at once.
   float4 v[KU][H];
-  float4 t0[H];
   constexpr int PREG = res_pre_reg_rows(B, PRE);
   float4 pre_reg[PREG > 0 ? PREG : 1][H];
   float4* s_pre = s_rows + size_t(a.lds_rows) * H * kResThreads;
   float mn = __builtin_inff(), mx = -__builtin_inff(), am = __builtin_inff();
   const bool whole_rows = wg_u0 + uint32_t(KU * kResThreads) <= wg_end;
-  auto pass1 = [&](auto whole) {
-    if (a.lds_rows > 0) {
+  const uint32_t wave_lane0 = __builtin_amdgcn_readfirstlane(threadIdx.x & ~uint32_t(kWave - 1));
+  for (uint32_t r = 0; r < a.lds_rows; r++) {
+    const uint32_t u = l0 + r * kResThreads;
+    if (u < wg_end) {
 #pragma unroll
-      for (int h = 0; h < H; h++)
-        t0[h] = l0 < wg_end ? ld4_stream(xp + size_t(l0) * UNIT + h * 4) : make_float4(qnan, qnan, qnan, qnan);
+      for (int h = 0; h < H; h++) ld4_stream_to_lds(xp + size_t(u) * UNIT + h * 4, s_rows + (r * H + h) * kResThreads + wave_lane0);
     }
+  }
+  auto pass1 = [&](auto whole) {
 #pragma unroll
     for (int k = 0; k < KU; k++) {
       const uint32_t u = u0 + k * rs;
@@ -577,6 +603,7 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
         v[k][h] = (decltype(whole)::value || (uint32_t(k) < R && u < wg_end)) ? ld4_stream(xp + size_t(u) * UNIT + h * 4)
                                                          : make_float4(qnan, qnan, qnan, qnan);
     }
+    __builtin_amdgcn_sched_barrier(0);  // every load is requested before any other work: nothing moves across this line
     if (RANDOM && PRE > 0) {
       uint32_t d[UNIT];
       const uint32_t x0 = a.seg.seed + u0 * BPU;
@@ -603,26 +630,17 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
         for (int q = 0; q < UNIT; q++) d[q] += lcg_mul(q % DPB + 2) * stride_bytes;
       }
     }
-    if (a.lds_rows > 0) {
-#pragma unroll
-      for (int h = 0; h < H; h++) {
-        s_rows[h * kResThreads + threadIdx.x] = t0[h];
-        acc3x4(t0[h], mn, mx, am);
-      }
-    }
 #pragma unroll
     for (int k = 0; k < KU; k++)
 #pragma unroll
       for (int h = 0; h < H; h++) acc3x4(v[k][h], mn, mx, am);
   };
   if (whole_rows) pass1(std::true_type{}); else pass1(std::false_type{});
-  for (uint32_t r = 1; r < a.lds_rows; r++) {
-    const uint32_t u = l0 + r * kResThreads;
+  if (a.lds_rows > 0) wait_vector_loads();  // the LDS rows were requested first and have long landed
+  for (uint32_t r = 0; r < a.lds_rows; r++) {
+    if (l0 + r * kResThreads < wg_end) {
 #pragma unroll
-    for (int h = 0; h < H; h++) {
-      const float4 f = u < wg_end ? ld4_stream(xp + size_t(u) * UNIT + h * 4) : make_float4(qnan, qnan, qnan, qnan);
-      s_rows[(r * H + h) * kResThreads + threadIdx.x] = f;
-      acc3x4(f, mn, mx, am);
+      for (int h = 0; h < H; h++) acc3x4(s_rows[(r * H + h) * kResThreads + threadIdx.x], mn, mx, am);
     }
   }
   uint32_t fz = 0xFFFFFFFFu;
@@ -632,10 +650,13 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
     for (int k = 0; k < KU; k++)
 #pragma unroll
       for (int h = 0; h < H; h++) acc_zero4(v[k][h], (u0 + k * rs) * UNIT + h * 4, d0, d1, fz);
-    for (uint32_t r = 0; r < a.lds_rows; r++)  // this lane's own LDS rows, read back
+    for (uint32_t r = 0; r < a.lds_rows; r++) {  // this lane's own LDS rows
+      if (l0 + r * kResThreads < wg_end) {
 #pragma unroll
-      for (int h = 0; h < H; h++)
-        acc_zero4(s_rows[(r * H + h) * kResThreads + threadIdx.x], (l0 + r * kResThreads) * UNIT + h * 4, d0, d1, fz);
+        for (int h = 0; h < H; h++)
+          acc_zero4(s_rows[(r * H + h) * kResThreads + threadIdx.x], (l0 + r * kResThreads) * UNIT + h * 4, d0, d1, fz);
+      }
+    }
   }
   if (blockIdx.x == 0 && threadIdx.x == 0)
     for (uint32_t e = full_units * UNIT; e < n; e++) acc_zero(xp[e], e, mn, mx, fz);
@@ -822,20 +843,21 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_multi_kernel(co
   float4* s_pre = s_rows + size_t(kWaves) * a.lds_rows * H * kWave + size_t(wave) * PRE * H * kWave;
 
   // ---- pass 1: load the piece, reduce ---------------------------------------------
-  // As in the single-tensor kernel: all loads at once (the first LDS row ahead of the register rows), the
+  // As in the single-tensor kernel: all loads at once (the LDS rows, straight into LDS, ahead of the register rows), the
   // random addends of the first PRE rows while they are in flight, then every row reduced as it arrives,
   // one straight block per case.
   float4 v[KU][H];
-  float4 t0[H];
   float mn = __builtin_inff(), mx = -__builtin_inff(), am = __builtin_inff();
   const bool whole_rows = u_beg + uint32_t(KU * kWave) <= u_end;
   const uint32_t ul0 = u0 + uint32_t(KU) * kWave;  // this lane's unit in the first LDS row
-  auto pass1 = [&](auto whole) {
-    if (a.lds_rows > 0) {
+  for (uint32_t r = 0; r < a.lds_rows; r++) {
+    const uint32_t u = ul0 + r * kWave;
+    if (u < u_end) {
 #pragma unroll
-      for (int h = 0; h < H; h++)
-        t0[h] = ul0 < u_end ? ld4_stream(xp + size_t(ul0) * UNIT + h * 4) : make_float4(qnan, qnan, qnan, qnan);
+      for (int h = 0; h < H; h++) ld4_stream_to_lds(xp + size_t(u) * UNIT + h * 4, s_mine + (r * H + h) * kWave);
     }
+  }
+  auto pass1 = [&](auto whole) {
 #pragma unroll
     for (int k = 0; k < KU; k++) {
       const uint32_t u = u0 + k * kWave;
@@ -844,6 +866,7 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_multi_kernel(co
         v[k][h] = (decltype(whole)::value || u < u_end) ? ld4_stream(xp + size_t(u) * UNIT + h * 4)
                                                         : make_float4(qnan, qnan, qnan, qnan);
     }
+    __builtin_amdgcn_sched_barrier(0);  // every load is requested before any other work: nothing moves across this line
     if (RANDOM && PRE > 0) {
       uint32_t d[UNIT];
       const uint32_t x0 = sg.seed + u0 * BPU;
@@ -861,26 +884,17 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_multi_kernel(co
         for (int q = 0; q < UNIT; q++) d[q] += lcg_mul(q % DPB + 2) * stride_bytes;
       }
     }
-    if (a.lds_rows > 0) {
-#pragma unroll
-      for (int h = 0; h < H; h++) {
-        s_mine[h * kWave + lane] = t0[h];
-        acc3x4(t0[h], mn, mx, am);
-      }
-    }
 #pragma unroll
     for (int k = 0; k < KU; k++)
 #pragma unroll
       for (int h = 0; h < H; h++) acc3x4(v[k][h], mn, mx, am);
   };
   if (whole_rows) pass1(std::true_type{}); else pass1(std::false_type{});
-  for (uint32_t r = 1; r < a.lds_rows; r++) {
-    const uint32_t u = ul0 + r * kWave;
+  if (a.lds_rows > 0) wait_vector_loads();
+  for (uint32_t r = 0; r < a.lds_rows; r++) {
+    if (ul0 + r * kWave < u_end) {
 #pragma unroll
-    for (int h = 0; h < H; h++) {
-      const float4 f = u < u_end ? ld4_stream(xp + size_t(u) * UNIT + h * 4) : make_float4(qnan, qnan, qnan, qnan);
-      s_mine[(r * H + h) * kWave + lane] = f;
-      acc3x4(f, mn, mx, am);
+      for (int h = 0; h < H; h++) acc3x4(s_mine[(r * H + h) * kWave + lane], mn, mx, am);
     }
   }
   uint32_t fz = 0xFFFFFFFFu;
@@ -890,10 +904,13 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_multi_kernel(co
     for (int k = 0; k < KU; k++)
 #pragma unroll
       for (int h = 0; h < H; h++) acc_zero4(v[k][h], (u0 + k * kWave) * UNIT + h * 4, d0, d1, fz);
-    for (uint32_t r = 0; r < a.lds_rows; r++)  // this lane's own LDS rows, read back
+    for (uint32_t r = 0; r < a.lds_rows; r++) {  // this lane's own LDS rows
+      if (ul0 + r * kWave < u_end) {
 #pragma unroll
-      for (int h = 0; h < H; h++)
-        acc_zero4(s_mine[(r * H + h) * kWave + lane], (ul0 + r * kWave) * UNIT + h * 4, d0, d1, fz);
+        for (int h = 0; h < H; h++)
+          acc_zero4(s_mine[(r * H + h) * kWave + lane], (ul0 + r * kWave) * UNIT + h * 4, d0, d1, fz);
+      }
+    }
   }
   if (ends_tensor && lane == 0)
     for (uint32_t e = full_units * UNIT; e < n; e++) acc_zero(xp[e], e, mn, mx, fz);
