@@ -98,20 +98,34 @@ struct DecArgs {
 };
 static_assert(sizeof(EncArgs<kCapLarge>) <= 9600 && sizeof(DecArgs<kCapLarge>) <= 9600, "kernel-argument budget");
 
+// Reductions over the 64 lanes of a wave through the lane-permuting forms of the move instruction (no LDS
+// round trips): within quads, within rows of 16, then row 0 into row 1 and row 2 into row 3, then rows 0-1
+// into rows 2-3; lane 63 holds the result and hands it to every lane.
+template <typename T, typename Op>
+__device__ __forceinline__ T wave_reduce(T v, Op op) {
+  static_assert(sizeof(T) == 4, "32-bit values");
+  auto perm = [](T x, auto ctrl, auto rows) {
+    const int xi = __builtin_bit_cast(int, x);
+    // lanes whose row is not named keep their own value
+    return __builtin_bit_cast(T, __builtin_amdgcn_update_dpp(xi, xi, decltype(ctrl)::value, decltype(rows)::value, 0xF, false));
+  };
+  using std::integral_constant;
+  v = op(v, perm(v, integral_constant<int, 0xB1>{}, integral_constant<int, 0xF>{}));   // quad_perm [1,0,3,2]
+  v = op(v, perm(v, integral_constant<int, 0x4E>{}, integral_constant<int, 0xF>{}));   // quad_perm [2,3,0,1]
+  v = op(v, perm(v, integral_constant<int, 0x141>{}, integral_constant<int, 0xF>{}));  // row_half_mirror
+  v = op(v, perm(v, integral_constant<int, 0x140>{}, integral_constant<int, 0xF>{}));  // row_mirror
+  v = op(v, perm(v, integral_constant<int, 0x142>{}, integral_constant<int, 0xA>{}));  // row_bcast:15 into rows 1 and 3
+  v = op(v, perm(v, integral_constant<int, 0x143>{}, integral_constant<int, 0xC>{}));  // row_bcast:31 into rows 2 and 3
+  return __builtin_bit_cast(T, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
 __device__ __forceinline__ float wave_min(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) { float t = __shfl_xor(v, o, 64); v = t < v ? t : v; }
-  return v;
+  return wave_reduce(v, [](float a, float b) { return b < a ? b : a; });
 }
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) { float t = __shfl_xor(v, o, 64); v = t > v ? t : v; }
-  return v;
+  return wave_reduce(v, [](float a, float b) { return b > a ? b : a; });
 }
 __device__ __forceinline__ uint32_t wave_min_u32(uint32_t v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) { uint32_t t = __shfl_xor(v, o, 64); v = t < v ? t : v; }
-  return v;
+  return wave_reduce(v, [](uint32_t a, uint32_t b) { return b < a ? b : a; });
 }
 
 // Block-wide (min, max, min-u32) over 4 waves.  Result valid in every thread.
@@ -197,9 +211,7 @@ __device__ __forceinline__ float from_okey(uint32_t k) {
   return __uint_as_float(k ^ ((k >> 31) ? 0x80000000u : 0xFFFFFFFFu));
 }
 __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) { uint32_t t = __shfl_xor(v, o, 64); v = t > v ? t : v; }
-  return v;
+  return wave_reduce(v, [](uint32_t a, uint32_t b) { return b > a ? b : a; });
 }
 
 // Pass 1 of encode.  Each workgroup reduces one kRedTile-element tile and folds its
@@ -943,17 +955,25 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_multi_kernel(co
 
   // ---- pass 2: the tensor's extremes, then quantise from registers ----------------
   {
+    // All loads of a lane are in flight together (a lane reads a way that is not in use again from way 0:
+    // a fold of maxima does not mind): one memory latency for the fold, not one per 64 ways.
+    static_assert(kSlotWays == 2 * kWave, "two ways per lane");
     uint32_t kx = 0u, kn = 0u, kz = 0u;
-    for (uint32_t w = lane; w < ways; w += kWave) {
-      const unsigned long long vx = __hip_atomic_load(sl + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const unsigned long long vn = __hip_atomic_load(sl + kSlotWays + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const unsigned long long vz = __hip_atomic_load(sl + 2 * kSlotWays + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const uint32_t x1 = (uint32_t(vx >> 32) == a.epoch) ? uint32_t(vx) : 0u;
-      const uint32_t n1 = (uint32_t(vn >> 32) == a.epoch) ? uint32_t(vn) : 0u;
-      const uint32_t z1 = (uint32_t(vz >> 32) == a.epoch) ? uint32_t(vz) : 0u;
-      kx = x1 > kx ? x1 : kx;
-      kn = n1 > kn ? n1 : kn;
-      kz = z1 > kz ? z1 : kz;
+    {
+      const uint32_t w0 = lane < ways ? lane : 0u, w1 = lane + kWave < ways ? lane + kWave : 0u;
+      unsigned long long v[6];
+      v[0] = __hip_atomic_load(sl + w0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      v[1] = __hip_atomic_load(sl + kSlotWays + w0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      v[2] = __hip_atomic_load(sl + 2 * kSlotWays + w0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      v[3] = __hip_atomic_load(sl + w1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      v[4] = __hip_atomic_load(sl + kSlotWays + w1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      v[5] = __hip_atomic_load(sl + 2 * kSlotWays + w1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      uint32_t k[6];
+#pragma unroll
+      for (int i = 0; i < 6; i++) k[i] = (uint32_t(v[i] >> 32) == a.epoch) ? uint32_t(v[i]) : 0u;
+      kx = k[0] > k[3] ? k[0] : k[3];
+      kn = k[1] > k[4] ? k[1] : k[4];
+      kz = k[2] > k[5] ? k[2] : k[5];
     }
     kx = wave_max_u32(kx);
     kn = wave_max_u32(kn);
