@@ -89,7 +89,7 @@ struct Workspace {
 constexpr size_t kStateWords = 4096;       // 16 KiB
 constexpr size_t kStatusWord = kStateWords - 16;  // sticky flags live here
 constexpr size_t kPinnedBytes = 1 << 16;
-constexpr size_t kBarWords = 40960;                       // 160 KiB of exchange memory for grid-wide barriers
+constexpr size_t kBarWords = 524288;                      // 2 MiB of exchange memory for grid-wide barriers
 constexpr size_t kPinnedFlagOffset = kPinnedBytes - 64;   // host word raised by a kernel whose barrier wait expired
 
 // The record for the calling thread's current device and `stream` (created on
@@ -237,84 +237,85 @@ __device__ __forceinline__ global_ptr<T> as_global(const T* p) {
 // For kernels launched with at most kBarMaxWorkgroups workgroups that are all
 // resident at once (the host guarantees it: grid <= CUs, one workgroup fits a CU,
 // and only one stream per device launches such kernels).
-constexpr int kBarGroup = 16;           // workgroups per group; also the largest number of groups
-constexpr int kBarMaxWorkgroups = kBarGroup * kBarGroup;
+constexpr int kBarMaxWorkgroups = 256;
+constexpr int kBarWaves = 4;            // waves of a workgroup that take part: each looks after a quarter of the grid
+constexpr int kBarQuarter = kBarMaxWorkgroups / kBarWaves;  // = the lanes of a wave
 constexpr int kBarRecWords = 4;         // 64-bit words per record (three used)
-constexpr int kBarAreaWords = kBarGroup * kBarRecWords;  // one area: 16 records = 64 words = 512 bytes
-// Exchange memory, in 64-bit words: group areas first (members report here), then
-// one area per workgroup (group leaders report here).
-constexpr size_t kBarGroupBase = 0;
-constexpr size_t kBarWgBase = size_t(kBarGroup) * kBarAreaWords;
-constexpr size_t kBarTotalWords = kBarWgBase + size_t(kBarMaxWorkgroups) * kBarAreaWords;
+// Exchange memory, in 64-bit words: one area per workgroup, holding one record per source workgroup.
+constexpr size_t kBarAreaWords = size_t(kBarMaxWorkgroups) * kBarRecWords;  // 8 KiB
+constexpr size_t kBarTotalWords = size_t(kBarMaxWorkgroups) * kBarAreaWords;
 static_assert(kBarTotalWords * 8 <= kBarWords * 4, "barrier memory too small");
-
+static_assert(kBarQuarter == kWave, "a wave's quarter is one source per lane-quad times four rounds");
 
 // Grid-wide exchange of (max key, min key, first-zero key) and barrier in one.
-// Every lane of wave 0 of every workgroup calls it once per launch with the
-// workgroup's three keys; on success every lane holds the grid-wide maximum of
-// key[lane & 3] (lanes with (lane & 3) == 3 hold nothing of use).
+// All lanes of the first kBarWaves waves of every workgroup call it once per launch
+// with the workgroup's three keys (the same in every caller of a workgroup) and the
+// caller's wave index.  On success k0, k1, k2 hold, the same in every lane, the maximum of
+// each key over the quarter of the grid this wave looks after (workgroups
+// 64 * wave ... 64 * wave + 63); the caller folds the quarters.
 //
-// The protocol uses only stores and polling loads, no read-modify-write and no
-// fence: a member writes its record (three self-validating words, generation in
-// the high half) into its group's area; the group's leader polls that area with
-// one wave-wide load until all records carry this generation, folds them, and
-// writes the group's record into the area of EVERY workgroup; each workgroup
-// polls its own area until all groups have reported.  A polled line has one
-// reader, a written line at most 16 writers, and the critical path is two
-// store-to-load hand-overs.  (A counter-based barrier - fence, two dependent
-// atomics, a release flag, then reading the reduction slots - took 7 us here;
-// polling one shared word from all 256 workgroups took 10.)
-__device__ __forceinline__ bool grid_exchange(uint64_t* bar, uint32_t gen, uint64_t spin_limit, uint32_t& key) {
-  const uint32_t lane = threadIdx.x;  // < 64
-  const uint32_t nwg = gridDim.x, grp = blockIdx.x / kBarGroup, mem = blockIdx.x % kBarGroup;
-  const uint32_t ngrp = (nwg + kBarGroup - 1) / kBarGroup;
-  const uint32_t left = nwg - grp * kBarGroup;
-  const uint32_t gsz = left < uint32_t(kBarGroup) ? left : uint32_t(kBarGroup);
+// The protocol is ONE hand-over and uses only stores and polling loads, no
+// read-modify-write and no fence: a workgroup writes its record (three
+// self-validating 64-bit words, generation in the high half) into the area of
+// EVERY workgroup, the three words from neighbouring lanes so that they leave as
+// one request; every workgroup polls its own area until all records carry this
+// generation.  A polled line has one reader and four writers; nothing is ever
+// reset (generations only grow).  With four waves at it, a wave keeps just four
+// loads in flight per round.  (Two hand-overs through group leaders - each member
+// reports to its leader, the leader to everyone - took 2.4 us against this
+// one's [see the measurements]; a counter-based barrier - fence, two dependent atomics, a release flag,
+// then reading the reduction slots - took 7 us; polling one shared word from all
+// 256 workgroups took 10.)
+__device__ __forceinline__ bool grid_exchange(uint64_t* bar, uint32_t gen, uint64_t spin_limit, uint32_t wave, uint32_t& k0, uint32_t& k1, uint32_t& k2) {
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const uint32_t nwg = gridDim.x, me = blockIdx.x;
+  const uint32_t rec = lane / kBarRecWords, word = lane % kBarRecWords;
+  const uint32_t q0 = wave * uint32_t(kBarQuarter);  // first workgroup of this wave's quarter
+  if (q0 >= nwg) {
+    k0 = k1 = k2 = 0u;
+    return true;
+  }
   const uint64_t tag = uint64_t(gen) << 32;
   const uint64_t t0 = wall_clock64();
-  unsigned long long* garea = reinterpret_cast<unsigned long long*>(bar) + kBarGroupBase + size_t(grp) * kBarAreaWords;
-  unsigned long long* warea = reinterpret_cast<unsigned long long*>(bar) + kBarWgBase + size_t(blockIdx.x) * kBarAreaWords;
-  const uint32_t rec = lane / kBarRecWords, word = lane % kBarRecWords;
+  unsigned long long* base = reinterpret_cast<unsigned long long*>(bar);
 
-  if (lane < 3) __hip_atomic_store(&garea[mem * kBarRecWords + lane], tag | key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-
-  bool ok = true;
-  if (mem == 0) {  // group leader
-    uint32_t k = 0;
-    for (;;) {
-      const unsigned long long v = __hip_atomic_load(&garea[lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const bool valid = word == 3 || rec >= gsz || uint32_t(v >> 32) == gen;
-      k = (word == 3 || rec >= gsz) ? 0u : uint32_t(v);
-      if (__ballot(valid) == ~0ull) break;
-      if (wall_clock64() - t0 > spin_limit) { ok = false; break; }
-      __builtin_amdgcn_s_sleep(1);
-    }
-    if (ok) {
+  // (written with masks: as a chain of selects the compiler turns it into a table in private memory)
+  const uint32_t mine_key = (k0 & (0u - uint32_t(word == 0))) | (k1 & (0u - uint32_t(word == 1))) | (k2 & (0u - uint32_t(word == 2)));
+  if (word < 3) {
 #pragma unroll
-      for (int o = kBarRecWords; o < kWave; o <<= 1) { const uint32_t t = __shfl_xor(k, o, 64); k = t > k ? t : k; }
-      // lane l now holds the group's key (l & 3); lanes 0..2 of each quad of lanes write it out
-      unsigned long long* wbase = reinterpret_cast<unsigned long long*>(bar) + kBarWgBase + size_t(grp) * kBarRecWords;
-      if (word < 3) {
-        for (uint32_t w = rec; w < nwg; w += kWave / kBarRecWords)
-          __hip_atomic_store(&wbase[size_t(w) * kBarAreaWords + word], tag | k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
+    for (uint32_t j = 0; j < uint32_t(kWave / (kWave / kBarRecWords)); j++) {
+      const uint32_t d = q0 + j * (kWave / kBarRecWords) + rec;
+      if (d < nwg)
+        __hip_atomic_store(&base[(size_t(d) * kBarMaxWorkgroups + me) * kBarRecWords + word], tag | mine_key, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
     }
   }
-  ok = __builtin_amdgcn_readfirstlane(ok ? 1 : 0) != 0;
-  if (!ok) return false;
 
+  const unsigned long long* area = base + size_t(me) * kBarAreaWords + size_t(q0) * kBarRecWords;
   uint32_t k = 0;
   for (;;) {
-    const unsigned long long v = __hip_atomic_load(&warea[lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const bool valid = word == 3 || rec >= ngrp || uint32_t(v >> 32) == gen;
-    k = (word == 3 || rec >= ngrp) ? 0u : uint32_t(v);
-    if (__ballot(valid) == ~0ull) break;
+    unsigned long long v[kBarRecWords];
+#pragma unroll
+    for (int j = 0; j < kBarRecWords; j++) v[j] = __hip_atomic_load(&area[j * kWave + lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    bool all = true;
+    k = 0;
+#pragma unroll
+    for (int j = 0; j < kBarRecWords; j++) {
+      const uint32_t src = q0 + uint32_t(j) * (kWave / kBarRecWords) + rec;
+      const bool idle = word == 3 || src >= nwg;
+      all = all && (idle || uint32_t(v[j] >> 32) == gen);
+      const uint32_t kk = idle ? 0u : uint32_t(v[j]);
+      k = kk > k ? kk : k;
+    }
+    if (__ballot(all) == ~0ull) break;
     if (wall_clock64() - t0 > spin_limit) return false;
     __builtin_amdgcn_s_sleep(1);
   }
 #pragma unroll
   for (int o = kBarRecWords; o < kWave; o <<= 1) { const uint32_t t = __shfl_xor(k, o, 64); k = t > k ? t : k; }
-  key = k;
+  k0 = __builtin_amdgcn_readlane(k, 0);
+  k1 = __builtin_amdgcn_readlane(k, 1);
+  k2 = __builtin_amdgcn_readlane(k, 2);
   return true;
 }
 

@@ -562,7 +562,7 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
   extern __shared__ float4 s_rows[];  // [lds_rows][H][kResThreads]
   __shared__ float s_mn[kWaves], s_mx[kWaves];
   __shared__ uint32_t s_fz[kWaves];
-  __shared__ uint32_t s_k[4];
+  __shared__ uint32_t s_q[kBarWaves][4];  // per quarter of the grid: the three keys, then 1 if its wait ended in time
 
   const float* __restrict__ xp = a.seg.x;
   const uint32_t n = static_cast<uint32_t>(a.seg.n);
@@ -680,41 +680,41 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
     s_mn[threadIdx.x / kWave] = mn; s_mx[threadIdx.x / kWave] = mx; s_fz[threadIdx.x / kWave] = fz;
   }
   __syncthreads();
-  if (threadIdx.x < kWave) {
-    if (threadIdx.x == 0) {
-#pragma unroll
-      for (int i = 1; i < kWaves; i++) {
-        mn = s_mn[i] < mn ? s_mn[i] : mn;
-        mx = s_mx[i] > mx ? s_mx[i] : mx;
-        fz = s_fz[i] < fz ? s_fz[i] : fz;
-      }
-    }
-    mn = __shfl(mn, 0, 64);
-    mx = __shfl(mx, 0, 64);
-    fz = __shfl(fz, 0, 64);
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  if (wave < uint32_t(kBarWaves)) {
+    // Each wave that takes part in the exchange folds the workgroup's sixteen results for itself.
+    const uint32_t i = threadIdx.x & (kWaves - 1);
+    mn = wave_min(s_mn[i]);
+    mx = wave_max(s_mx[i]);
+    fz = wave_min_u32(s_fz[i]);
     const bool has = mx >= mn;  // false only for a workgroup whose share is empty
-    // lane 0: largest key of x; lane 1: largest complemented key (the minimum);
-    // lane 2: complemented index of the first zero, 0 for none
-    uint32_t key = threadIdx.x == 0 ? (has ? okey(mx) : 0u)
-                 : threadIdx.x == 1 ? (has ? ~okey(mn) : 0u)
-                                    : (fz != 0xFFFFFFFFu ? 0xFFFFFFFEu - fz : 0u);
-    const bool ok = grid_exchange(a.bar, a.gen, a.spin_limit, key);
-    if (threadIdx.x < 3) s_k[threadIdx.x] = key;
-    if (threadIdx.x == 0) {
+    // largest key of x; largest complemented key (the minimum); complemented index of the first zero, 0 for none
+    uint32_t k0 = has ? okey(mx) : 0u, k1 = has ? ~okey(mn) : 0u, k2 = fz != 0xFFFFFFFFu ? 0xFFFFFFFEu - fz : 0u;
+    const bool ok = grid_exchange(a.bar, a.gen, a.spin_limit, wave, k0, k1, k2);
+    if ((threadIdx.x & (kWave - 1)) == 0) {
       if (!ok) __hip_atomic_store(a.host_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-      s_k[3] = ok ? 1u : 0u;
+      s_q[wave][0] = k0; s_q[wave][1] = k1; s_q[wave][2] = k2;
+      s_q[wave][3] = ok ? 1u : 0u;
     }
   }
   __syncthreads();
-  if (s_k[3] == 0u) return;
+  uint32_t kx = 0u, kn = 0u, kz = 0u, oks = 1u;
+#pragma unroll
+  for (int q = 0; q < kBarWaves; q++) {
+    kx = s_q[q][0] > kx ? s_q[q][0] : kx;
+    kn = s_q[q][1] > kn ? s_q[q][1] : kn;
+    kz = s_q[q][2] > kz ? s_q[q][2] : kz;
+    oks &= s_q[q][3];
+  }
+  if (oks == 0u) return;
 
   // ---- pass 2: quantise from registers -------------------------------------------
-  mx = from_okey(s_k[0]);
-  mn = from_okey(~s_k[1]);
-  if ((mn == 0.0f || mx == 0.0f) && s_k[2] != 0u) {
+  mx = from_okey(kx);
+  mn = from_okey(~kn);
+  if ((mn == 0.0f || mx == 0.0f) && kz != 0u) {
     // thrust::minmax_element returns the first extreme: a zero extreme carries the
     // sign of the first zero of the tensor.
-    const float zv = xp[0xFFFFFFFEu - s_k[2]];
+    const float zv = xp[0xFFFFFFFEu - kz];
     if (mn == 0.0f) mn = zv;
     if (mx == 0.0f) mx = zv;
   }
@@ -829,7 +829,7 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_multi_kernel(co
   constexpr int kWaves = kResThreads / kWave;
   constexpr uint32_t stride_bytes = uint32_t(kWave) * BPU;
   extern __shared__ float4 s_rows[];  // [wave][lds_rows][H][64], then the prepared draws [wave][PRE][H][64]
-  __shared__ uint32_t s_ok;
+  __shared__ uint32_t s_ok[kBarWaves];
 
   // The wave index is the same in every lane: taken from the first lane, it and all that is derived from it
   // (piece, tensor, bounds) live in scalar registers.
@@ -942,16 +942,19 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_multi_kernel(co
     __asm__ volatile("" ::"v"(old));
   }
   __syncthreads();
-  if (threadIdx.x < kWave) {
-    uint32_t key = 0u;
-    const bool ok = grid_exchange(a.bar, a.gen, a.spin_limit, key);
-    if (threadIdx.x == 0) {
+  if (wave < uint32_t(kBarWaves)) {
+    uint32_t k0 = 0u, k1 = 0u, k2 = 0u;  // the exchange only serves as the barrier here
+    const bool ok = grid_exchange(a.bar, a.gen, a.spin_limit, wave, k0, k1, k2);
+    if (lane == 0) {
       if (!ok) __hip_atomic_store(a.host_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-      s_ok = ok ? 1u : 0u;
+      s_ok[wave] = ok ? 1u : 0u;
     }
   }
   __syncthreads();
-  if (s_ok == 0u || !active) return;
+  uint32_t oks = 1u;
+#pragma unroll
+  for (int q = 0; q < kBarWaves; q++) oks &= s_ok[q];
+  if (oks == 0u || !active) return;
 
   // ---- pass 2: the tensor's extremes, then quantise from registers ----------------
   {
