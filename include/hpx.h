@@ -76,6 +76,11 @@ int hpx_release_stream(hpx_stream_t stream);
  *                             least terngrad_resident_min elements and fit the
  *                             chip together takes ONE resident launch for all of
  *                             them; 0: each tensor is looked at on its own
+ *   "terngrad_resident_workgroups" workgroups of a resident launch; 0
+ *                             (default): one per CU of the device.  A process
+ *                             that may only use some of the CUs (a CU mask)
+ *                             must set it to that number: the workgroups of a
+ *                             resident launch wait for each other
  * Unknown names return HPX_ERR_ARG. */
 int hpx_set_option(const char* name, int64_t value);
 int hpx_get_option(const char* name, int64_t* value);

@@ -330,6 +330,27 @@ def test_resident_shares_between_one_row_and_the_register_rows(tg, oracle_cpu, r
     assert_bits_equal(host(out), ref, f"message n={n} b={b}")
 
 
+@pytest.mark.parametrize("wgs", [1, 17, 63, 64, 65, 128, 200, 255])
+def test_resident_launches_with_fewer_workgroups_than_cus(tg, oracle_cpu, capi, resident_forced, wgs):
+    # the grid-wide exchange with a quarter that is partly filled, exactly filled, or empty; shares grow with
+    # the smaller grid, so the sizes keep within what that many workgroups hold
+    old = capi.set_option("terngrad_resident_workgroups", wgs)
+    try:
+        rng = np.random.default_rng(wgs)
+        per_wg = 32 * 1024 * 4                                   # elements one workgroup can hold at 2 bits
+        sizes = [max(5, min(3_000_001, wgs * per_wg - 7)), 100_003, 7]
+        xs = [rng.normal(0, 1e-2, n).astype(np.float32) for n in sizes]
+        xs[0][rng.integers(0, sizes[0], 50)] = 0.0
+        _check(tg, oracle_cpu, xs, [2, 2, 4], [1, 0, 1], [11, 12, 13], [0, 0, 0], rng)
+        # and several tensors in one launch
+        capi.set_option("terngrad_resident_bucket", 1)
+        ys = [rng.normal(0, 1e-2, n).astype(np.float32) for n in (40_001, 90_000, 13, 70_007)]
+        _check(tg, oracle_cpu, ys, [2] * 4, [1] * 4, [21, 22, 23, 24], [0] * 4, rng)
+    finally:
+        capi.set_option("terngrad_resident_workgroups", old)
+        capi.set_option("terngrad_resident_bucket", 0)
+
+
 def test_resident_and_tiled_tensors_in_one_call(tg, oracle_cpu, resident_from_2m):
     rng = np.random.default_rng(77)
     sizes = [3_000_001, 1000, 2_500_000, 70001, 2_097_152, 2_097_151]

@@ -188,6 +188,9 @@ enum Option {
   kOptTerngradBarrierMs,        // "terngrad_barrier_ms": bound on the resident kernel's barrier wait.  Default 2000.
   kOptTerngradResidentBucket,   // "terngrad_resident_bucket": 1 = a call with several tensors that fit the chip together
                                 // and add up to terngrad_resident_min elements takes ONE resident launch.  Default 1.
+  kOptTerngradResidentWorkgroups,  // "terngrad_resident_workgroups": workgroups of a resident launch; 0 (default) = one per CU.
+                                   // For a process that may only use some of the CUs (a CU mask), which the device's CU
+                                   // count does not show: a resident launch needs all its workgroups running at once.
   kOptCount
 };
 int64_t option(Option o);

@@ -192,6 +192,7 @@ const OptionDef kOptions[kOptCount] = {
     {"terngrad_resident_min", "HPX_TERNGRAD_RESIDENT_MIN", int64_t(5) << 20},
     {"terngrad_barrier_ms", "HPX_TERNGRAD_BARRIER_MS", 2000},
     {"terngrad_resident_bucket", "HPX_TERNGRAD_RESIDENT_BUCKET", 1},
+    {"terngrad_resident_workgroups", "HPX_TERNGRAD_RESIDENT_WORKGROUPS", 0},
 };
 std::atomic<int64_t> g_opt[kOptCount];
 std::once_flag g_opt_once;

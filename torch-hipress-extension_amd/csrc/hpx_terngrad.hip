@@ -1537,14 +1537,22 @@ uint64_t resident_spin_limit() {
   return uint64_t(ms < 0 ? 0 : ms) * 100000ull;  // wall_clock64 ticks at 100 MHz
 }
 
+// Workgroups of a resident launch: one per CU, or fewer when the option says so (a process that has been
+// given only some of the CUs must say so: the workgroups of such a launch wait for each other, so all of them
+// have to run at the same time).
+int resident_grid(const hpx::Workspace* ws) {
+  const int64_t cap = hpx::option(hpx::kOptTerngradResidentWorkgroups);
+  return (cap > 0 && cap < ws->num_cus) ? int(cap) : ws->num_cus;
+}
+
 // Fills chunk_units / lds_rows when tensor (n, bits) fits the chip; false otherwise.
 bool resident_plan(int32_t n, int bits, bool random, const hpx::Workspace* ws, ResArgs& ra) {
   const int64_t min_elems = hpx::option(hpx::kOptTerngradResidentMin);
-  if (min_elems < 0 || n < min_elems || ws->num_cus <= 0 || ws->num_cus > kBarMaxWorkgroups) return false;
+  if (min_elems < 0 || n < min_elems || resident_grid(ws) <= 0 || resident_grid(ws) > kBarMaxWorkgroups) return false;
   const int unit = (8 / bits) > 4 ? (8 / bits) : 4;
   const int h = unit / 4;
   const int64_t full_units = n / unit;
-  const int64_t per_wg = (full_units + ws->num_cus - 1) / ws->num_cus;
+  const int64_t per_wg = (full_units + resident_grid(ws) - 1) / resident_grid(ws);
   int64_t rows = (per_wg + kResThreads - 1) / kResThreads;
   if (rows < 1) rows = 1;
   const int reg_rows = res_reg_groups(bits, random) / h, lds_rows_max = kResLdsGroups / h;
@@ -1615,13 +1623,13 @@ int next_barrier_generation(hpx::Workspace* ws, hipStream_t st) {
 // mode of the first, are at most kCapLarge, and their pieces at the largest row count fit the chip.
 int resident_multi_extent(int count, const int32_t* in_sizes, const uint8_t* bitwidths, const int32_t* enable_randoms,
                           const hpx::Workspace* ws) {
-  if (ws->num_cus <= 0 || ws->num_cus > kBarMaxWorkgroups) return 0;
+  if (resident_grid(ws) <= 0 || resident_grid(ws) > kBarMaxWorkgroups) return 0;
   const int bits = bitwidths[0];
   const bool random = enable_randoms[0] != 0;
   const int unit = (8 / bits) > 4 ? (8 / bits) : 4;
   const int h = unit / 4;
   const int64_t rows_max = res_reg_groups(bits, random) / h + kResLdsGroups / h;
-  const int64_t waves = int64_t(ws->num_cus) * (kResThreads / kWave);
+  const int64_t waves = int64_t(resident_grid(ws)) * (kResThreads / kWave);
   int64_t pieces = 0;
   int k = 0;
   for (; k < count && k < kCapLarge; k++) {
@@ -1639,7 +1647,7 @@ bool resident_multi_plan(int count, const int32_t* in_sizes, const uint8_t* bitw
                          const hpx::Workspace* ws, ResMultiArgs& ma, uint32_t& pre_rows) {
   const int64_t min_elems = hpx::option(hpx::kOptTerngradResidentMin);
   if (min_elems < 0 || hpx::option(hpx::kOptTerngradResidentBucket) == 0) return false;
-  if (count < 2 || count > kCapLarge || ws->num_cus <= 0 || ws->num_cus > kBarMaxWorkgroups) return false;
+  if (count < 2 || count > kCapLarge || resident_grid(ws) <= 0 || resident_grid(ws) > kBarMaxWorkgroups) return false;
   const int bits = bitwidths[0];
   const bool random = enable_randoms[0] != 0;
   int64_t total = 0;
@@ -1651,7 +1659,7 @@ bool resident_multi_plan(int count, const int32_t* in_sizes, const uint8_t* bitw
   const int unit = (8 / bits) > 4 ? (8 / bits) : 4;
   const int h = unit / 4;
   const int reg_rows = res_reg_groups(bits, random) / h, lds_rows_max = kResLdsGroups / h;
-  const int64_t waves = int64_t(ws->num_cus) * (kResThreads / kWave);
+  const int64_t waves = int64_t(resident_grid(ws)) * (kResThreads / kWave);
   int64_t total_units = 0;
   for (int i = 0; i < count; i++) total_units += in_sizes[i] / unit;
   int64_t rows = (total_units + waves * kWave - 1) / (waves * kWave);
@@ -2050,7 +2058,7 @@ HPX_API int hpx_terngrad_encode(int count, const float* const* ins, const int32_
         ma.bar = reinterpret_cast<uint64_t*>(ws->bar);
         ma.host_flag = expired;
         ma.spin_limit = resident_spin_limit();
-        rc = launch_resident_multi(ma, bitwidths[i], enable_randoms[i] != 0, pre_rows, ws->num_cus, st);
+        rc = launch_resident_multi(ma, bitwidths[i], enable_randoms[i] != 0, pre_rows, resident_grid(ws), st);
         if (rc != HPX_OK) return rc;
         i = j;
         continue;
@@ -2075,7 +2083,7 @@ HPX_API int hpx_terngrad_encode(int count, const float* const* ins, const int32_
       ra.bar = reinterpret_cast<uint64_t*>(ws->bar);
       ra.host_flag = expired;
       ra.spin_limit = resident_spin_limit();
-      rc = launch_resident(ra, ws->num_cus, st);
+      rc = launch_resident(ra, resident_grid(ws), st);
       if (rc != HPX_OK) return rc;
     }
   }
