@@ -452,7 +452,9 @@ def x_dgc(torch, np, capi, L, stream, gen, res):
     # ---- DGC / GradDrop top-0.1 %: 138,357,544 elements --------------------------------------
     n = N_DGC
     u = torch.rand(n, device="cuda", generator=gen) - 0.5
-    g = (-1e-3 * torch.sign(u) * torch.log1p(-2 * u.abs())).float()
+    # Laplace(0, 1e-3) by inversion; |u| is kept below 1/2 (a draw of exactly 0 would otherwise become an
+    # infinite gradient, which the configuration's float64 Laplace sampler never produces)
+    g = (-1e-3 * torch.sign(u) * torch.log1p(-2 * u.abs().clamp_(max=0.5 - 2.0 ** -25))).float()
     del u
     r0 = torch.randn(n, device="cuda", generator=gen) * 1e-4
     r = r0.clone()

@@ -139,6 +139,25 @@ def test_cut_branch_many_ties(gd, oracle_cpu):
     assert np.unique(np.abs(vals)).size < 40      # ties dominate
 
 
+@pytest.mark.parametrize("ratio,bits", [(1 + 2.0**-8, 16), (1 + 2.0**-6, 18), (1.5, 22), (6.0, 26), (300.0, 27), (1e4, 28)])
+def test_cut_branch_key_widths(gd, oracle_cpu, ratio, bits):
+    # The sort of the cut branch picks its digit width and number of passes from the widest key (the distance of
+    # the largest |r| above the threshold, in fp32 bit patterns).  Sampled positions hold the smallest values, so
+    # every other element is a candidate and the cut runs; the other values spread up to `ratio` times the
+    # threshold: keys of about `bits` bits, i.e. 2 x 8, 2 x 9, 3 x 8, 3 x 9, 3 x 9 and 4 x 8 bits.
+    rng = np.random.default_rng(int(bits))
+    n, sr, dr, seed = 150_000, 0.01, 0.99, 5
+    g = np.exp(rng.uniform(np.log(1.0005), np.log(ratio), n)).astype(np.float32) * rng.choice([-1.0, 1.0], n).astype(np.float32)
+    g[np.abs(g) < 1.0005] = np.float32(1.0005)
+    sampled = np.array([oracle_cpu.gd_sample_index(seed, x, n) for x in range(1500)])
+    g[sampled] = (1.0 + 1e-4 * np.arange(1500) / 1500.0).astype(np.float32)
+    out, msg, info = _check_encode(gd, oracle_cpu, g, np.zeros(n, np.float32), sr, dr, seed)
+    kept = oracle_cpu.gd_sizes(n, sr, dr)[1]
+    assert info["candidates"] > 140_000 and info["kept"] == kept
+    top = np.abs(g).max().view(np.uint32) - np.float32(info["threshold"]).view(np.uint32)
+    assert int(top).bit_length() in (bits - 1, bits, bits + 1), (int(top).bit_length(), bits)
+
+
 def test_nothing_selected(gd, oracle_cpu):
     n = 50_000
     _check_encode(gd, oracle_cpu, np.zeros(n, np.float32), np.zeros(n, np.float32), 0.05, 0.99, 0)

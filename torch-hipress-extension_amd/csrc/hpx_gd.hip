@@ -86,6 +86,7 @@ constexpr int kSortThreads = 1024;
 constexpr int kSortPer = 8;
 constexpr int kSortTile = kSortThreads * kSortPer;   // tiles of 8192 pairs
 constexpr int kSortWaves = kSortThreads / kWave;
+constexpr int kSortBinsMax = 512;                    // bins of the widest digit the sort uses (9 bits)
 struct CutLayout {
   size_t ka, kb, ia, ib, sc, end;
 };
@@ -96,7 +97,7 @@ __host__ __device__ inline CutLayout cut_layout(uint64_t pairs) {
   c.kb = at; at += align256(sizeof(uint32_t) * size_t(pairs));
   c.ia = at; at += align256(sizeof(int32_t) * size_t(pairs));
   c.ib = at; at += align256(sizeof(int32_t) * size_t(pairs));
-  c.sc = at; at += align256(sizeof(uint32_t) * 256 * size_t(cdiv(pairs, kSortTile)));
+  c.sc = at; at += align256(sizeof(uint32_t) * kSortBinsMax * size_t(cdiv(pairs, kSortTile)));
   c.end = at;
   return c;
 }
@@ -138,25 +139,33 @@ __device__ __forceinline__ void find_digit(const uint32_t* __restrict__ hist, ui
                                            uint32_t& digit, uint32_t& rank_out) {
   constexpr int PER = BINS / kSelThreads;
   static_assert(PER >= 1, "one bin per thread at least");
-  __shared__ uint32_t s_scan[kSelThreads];
+  constexpr int kWaves = kSelThreads / kWave;
+  __shared__ uint32_t s_wave[kWaves];
   __shared__ uint32_t s_res[2];
   const int t = threadIdx.x;
+  const uint32_t lane = t & (kWave - 1), wave = t / kWave;
   uint32_t h[PER], sum = 0;
 #pragma unroll
   for (int j = 0; j < PER; j++) {
     h[j] = hist[BINS - 1 - (t * PER + j)];
     sum += h[j];
   }
-  if (t == 0) { s_res[0] = 0; s_res[1] = 0; }
-  s_scan[t] = sum;
-  __syncthreads();
-  for (int off = 1; off < kSelThreads; off <<= 1) {
-    const uint32_t v = t >= off ? s_scan[t - off] : 0u;
-    __syncthreads();
-    s_scan[t] += v;
-    __syncthreads();
+  // Inclusive prefix over the threads in order: within each wave by shuffles, then the sixteen wave totals
+  // (three workgroup barriers in all; a workgroup-wide scan through LDS, ten rounds of two barriers each, was
+  // most of the time of the launches that call this).
+  uint32_t incl = sum;
+#pragma unroll
+  for (int o = 1; o < kWave; o <<= 1) {
+    const uint32_t v = __shfl_up(incl, o, kWave);
+    if (lane >= uint32_t(o)) incl += v;
   }
-  const uint32_t excl = s_scan[t] - sum;
+  if (lane == kWave - 1) s_wave[wave] = incl;
+  if (t == 0) { s_res[0] = 0; s_res[1] = 0; }
+  __syncthreads();
+  uint32_t before = 0;
+#pragma unroll
+  for (int w = 0; w < kWaves; w++) before += uint32_t(w) < wave ? s_wave[w] : 0u;
+  const uint32_t excl = before + incl - sum;
   if (rank_in >= excl && rank_in - excl < sum) {
     uint32_t c = excl;
 #pragma unroll
@@ -508,9 +517,11 @@ __global__ __launch_bounds__(kThreads) void gd_expand_kernel(const GdArgs<CAP> a
 }
 
 // ---- cut to the `expected` largest |r| (gd_body.h:176-187) ------------------
-// Stable LSD radix sort of (key, index) pairs, 8 bits per pass, descending
-// (bin = 255 - digit).  A pass is a count launch and a scatter launch over tiles
-// of 8192 pairs (1024 lanes x 8), counts[tile * 256 + bin]; the last pass writes
+// Stable LSD radix sort of (key, index) pairs, 8 or 9 bits per pass (9 when that
+// saves a pass: keys of 25 to 27 bits, as the configuration's heavy-tailed gradient
+// gives, take three passes instead of four), descending (bin = BINS - 1 - digit).
+// A pass is a count launch and a scatter launch over tiles of 8192 pairs
+// (1024 lanes x 8), counts[tile * BINS + bin]; the last pass writes
 // the message's index block instead of a sorted list.  All tensors of a call that
 // have to be cut share these launches (a table of tensors in the kernel arguments);
 // the number of passes is that of the tensor with the largest key (a pass over a
@@ -524,7 +535,7 @@ __global__ __launch_bounds__(kThreads) void gd_expand_kernel(const GdArgs<CAP> a
 struct SortSeg {           // one tensor that is being cut; 64 bytes
   uint32_t* keys[2];       // the pass with parity p reads keys[p], idx[p] and writes keys[1 - p], idx[1 - p]
   int32_t* idx[2];
-  uint32_t* counts;        // [tile][256] of the current pass
+  uint32_t* counts;        // [tile][bins] of the current pass
   uint8_t* msg;            // the message: its index block gets the first `keep` indices from the last pass
   float* r;                // values are read from here, and cleared
   uint32_t n;              // candidates
@@ -566,10 +577,11 @@ __global__ __launch_bounds__(kThreads) void gd_gather_kernel(const SortArgs<CAP>
 }
 
 // Lanes of the wave whose `bin` equals this lane's, among the lanes in `live`.
+template <int BITS>
 __device__ __forceinline__ uint64_t match_bin(uint32_t bin, bool live) {
   uint64_t same = __ballot(live);
 #pragma unroll
-  for (int b = 0; b < 8; b++) {
+  for (int b = 0; b < BITS; b++) {
     const uint64_t m = __ballot((bin >> b) & 1u);
     same &= ((bin >> b) & 1u) ? m : ~m;
   }
@@ -579,8 +591,9 @@ __device__ __forceinline__ uint64_t match_bin(uint32_t bin, bool live) {
 // One LDS atomic per distinct bin of a wave's 64 keys, not one per key: the top
 // digit of keys that are all just above one threshold is the same for nearly all
 // of them, and 8192 atomics on one LDS word took longer than the rest of the pass.
-template <int CAP>
+template <int CAP, int BITS>
 __global__ __launch_bounds__(kSortThreads) void gd_sort_count_kernel(const SortArgs<CAP> a) {
+  constexpr uint32_t BINS = 1u << BITS;
   const int tile = blockIdx.x;
   const int s = find_segment<CAP>(a.tile_start, a.nseg, tile);
   const uint32_t* __restrict__ keys = a.seg[s].keys[a.parity];
@@ -588,10 +601,10 @@ __global__ __launch_bounds__(kSortThreads) void gd_sort_count_kernel(const SortA
   const int shift = a.shift;
   const uint32_t ltile = uint32_t(tile - a.tile_start[s]);
   uint32_t* __restrict__ counts = a.seg[s].counts;
-  __shared__ uint32_t s_hist[256];
+  __shared__ uint32_t s_hist[BINS];
   const uint32_t t = threadIdx.x;
   const uint32_t lane = t & (kWave - 1);
-  if (t < 256) s_hist[t] = 0;
+  if (t < BINS) s_hist[t] = 0;
   const uint32_t b0 = ltile * uint32_t(kSortTile);
   uint32_t key[kSortPer];
 #pragma unroll
@@ -603,12 +616,12 @@ __global__ __launch_bounds__(kSortThreads) void gd_sort_count_kernel(const SortA
 #pragma unroll
   for (int j = 0; j < kSortPer; j++) {
     const bool live = b0 + j * kSortThreads + t < n;
-    const uint32_t bin = 255u - ((key[j] >> shift) & 255u);
-    const uint64_t same = match_bin(bin, live);
+    const uint32_t bin = (BINS - 1) - ((key[j] >> shift) & (BINS - 1));
+    const uint64_t same = match_bin<BITS>(bin, live);
     if (live && (same & ((uint64_t(1) << lane) - 1)) == 0) atomicAdd(&s_hist[bin], uint32_t(__popcll(same)));
   }
   __syncthreads();
-  if (t < 256) counts[size_t(ltile) * 256 + t] = s_hist[t];
+  if (t < BINS) counts[size_t(ltile) * BINS + t] = s_hist[t];
 }
 
 // A wave owns 512 consecutive pairs of the tile and takes them 64 at a time, so
@@ -619,13 +632,15 @@ __global__ __launch_bounds__(kSortThreads) void gd_sort_count_kernel(const SortA
 // per bin within the tile; the pairs are then put in that order in LDS, so that
 // consecutive lanes write consecutive slots of a bin's run (scattering straight
 // from registers costs one address per lane and made the pass twice as long).
-template <int CAP>
+template <int CAP, int BITS>
 __global__ __launch_bounds__(kSortThreads) void gd_sort_pass_kernel(const SortArgs<CAP> a) {
+  constexpr uint32_t BINS = 1u << BITS;
+  constexpr uint32_t kBinWaves = BINS / kWave;    // waves whose lanes each look after one bin
   extern __shared__ uint32_t s_stage[];          // [kSortTile] keys, then [kSortTile] indices
-  __shared__ uint32_t s_cnt[kSortWaves][256];    // per wave: pairs per bin, then the wave's first place per bin
-  __shared__ uint32_t s_first[256];              // first place of the bin within the tile
-  __shared__ uint32_t s_slot[256];               // first global slot of the bin's pairs of this tile
-  __shared__ uint32_t s_part[8];
+  __shared__ uint32_t s_cnt[kSortWaves][BINS];   // per wave: pairs per bin, then the wave's first place per bin
+  __shared__ uint32_t s_first[BINS];             // first place of the bin within the tile
+  __shared__ uint32_t s_slot[BINS];              // first global slot of the bin's pairs of this tile
+  __shared__ uint32_t s_part[2 * kBinWaves];
   uint32_t* s_key = s_stage;
   uint32_t* s_id = s_stage + kSortTile;
   const uint32_t t = threadIdx.x;
@@ -652,14 +667,14 @@ __global__ __launch_bounds__(kSortThreads) void gd_sort_pass_kernel(const SortAr
     key[j] = x < n ? keys_in[x] : 0u;
     id[j] = x < n ? idx_in[x] : 0;
   }
-  // bin t (first 256 lanes): pairs in all tiles, in the tiles before this one, in this one.
+  // bin t (first BINS lanes): pairs in all tiles, in the tiles before this one, in this one.
   // The first 32 tiles are read with independent loads.
   uint32_t total = 0, before = 0, mine = 0;
-  if (t < 256) {
+  if (t < BINS) {
     constexpr uint32_t kFlat = 32;
     uint32_t c[kFlat];
 #pragma unroll
-    for (uint32_t q = 0; q < kFlat; q++) c[q] = q < nblk ? counts[size_t(q) * 256 + t] : 0u;
+    for (uint32_t q = 0; q < kFlat; q++) c[q] = q < nblk ? counts[size_t(q) * BINS + t] : 0u;
 #pragma unroll
     for (uint32_t q = 0; q < kFlat; q++) {
       total += c[q];
@@ -667,7 +682,7 @@ __global__ __launch_bounds__(kSortThreads) void gd_sort_pass_kernel(const SortAr
       mine += q == blk ? c[q] : 0u;
     }
     for (uint32_t q = kFlat; q < nblk; q++) {
-      const uint32_t v = counts[size_t(q) * 256 + t];
+      const uint32_t v = counts[size_t(q) * BINS + t];
       total += v;
       before += q < blk ? v : 0u;
       mine += q == blk ? v : 0u;
@@ -675,7 +690,7 @@ __global__ __launch_bounds__(kSortThreads) void gd_sort_pass_kernel(const SortAr
   }
   if (msg) {
     // Last pass: if every key has the same digit the input is already in order.
-    if (__syncthreads_or(t < 256 && total == n)) {
+    if (__syncthreads_or(t < BINS && total == n)) {
 #pragma unroll
       for (int j = 0; j < kSortPer; j++) {
         const uint32_t x = x0 + j * kWave;
@@ -685,14 +700,14 @@ __global__ __launch_bounds__(kSortThreads) void gd_sort_pass_kernel(const SortAr
     }
   }
 #pragma unroll
-  for (int q = 0; q < 256 / kWave; q++) s_cnt[wave][q * kWave + lane] = 0;  // own row: no barrier needed before use
+  for (uint32_t q = 0; q < kBinWaves; q++) s_cnt[wave][q * kWave + lane] = 0;  // own row: no barrier needed before use
 
   uint32_t place[kSortPer], bin[kSortPer];
 #pragma unroll
   for (int j = 0; j < kSortPer; j++) {
     const bool live = x0 + j * kWave < n;
-    bin[j] = 255u - ((key[j] >> a.shift) & 255u);
-    const uint64_t same = match_bin(bin[j], live);
+    bin[j] = (BINS - 1) - ((key[j] >> a.shift) & (BINS - 1));
+    const uint64_t same = match_bin<BITS>(bin[j], live);
     const uint32_t rank = __popcll(same & ((uint64_t(1) << lane) - 1));
     uint32_t base = 0;
     if (live && rank == 0) {
@@ -703,19 +718,19 @@ __global__ __launch_bounds__(kSortThreads) void gd_sort_pass_kernel(const SortAr
     place[j] = base + rank;
   }
 
-  // Exclusive scans over the 256 bins, of the global totals and of this tile's
-  // counts: within each of the first four waves, then across them.
+  // Exclusive scans over the bins, of the global totals and of this tile's
+  // counts: within each of the first BINS / 64 waves, then across them.
   uint32_t incl_g = total, incl_l = mine;
 #pragma unroll
   for (int o = 1; o < kWave; o <<= 1) {
     const uint32_t vg = __shfl_up(incl_g, o, kWave), vl = __shfl_up(incl_l, o, kWave);
     if (lane >= uint32_t(o)) { incl_g += vg; incl_l += vl; }
   }
-  if (t < 256 && lane == kWave - 1) { s_part[wave] = incl_g; s_part[4 + wave] = incl_l; }
+  if (t < BINS && lane == kWave - 1) { s_part[wave] = incl_g; s_part[kBinWaves + wave] = incl_l; }
   __syncthreads();  // also: every wave's row of s_cnt is complete
-  if (t < 256) {
+  if (t < BINS) {
     uint32_t slot = incl_g - total + before, first = incl_l - mine;
-    for (uint32_t w = 0; w < wave; w++) { slot += s_part[w]; first += s_part[4 + w]; }
+    for (uint32_t w = 0; w < wave; w++) { slot += s_part[w]; first += s_part[kBinWaves + w]; }
     s_slot[t] = slot;
     s_first[t] = first;
     uint32_t run = first;
@@ -743,7 +758,7 @@ __global__ __launch_bounds__(kSortThreads) void gd_sort_pass_kernel(const SortAr
     if (p < live_n) {
       const uint32_t k = s_key[p];
       const int32_t i = int32_t(s_id[p]);
-      const uint32_t b = 255u - ((k >> a.shift) & 255u);
+      const uint32_t b = (BINS - 1) - ((k >> a.shift) & (BINS - 1));
       const uint32_t slot = s_slot[b] + (p - s_first[b]);
       if (msg) {
         // last pass: the indices that survive the cut go straight into the message
@@ -781,14 +796,13 @@ __global__ __launch_bounds__(kThreads) void gd_scatter_kernel(const int32_t* __r
 // One tensor of the cut path as the host sees it.
 struct CutJob {
   SortSeg seg;
-  int passes;  // byte digits its largest key has
+  int bits;  // significant bits of its largest key (at least 1)
 };
 
-// The cut path for up to CAP tensors: `passes` x (count launch, scatter launch) over all of them, lowest digit
-// first, the last scatter writing the index blocks of the messages; then one gather launch that adds values
-// and headers and clears the residual entries.
-template <int CAP>
-int sort_and_cut(const CutJob* jobs, int count, hipStream_t st) {
+// The sort's launches for digits of BITS bits: `passes` x (count launch, scatter launch), lowest digit first, the
+// last scatter writing the index blocks of the messages.
+template <int CAP, int BITS>
+int sort_passes(SortArgs<CAP>& a, int passes, hipStream_t st) {
   constexpr int kStageBytes = 2 * kSortTile * int(sizeof(uint32_t));
   // The dynamic-LDS limit is a property of the function on one device: raise it once per device.
   static std::mutex attr_mu;
@@ -798,31 +812,44 @@ int sort_and_cut(const CutJob* jobs, int count, hipStream_t st) {
     HPX_HIP(hipGetDevice(&dev));
     std::lock_guard<std::mutex> g(attr_mu);
     if (dev >= 64 || !(attr_done >> dev & 1)) {
-      HPX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gd_sort_pass_kernel<CAP>),
+      HPX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&gd_sort_pass_kernel<CAP, BITS>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, kStageBytes));
       if (dev < 64) attr_done |= uint64_t(1) << dev;
     }
   }
+  const dim3 grid(uint32_t(a.tile_start[a.nseg]));
+  for (int pass = 0; pass < passes; pass++) {
+    a.shift = pass * BITS;
+    a.parity = pass & 1;
+    a.last = pass == passes - 1;
+    if (hpx::g_prof_on) hpx::prof_begin("gd_sort_count_kernel", st);
+    hipLaunchKernelGGL((gd_sort_count_kernel<CAP, BITS>), grid, dim3(kSortThreads), 0, st, a);
+    if (hpx::g_prof_on) hpx::prof_end(st);
+    if (hpx::g_prof_on) hpx::prof_begin("gd_sort_pass_kernel", st);
+    hipLaunchKernelGGL((gd_sort_pass_kernel<CAP, BITS>), grid, dim3(kSortThreads), kStageBytes, st, a);
+    if (hpx::g_prof_on) hpx::prof_end(st);
+    HPX_HIP(hipGetLastError());
+  }
+  return HPX_OK;
+}
+
+// The cut path for up to CAP tensors: the sort over all of them (as many digits as the largest key of any of
+// them has; digits of 9 bits where that takes fewer passes than bytes), then one gather launch that adds values
+// and headers and clears the residual entries.
+template <int CAP>
+int sort_and_cut(const CutJob* jobs, int count, hipStream_t st) {
   SortArgs<CAP> a;
   a.nseg = count;
-  int passes = 1;
+  int bits = 1;
   a.tile_start[0] = 0;
   for (int i = 0; i < count; i++) {
     a.seg[i] = jobs[i].seg;
     a.tile_start[i + 1] = a.tile_start[i] + int32_t(cdiv(jobs[i].seg.n, kSortTile));
-    passes = jobs[i].passes > passes ? jobs[i].passes : passes;
+    bits = jobs[i].bits > bits ? jobs[i].bits : bits;
   }
-  const dim3 grid(uint32_t(a.tile_start[count]));
-  for (int pass = 0; pass < passes; pass++) {
-    a.shift = pass * 8;
-    a.parity = pass & 1;
-    a.last = pass == passes - 1;
-    HPX_LAUNCH("gd_sort_count_kernel", gd_sort_count_kernel<CAP>, grid, dim3(kSortThreads), st, a);
-    if (hpx::g_prof_on) hpx::prof_begin("gd_sort_pass_kernel", st);
-    hipLaunchKernelGGL(gd_sort_pass_kernel<CAP>, grid, dim3(kSortThreads), kStageBytes, st, a);
-    if (hpx::g_prof_on) hpx::prof_end(st);
-    HPX_HIP(hipGetLastError());
-  }
+  const int bytes = (bits + 7) / 8, nines = (bits + 8) / 9;
+  const int rc = nines < bytes ? sort_passes<CAP, 9>(a, nines, st) : sort_passes<CAP, 8>(a, bytes, st);
+  if (rc != HPX_OK) return rc;
   for (int i = 0; i < count; i++) {
     const uint32_t k = jobs[i].seg.keep;
     a.tile_start[i + 1] = a.tile_start[i] + int32_t(cdiv(k > 0 ? k : 1, kThreads));
@@ -996,7 +1023,7 @@ int gd_encode_batch(int count, float* const* grads, const int32_t* Ns, float* co
       // keys are |r| bits minus threshold bits: the largest tells how many byte digits are in use
       const uint32_t max_key = max_bits > thr_bits ? max_bits - thr_bits : 0u;
       CutJob job;
-      job.passes = max_key >> 24 ? 4 : max_key >> 16 ? 3 : max_key >> 8 ? 2 : 1;
+      job.bits = max_key ? 32 - __builtin_clz(max_key) : 1;
       job.seg.msg = sg.out;
       job.seg.r = sg.r;
       job.seg.n = found;
