@@ -14,15 +14,17 @@
 //   stream      ONE pass over the tensor: r = g + r, store r, compare with the
 //               threshold, wave64 ballot -> one 64-bit word per 64 elements
 //               (bit i = element i), a popcount and the largest |r| per workgroup
-//   scan        two-level exclusive prefix of the per-workgroup counts; reports
-//               count, threshold and largest |r| of each tensor to the host
-//   expand      bit words -> ascending indices at the scanned offsets, values
-//               out, residual entries zeroed, header written
+//   scan        exclusive prefix of the per-workgroup counts within chunks of 4096,
+//               the chunks' totals and largest |r|
+//   expand      folds the chunk totals (each wave for itself), reports count,
+//               threshold and largest |r| of each tensor to the host; bit words ->
+//               ascending indices at the scanned offsets, values out, residual
+//               entries zeroed, header written
 //
 // The stream pass moves 12 bytes per element (g, r in; r out) plus 1/8 byte of
 // mask; everything else touches O(sample + selected) data.  The host learns the
 // candidate counts from pinned memory while the expand launch is still running
-// (it polls the words the scan launch writes; no wait for the stream), and only
+// (it polls the words the expand launch writes first; no wait for the stream), and only
 // for tensors with more than `expected` candidates queues the cut: a stable LSD
 // radix sort by |r| (ties keep ascending index) over as many byte digits as the
 // largest key has, whose last pass writes the message.  The expand launch has
@@ -49,10 +51,9 @@ constexpr int kCapLarge = 128;                   // tensors per launch table (8.
 constexpr int kCapSmall = 4;                     // calls with a few tensors pass a table of a few hundred bytes
 
 struct GdState {
-  uint32_t total;     // candidates found by the stream pass
+  uint32_t unused0;
   uint32_t thr_bits;  // threshold as fp32 bits
-  uint32_t arrive;    // arrival counter of the scan kernel's workgroups
-  uint32_t pad[61];
+  uint32_t pad[62];
 };
 constexpr int kScanChunk = 4096;   // per-tile counts scanned by one workgroup
 constexpr int kMaxChunks = 128;    // 2^31 elements / kTile / kScanChunk
@@ -190,7 +191,7 @@ __device__ __forceinline__ uint32_t sample_index(uint32_t seed, uint32_t x, uint
 }
 
 // One sample per lane: all the random gathers of the sample are in flight at
-// once.  The same launch clears the histograms and the counters of this call.
+// once.  The same launch clears the histograms of this call.
 template <int CAP>
 __global__ __launch_bounds__(kThreads) void gd_sample_kernel(const GdArgs<CAP> a) {
   const int tile = blockIdx.x;
@@ -201,10 +202,6 @@ __global__ __launch_bounds__(kThreads) void gd_sample_kernel(const GdArgs<CAP> a
   uint32_t* samples = reinterpret_cast<uint32_t*>(sg.ws + l.samples);
   const uint32_t x = uint32_t(tile - a.tile_start[s]) * kThreads + threadIdx.x;
   if (x < uint32_t(kHistWords)) hist[x] = 0;
-  if (x == 0) {
-    seg_state(sg)->total = 0;
-    seg_state(sg)->arrive = 0;
-  }
   if (x < sg.sample_cnt) {
     const uint32_t i = sample_index(sg.seed, x, sg.n);
     // with a residual: |G[i] + R[i]|, the value the update is about to store; without (dgc_body.h:18-30): |G[i]|
@@ -355,15 +352,13 @@ __global__ __launch_bounds__(kThreads) void gd_stream_kernel(const GdArgs<CAP> a
   }
 }
 
-// Exclusive prefix of the per-tile counts, two levels.  Workgroup c of a tensor scans counts
-// [c*4096, (c+1)*4096) into `off` (relative to its chunk) and publishes the chunk
-// total and the chunk's largest |r|; the last workgroup of the tensor to arrive (at most 128 of
-// them, so the shared counter costs microseconds at worst) turns the totals into chunk offsets and
-// the grand total, and reports to the host.
+// Exclusive prefix of the per-tile counts within chunks of 4096 tiles: workgroup c of a tensor scans counts
+// [c*4096, (c+1)*4096) into `off` (relative to its chunk) and leaves the chunk's total and largest |r|.
+// The second level - at most 128 chunk totals per tensor - is folded by the expand launch itself, each
+// wave for its own tiles, so no workgroup here waits for or counts the others.
 template <int CAP>
 __global__ __launch_bounds__(kSelThreads) void gd_scan_kernel(const GdArgs<CAP> a) {
   __shared__ uint32_t s_wave[kSelThreads / kWave], s_wmax[kSelThreads / kWave];
-  __shared__ uint32_t s_last;
   const int tile = blockIdx.x;
   const int s = find_segment<CAP>(a.tile_start, a.nseg, tile);
   const GdSeg& sg = a.seg[s];
@@ -373,11 +368,8 @@ __global__ __launch_bounds__(kSelThreads) void gd_scan_kernel(const GdArgs<CAP> 
   uint32_t* __restrict__ off = reinterpret_cast<uint32_t*>(sg.ws + l.off);
   uint32_t* chunk_tot = reinterpret_cast<uint32_t*>(sg.ws + l.ctot);
   uint32_t* chunk_max = reinterpret_cast<uint32_t*>(sg.ws + l.cmax);
-  uint32_t* chunk_off = reinterpret_cast<uint32_t*>(sg.ws + l.coff);
-  GdState* st = seg_state(sg);
   const uint32_t n = cdiv(sg.n, kTile);                                   // tiles of this tensor
   const uint32_t chunk = uint32_t(tile - a.tile_start[s]);
-  const uint32_t nchunks = uint32_t(a.tile_start[s + 1] - a.tile_start[s]);
   const uint32_t t = threadIdx.x, lane = t & (kWave - 1), wave = t / kWave;
   const uint32_t i0 = chunk * uint32_t(kScanChunk) + t * 4;
   uint32_t c[4], big = 0;
@@ -415,49 +407,24 @@ __global__ __launch_bounds__(kSelThreads) void gd_scan_kernel(const GdArgs<CAP> 
   if (t == 0) {
     chunk_tot[chunk] = all;
     chunk_max[chunk] = allmax;
-    __threadfence();
-    s_last = (atomicAdd(&st->arrive, 1u) == nchunks - 1);
-  }
-  __syncthreads();
-  if (!s_last) return;
-  __threadfence();
-  if (t < kWave) {
-    // up to 128 chunk totals: two per lane
-    const uint32_t a0 = (2 * t < nchunks) ? __hip_atomic_load(&chunk_tot[2 * t], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
-    const uint32_t a1 = (2 * t + 1 < nchunks) ? __hip_atomic_load(&chunk_tot[2 * t + 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
-    const uint32_t m0 = (2 * t < nchunks) ? __hip_atomic_load(&chunk_max[2 * t], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
-    const uint32_t m1 = (2 * t + 1 < nchunks) ? __hip_atomic_load(&chunk_max[2 * t + 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
-    uint32_t inc2 = a0 + a1, mm = m0 > m1 ? m0 : m1;
-#pragma unroll
-    for (int o = 1; o < kWave; o <<= 1) {
-      const uint32_t v = __shfl_up(inc2, o, kWave);
-      if (t >= uint32_t(o)) inc2 += v;
-    }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) { const uint32_t v = __shfl_xor(mm, o, kWave); mm = v > mm ? v : mm; }
-    const uint32_t ex = inc2 - a0 - a1;
-    if (2 * t < nchunks) chunk_off[2 * t] = ex;
-    if (2 * t + 1 < nchunks) chunk_off[2 * t + 1] = ex + a0;
-    if (t == kWave - 1) {
-      st->total = inc2;
-      // Pinned host words the host polls (no copy command, no wait for the stream).  The host waits for each
-      // of the three words to change, so plain system-scope stores do (a release would write the whole L2 back).
-      uint32_t* rep = a.report + size_t(s) * kReportWords;
-      __hip_atomic_store(rep + 0, inc2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-      __hip_atomic_store(rep + 1, st->thr_bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-      __hip_atomic_store(rep + 2, mm, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-    }
   }
 }
 
-// Turns the per-tile bit masks into the ascending index list, one wave per tile,
-// at the offsets the scan produced.  If the stream pass found at most `limit`
+// Turns the per-tile bit masks into the ascending index list, kExpandTiles consecutive tiles
+// per wave (their mask words, and then the values of their first candidates, are loaded
+// together: a wave with one tile spent its time waiting for one load after the other, and
+// the launch needed four rounds of such waves), at the offsets the scan produced.  Every wave
+// folds the chunk totals for itself (at most 128 of them): the offset of its tiles' chunks and the
+// tensor's candidate count; the wave of a tensor's first tile reports count, threshold and
+// largest |r| to the host.  If the stream pass found at most `limit`
 // candidates this is the finish (gd_body.h:193-229): indices, values and header
 // are written and the residual entries cleared.  If it found more, the candidates
 // and their keys (bits of |r|) go to the cut path's buffers instead and
 // nothing else is touched; more than `cap` candidates do not fit those buffers
-// and the kernel does nothing for that tensor (the host then calls it again with larger ones and
-// limit = 0).
+// and the kernel does nothing for that tensor (the host then calls it again with larger ones,
+// limit = 0 and no report).
+constexpr int kExpandTiles = 4;
+constexpr int kExpandPerBlock = (kThreads / kWave) * kExpandTiles;  // tiles per workgroup
 template <int CAP>
 __global__ __launch_bounds__(kThreads) void gd_expand_kernel(const GdArgs<CAP> a) {
   const int blk = blockIdx.x;
@@ -468,51 +435,119 @@ __global__ __launch_bounds__(kThreads) void gd_expand_kernel(const GdArgs<CAP> a
   const GdState* st = seg_state(sg);
   const uint64_t* __restrict__ masks = reinterpret_cast<const uint64_t*>(sg.ws + l.masks);
   const uint32_t* __restrict__ tile_off = reinterpret_cast<const uint32_t*>(sg.ws + l.off);
-  const uint32_t* __restrict__ chunk_off = reinterpret_cast<const uint32_t*>(sg.ws + l.coff);
+  const uint32_t* __restrict__ chunk_tot = reinterpret_cast<const uint32_t*>(sg.ws + l.ctot);
   uint8_t* __restrict__ out = sg.out;
   float* __restrict__ r = sg.r;
   const uint32_t ntiles = cdiv(sg.n, kTile);
-  const uint32_t total = st->total;
-  const bool cut = total > sg.limit;
-  if (cut && total > sg.cap) return;
+  const uint32_t nchunks = cdiv(ntiles, kScanChunk);
   const uint32_t lane = threadIdx.x & (kWave - 1);
-  const uint32_t tile = uint32_t(blk - a.tile_start[s]) * (kThreads / kWave) + threadIdx.x / kWave;
-  if (!cut && tile == 0 && lane == 0) *reinterpret_cast<int32_t*>(out) = int32_t(4 + total * 8);
-  if (tile >= ntiles) return;
-  uint64_t m = masks[size_t(tile) * kWave + lane];
-  const uint32_t c = __popcll(m);
-  uint32_t incl = c;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const uint32_t tile0 = (uint32_t(blk - a.tile_start[s]) * (kThreads / kWave) + wave) * kExpandTiles;
+
+  // the masks of this wave's tiles: requested first, used last
+  uint64_t m[kExpandTiles];
+#pragma unroll
+  for (int j = 0; j < kExpandTiles; j++) m[j] = tile0 + j < ntiles ? masks[size_t(tile0 + j) * kWave + lane] : 0ull;
+
+  // chunk totals, two per lane: inclusive prefix over the lanes
+  const uint32_t a0 = 2 * lane < nchunks ? chunk_tot[2 * lane] : 0u, a1 = 2 * lane + 1 < nchunks ? chunk_tot[2 * lane + 1] : 0u;
+  uint32_t inc2 = a0 + a1;
 #pragma unroll
   for (int o = 1; o < kWave; o <<= 1) {
-    const uint32_t v = __shfl_up(incl, o, kWave);
-    if (lane >= uint32_t(o)) incl += v;
+    const uint32_t v = __shfl_up(inc2, o, kWave);
+    if (lane >= uint32_t(o)) inc2 += v;
   }
-  uint32_t pos = chunk_off[tile / kScanChunk] + tile_off[tile] + incl - c;
-  const uint32_t e0 = tile * uint32_t(kTile) + lane * kWave;
+  const uint32_t total = __builtin_amdgcn_readlane(inc2, kWave - 1);
+  const uint32_t ex0 = inc2 - a0 - a1, ex1 = ex0 + a0;  // exclusive prefixes of chunks 2 * lane and 2 * lane + 1
+  if (tile0 == 0 && a.report != nullptr) {
+    // Pinned host words the host polls (no copy command, no wait for the stream).  The host waits for each
+    // of the three words to change, so plain system-scope stores do (a release would write the whole L2 back).
+    const uint32_t* __restrict__ chunk_max = reinterpret_cast<const uint32_t*>(sg.ws + l.cmax);
+    const uint32_t m0 = 2 * lane < nchunks ? chunk_max[2 * lane] : 0u, m1 = 2 * lane + 1 < nchunks ? chunk_max[2 * lane + 1] : 0u;
+    uint32_t mm = m0 > m1 ? m0 : m1;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) { const uint32_t v = __shfl_xor(mm, o, kWave); mm = v > mm ? v : mm; }
+    if (lane == 0) {
+      uint32_t* rep = a.report + size_t(s) * kReportWords;
+      __hip_atomic_store(rep + 0, total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      __hip_atomic_store(rep + 1, st->thr_bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      __hip_atomic_store(rep + 2, mm, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+  }
+  const bool cut = total > sg.limit;
+  if (cut && total > sg.cap) return;
+  if (!cut && tile0 == 0 && lane == 0) *reinterpret_cast<int32_t*>(out) = int32_t(4 + total * 8);
+  if (tile0 >= ntiles) return;
+
+  // first place of every tile's candidates, then of this lane's within the tile
+  uint32_t pos[kExpandTiles];
+#pragma unroll
+  for (int j = 0; j < kExpandTiles; j++) {
+    const uint32_t tile = tile0 + j < ntiles ? tile0 + j : ntiles - 1;
+    const uint32_t chunk = tile / kScanChunk;
+    const uint32_t coff = __shfl((chunk & 1u) ? ex1 : ex0, int(chunk >> 1), kWave);
+    const uint32_t c = __popcll(m[j]);
+    uint32_t incl = c;
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+      const uint32_t v = __shfl_up(incl, o, kWave);
+      if (lane >= uint32_t(o)) incl += v;
+    }
+    pos[j] = coff + tile_off[tile] + incl - c;
+  }
+  // The first candidate of each of the lane's 64-element groups: their values are loaded together.
+  uint32_t e1[kExpandTiles];
+  float v1[kExpandTiles];
+#pragma unroll
+  for (int j = 0; j < kExpandTiles; j++) {
+    e1[j] = (tile0 + j) * uint32_t(kTile) + lane * kWave + uint32_t(m[j] ? __builtin_ctzll(m[j]) : 0);
+    v1[j] = m[j] ? r[e1[j]] : 0.0f;
+  }
   if (cut) {
     int32_t* __restrict__ cand = reinterpret_cast<int32_t*>(sg.cut + cl.ia);
     uint32_t* __restrict__ keys = reinterpret_cast<uint32_t*>(sg.cut + cl.ka);
     const uint32_t thr_bits = st->thr_bits;
-    while (m) {
-      const uint32_t e = e0 + uint32_t(__builtin_ctzll(m));
-      m &= m - 1;
-      cand[pos] = int32_t(e);
-      // Sort key: distance of |r| above the threshold in fp32 bit patterns (same order as |r|;
-      // the high digits of such keys are mostly zero, which lets the sort skip its last passes).
-      keys[pos] = __float_as_uint(__builtin_fabsf(r[e])) - thr_bits;
-      pos++;
+    // Sort key: distance of |r| above the threshold in fp32 bit patterns (same order as |r|;
+    // the high digits of such keys are mostly zero, which lets the sort skip its last passes).
+#pragma unroll
+    for (int j = 0; j < kExpandTiles; j++) {
+      if (m[j]) {
+        cand[pos[j]] = int32_t(e1[j]);
+        keys[pos[j]] = __float_as_uint(__builtin_fabsf(v1[j])) - thr_bits;
+        pos[j]++;
+        m[j] &= m[j] - 1;
+      }
+      const uint32_t e0 = (tile0 + j) * uint32_t(kTile) + lane * kWave;
+      while (m[j]) {  // further candidates of the same group: rare
+        const uint32_t e = e0 + uint32_t(__builtin_ctzll(m[j]));
+        m[j] &= m[j] - 1;
+        cand[pos[j]] = int32_t(e);
+        keys[pos[j]] = __float_as_uint(__builtin_fabsf(r[e])) - thr_bits;
+        pos[j]++;
+      }
     }
     return;
   }
   int32_t* idx = reinterpret_cast<int32_t*>(out + 4);
   float* val = reinterpret_cast<float*>(out + 4 + size_t(total) * 4);
-  while (m) {
-    const uint32_t e = e0 + uint32_t(__builtin_ctzll(m));
-    m &= m - 1;
-    idx[pos] = int32_t(e);
-    val[pos] = r[e];
-    r[e] = 0.0f;
-    pos++;
+#pragma unroll
+  for (int j = 0; j < kExpandTiles; j++) {
+    if (m[j]) {
+      idx[pos[j]] = int32_t(e1[j]);
+      val[pos[j]] = v1[j];
+      r[e1[j]] = 0.0f;
+      pos[j]++;
+      m[j] &= m[j] - 1;
+    }
+    const uint32_t e0 = (tile0 + j) * uint32_t(kTile) + lane * kWave;
+    while (m[j]) {
+      const uint32_t e = e0 + uint32_t(__builtin_ctzll(m[j]));
+      m[j] &= m[j] - 1;
+      idx[pos[j]] = int32_t(e);
+      val[pos[j]] = r[e];
+      r[e] = 0.0f;
+      pos[j]++;
+    }
   }
 }
 
@@ -901,15 +936,15 @@ int launch_phases(const Plan* plans, int count, bool residual, uint32_t* report,
   HPX_HIP(hipGetLastError());
   // Queued before the host knows the counts: the finish where nothing has to be cut,
   // else the candidate list and keys of the cut path.
-  grid = tiles([](const GdSeg& sg) { return cdiv(cdiv(sg.n, kTile), kThreads / kWave); });
+  grid = tiles([](const GdSeg& sg) { return cdiv(cdiv(sg.n, kTile), kExpandPerBlock); });
   HPX_LAUNCH("gd_expand_kernel", gd_expand_kernel<CAP>, grid, dim3(kThreads), st, a);
   HPX_HIP(hipGetLastError());
   return HPX_OK;
 }
 
-// Waits until the scan launch has reported every tensor of `count` (the words are in pinned host memory and
-// the kernel writes them with system-scope stores, so they arrive while the stream is still busy with the
-// expand launch).  Polls memory; every 20 us or so it also asks whether the stream has drained, which ends the
+// Waits until the expand launch has reported every tensor of `count` (the words are in pinned host memory and
+// the kernel writes them with system-scope stores as the first thing it does, so they arrive while the stream
+// is still busy with that launch).  Polls memory; every 20 us or so it also asks whether the stream has drained, which ends the
 // wait if the words can only be seen once the kernels have finished, or if a launch failed.
 int wait_reports(volatile uint32_t* report, int count, hipStream_t st) {
   for (int t = 0; t < count; t++) {
@@ -1062,13 +1097,13 @@ int gd_encode_batch(int count, float* const* grads, const int32_t* Ns, float* co
         GdArgs<kCapSmall> a;
         a.nseg = 1;
         a.residual = residuals != nullptr;
-        a.report = const_cast<uint32_t*>(report);  // not written by this kernel
+        a.report = nullptr;  // the host has its report
         a.seg[0] = plan.seg;
         a.seg[0].cut = cut;
         a.seg[0].cap = job.seg.n;
         a.seg[0].limit = 0u;
         a.tile_start[0] = 0;
-        a.tile_start[1] = int32_t(cdiv(cdiv(plan.seg.n, kTile), kThreads / kWave));
+        a.tile_start[1] = int32_t(cdiv(cdiv(plan.seg.n, kTile), kExpandPerBlock));
         HPX_LAUNCH("gd_expand_kernel", gd_expand_kernel<kCapSmall>, dim3(uint32_t(a.tile_start[1])), dim3(kThreads), st, a);
         HPX_HIP(hipGetLastError());
       }
