@@ -36,11 +36,11 @@ N_DGC = 138_357_544
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, each scaled by what the same
 # counter reads for a plain copy of known size.
-MEASURED_TRAFFIC_BYTES = {  # profiles/terngrad_25M_pmc_fetch_write.txt (FETCH x1.99949 + WRITE x1.0, KiB -> bytes)
-    "terngrad_resident_kernel": int((50274.6 * 1.99948 + 6383.5) * 1024),
-    "terngrad_minmax_kernel": int((49946.2 * 1.99949 + 122.1) * 1024),
-    "terngrad_quant_kernel": int((49957.5 * 1.99949 + 6434.6) * 1024),
-    "terngrad_decode_kernel": int((3571.8 * 1.99948 + 99904.3) * 1024),
+MEASURED_TRAFFIC_BYTES = {  # profiles/terngrad_25M_pmc_fetch_write.txt (FETCH x1.99942 + WRITE x1.0, KiB -> bytes)
+    "terngrad_resident_kernel": int((52081.1 * 1.99942 + 8295.5) * 1024),  # includes the grid-wide exchange's polls and records
+    "terngrad_minmax_kernel": int((49939.7 * 1.99942 + 390.2) * 1024),
+    "terngrad_quant_kernel": int((49990.4 * 1.99942 + 6434.5) * 1024),
+    "terngrad_decode_kernel": int((3574.9 * 1.99942 + 99906.6) * 1024),
 }
 
 
