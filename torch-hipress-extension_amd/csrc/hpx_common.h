@@ -265,8 +265,8 @@ static_assert(kBarQuarter == kWave, "a wave's quarter is one source per lane-qua
 // generation.  A polled line has one reader and four writers; nothing is ever
 // reset (generations only grow).  With four waves at it, a wave keeps just four
 // loads in flight per round.  (Two hand-overs through group leaders - each member
-// reports to its leader, the leader to everyone - took 2.4 us against this
-// one's [see the measurements]; a counter-based barrier - fence, two dependent atomics, a release flag,
+// reports to its leader, the leader to everyone - took 2.4 us from the last
+// arrival, this takes 1.4; a counter-based barrier - fence, two dependent atomics, a release flag,
 // then reading the reduction slots - took 7 us; polling one shared word from all
 // 256 workgroups took 10.)
 __device__ __forceinline__ bool grid_exchange(uint64_t* bar, uint32_t gen, uint64_t spin_limit, uint32_t wave, uint32_t& k0, uint32_t& k1, uint32_t& k2) {

@@ -485,14 +485,14 @@ __global__ __launch_bounds__(kThreads) void terngrad_quant_kernel(const EncArgs<
 // One launch for one large tensor.  The chip's register files and LDS together
 // hold more than 128 MB, so a tensor of up to ~33M elements can stay on chip
 // between the min/max pass and the quantise pass: every workgroup (one per CU,
-// 1024 lanes) loads its contiguous share once, 24 float4 per lane into registers
+// 1024 lanes) loads its contiguous share once, up to 24 float4 per lane into registers
 // and the rest into LDS, publishes its extremes, waits at a grid-wide barrier and
 // then quantises out of registers.  The tensor is read from HBM once instead of
 // twice.
 //
-// The barrier is a two-level arrival count on monotonic counters (they are never
-// reset; launch number `gen` waits for gen * arrivals).  All workgroups of the grid
-// must be resident together, which holds because the grid is one workgroup per
+// The barrier is the exchange of hpx_common.h (records tagged with the number of
+// the launch, `gen`; nothing is ever reset).  All workgroups of the grid
+// must be resident together, which holds because the grid is at most one workgroup per
 // CU and a workgroup fits a CU by construction; other work sharing the GPU only
 // delays the barrier.  The wait is bounded by `spin_limit` ticks of the 100 MHz
 // wall clock: on expiry the workgroup raises *host_flag and leaves, so the grid
@@ -502,9 +502,6 @@ constexpr int kResRegGroups = 24;  // float4 per lane held in registers ...
 // ... except at 1 bit with stochastic rounding, whose eight draws per lane need the room.
 // Rows of prepared random addends when the LDS has room for them (8 float4 per lane).
 constexpr int res_pre_rows(int bits) { return bits == 1 ? 4 : 8; }
-// Further rows whose addends are prepared into registers, after those that go into LDS: pass 2 takes the
-// prepared rows first and gives registers back as it goes, so a few float4 per lane are free until then.
-constexpr int res_pre_reg_rows(int bits, int pre) { return (pre > 0 && bits != 1) ? 0 : 0; }
 constexpr int res_reg_groups(int bits, bool random) { return (bits == 1 && random) ? 14 : kResRegGroups; }
 constexpr int kResLdsGroups = 8;   // float4 per lane of the tensor held in LDS (128 KiB per workgroup)
 constexpr int kResLdsTotalGroups = 9;  // ... and what the workgroup may use altogether (144 KiB): the rest holds prepared draws
@@ -593,8 +590,6 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
   // workgroup whose register rows are all whole, and the others - because behind a join of the
   // two the compiler no longer knows the order of the loads and waits for all of them at once.
   float4 v[KU][H];
-  constexpr int PREG = res_pre_reg_rows(B, PRE);
-  float4 pre_reg[PREG > 0 ? PREG : 1][H];
   float4* s_pre = s_rows + size_t(a.lds_rows) * H * kResThreads;
   float mn = __builtin_inff(), mx = -__builtin_inff(), am = __builtin_inff();
   const bool whole_rows = wg_u0 + uint32_t(KU * kResThreads) <= wg_end;
@@ -628,15 +623,6 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
 #pragma unroll
         for (int h = 0; h < H; h++)
           s_pre[(k * H + h) * kResThreads + threadIdx.x] =
-              make_float4(u01_scaled(d[4 * h]), u01_scaled(d[4 * h + 1]), u01_scaled(d[4 * h + 2]), u01_scaled(d[4 * h + 3]));
-#pragma unroll
-        for (int q = 0; q < UNIT; q++) d[q] += lcg_mul(q % DPB + 2) * stride_bytes;
-      }
-#pragma unroll
-      for (int k = 0; k < PREG; k++) {
-#pragma unroll
-        for (int h = 0; h < H; h++)
-          pre_reg[k][h] =
               make_float4(u01_scaled(d[4 * h]), u01_scaled(d[4 * h + 1]), u01_scaled(d[4 * h + 2]), u01_scaled(d[4 * h + 3]));
 #pragma unroll
         for (int q = 0; q < UNIT; q++) d[q] += lcg_mul(q % DPB + 2) * stride_bytes;
@@ -724,7 +710,7 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
   uint8_t* __restrict__ pay = a.seg.out + 10;
   uint32_t draw[UNIT];
   if (RANDOM) {
-    const uint32_t x0 = a.seg.seed + u0 * BPU + uint32_t(PRE + PREG) * stride_bytes;  // first row that draws for itself
+    const uint32_t x0 = a.seg.seed + u0 * BPU + uint32_t(PRE) * stride_bytes;  // first row that draws for itself
 #pragma unroll
     for (int q = 0; q < UNIT; q++) {
       const int jb = q / DPB, j = q % DPB;
@@ -743,8 +729,6 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
 #pragma unroll
         for (int h = 0; h < H; h++) sc[h] = s_pre[(k * H + h) * kResThreads + threadIdx.x];
         packed = quant_unit_prepared<B>(v[k], sc, mn, gi);
-      } else if (RANDOM && k < PRE + PREG) {
-        packed = quant_unit_prepared<B>(v[k], pre_reg[k - PRE < 0 ? 0 : k - PRE], mn, gi);
       } else {
         packed = quant_unit<B, RANDOM>(v[k], mn, gi, draw, stride_bytes);
       }
