@@ -360,12 +360,13 @@ def x_tbq(torch, np, capi, L, stream, gen, res):
         "roofline": kernel_roofline(kt, {"tbq_encode_kernel": 12.25 * tot, "tbq_decode_kernel": 4.25 * tot})}
     # the root's gather-decode: 7 gathered messages per tensor accumulate into the tensor (hp_cuda.cpp:241-259)
     slots = 7
-    msgs7 = [[torch.randint(0, 255, ((int(s) + 3) // 4,), dtype=torch.uint8, device="cuda", generator=gen) & 0xA5
-              for s in sizes] for _ in range(slots)]
+    # the gathered messages of a tensor are the slots of its piece of the communication buffer, one after the other,
+    # as the scheduler hands them over (the library then describes a tensor's messages by a base and a distance)
+    bufs7 = [torch.randint(0, 255, (slots * ((int(s) + 3) // 4),), dtype=torch.uint8, device="cuda", generator=gen) & 0xA5 for s in sizes]
     outs7, ins7 = [], []
     for k in range(slots):
         outs7 += os_
-        ins7 += msgs7[k]
+        ins7 += [b_[k * ((int(s) + 3) // 4):(k + 1) * ((int(s) + 3) // 4)] for b_, s in zip(bufs7, sizes)]
     root = Call(L.hpx_tbq_decode, slots * len(sizes), capi.ptr_array([o.data_ptr() for o in outs7]),
                 capi.i32_array([int(s) for s in sizes] * slots), capi.ptr_array([m_.data_ptr() for m_ in ins7]),
                 capi.f32_array([1e-2] * (slots * len(sizes))), capi.i32_array([1] * (slots * len(sizes))), stream)

@@ -224,6 +224,42 @@ def test_several_messages_into_one_tensor(tbq, oracle_cpu, n):
         assert_bits_equal(host(out), ref, f"accumulated n={n} adds={adds}")
 
 
+@pytest.mark.parametrize("ntensors,slots,first_add", [(3, 7, 1), (200, 7, 1), (208, 3, 0), (209, 3, 1), (5, 32, 1), (5, 33, 1)])
+def test_messages_at_a_fixed_distance(tbq, oracle_cpu, ntensors, slots, first_add):
+    # The gathered slots of the reference's communication buffer: the messages of a tensor lie at one distance from
+    # each other and share the tensor's threshold.  Up to 208 tensors with up to 32 such messages each are one
+    # launch with a 40-byte table entry per tensor; one tensor or message more, and the call takes the general
+    # table again.  Odd slot sizes, so that messages start at any byte.
+    rng = np.random.default_rng(ntensors * 100 + slots)
+    sizes = [int(v) for v in rng.integers(1, 9000, ntensors)]
+    sizes[0] = 3 * 4096 + 1027
+    outs, refs, dms, thrs, ins, adds, souts = [], [], [], [], [], [], []
+    for t, n in enumerate(sizes):
+        thr = float(np.float32(rng.uniform(1e-3, 5e-3)))
+        slot = (n + 3) // 4 + int(rng.integers(0, 7))                      # distance between this tensor's messages
+        buf = np.zeros(slot * slots + 3, np.uint8)
+        base = rng.normal(0, 1, n).astype(np.float32)
+        ref = base.copy()
+        for k in range(slots):
+            g = rng.normal(0, 2e-3, n).astype(np.float32)
+            m = oracle_cpu.tbq_encode(g, np.zeros(n, np.float32), thr)
+            buf[1 + k * slot:1 + k * slot + m.size] = m
+            ref = oracle_cpu.tbq_decode(m, n, thr, ref, 1 if (k or first_add) else 0)
+        db = dev(buf)
+        dms.append(db)
+        out = dev(base)
+        outs.append(out); refs.append(ref)
+        for k in range(slots):
+            ins.append(db[1 + k * slot:1 + k * slot + (n + 3) // 4]); souts.append(out); thrs.append(thr)
+            adds.append(1 if (k or first_add) else 0)
+    # messages of different tensors interleaved, as the scheduler's batches hand them over: slot k of every tensor, then slot k + 1
+    order = [t * slots + k for k in range(slots) for t in range(ntensors)]
+    tbq.decode([ins[i] for i in order], [souts[i] for i in order], [thrs[i] for i in order], [adds[i] for i in order])
+    torch.cuda.synchronize()
+    for t in range(ntensors):
+        assert_bits_equal(host(outs[t]), refs[t], f"tensor {t} of {ntensors}, n={sizes[t]}, {slots} messages")
+
+
 @pytest.mark.parametrize("count", [2, 3, 5, 8, 9])
 def test_message_counts_of_the_straight_line_path(tbq, oracle_cpu, count):
     # whole tiles with 2 to 8 messages take code generated per message count; payloads start at odd addresses

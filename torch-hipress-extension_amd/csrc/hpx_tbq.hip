@@ -295,21 +295,60 @@ struct MArgs {
   MSlot slot[kMultiSlots];
 };
 static_assert(sizeof(MArgs) <= 9600, "kernel-argument budget");
+// The same for tensors whose messages lie at a fixed distance from each other, share one threshold and are all
+// added (the first one may also overwrite): the gathered slots of the reference's communication buffer
+// (hp_cuda.cpp:241-259).  A tensor then takes 40 bytes of table whatever its number of messages, and a bucket of
+// 200 tensors with 7 messages each is ONE launch instead of four.
+constexpr int kStrideSegs = 208;
+struct SSeg {
+  float* out;
+  const uint8_t* in0;  // the first message
+  int64_t stride;      // bytes from one message to the next
+  int32_t n;
+  float thr;
+  int16_t nslots;
+  int16_t add0;        // the first message is added to what the tensor holds
+  int32_t pad;
+};
+struct SArgs {
+  int32_t nseg;
+  int32_t tile_start[kStrideSegs + 1];
+  SSeg seg[kStrideSegs];
+};
+static_assert(sizeof(SSeg) == 40 && sizeof(SArgs) <= 9600, "kernel-argument budget");
 
-__global__ __launch_bounds__(kThreads) void tbq_decode_multi_kernel(const MArgs a) {
-  __shared__ const uint8_t* s_in[kMultiSlotsPerSeg];
-  __shared__ float s_thr[kMultiSlotsPerSeg];
-  __shared__ int32_t s_add[kMultiSlotsPerSeg];
-  const int tile = blockIdx.x;
-  const int s = find_segment<kMultiSegs>(a.tile_start, a.nseg, tile);
-  float* __restrict__ op = a.seg[s].out;
-  const uint32_t n = static_cast<uint32_t>(a.seg[s].n);
+// What the two tables have in common for the kernel: the tensor of a tile, and its messages in LDS.
+__device__ __forceinline__ int multi_segment(const MArgs& a, int tile) { return find_segment<kMultiSegs>(a.tile_start, a.nseg, tile); }
+__device__ __forceinline__ int multi_segment(const SArgs& a, int tile) { return find_segment<kStrideSegs>(a.tile_start, a.nseg, tile); }
+__device__ __forceinline__ int multi_slots(const MArgs& a, int s, const uint8_t** s_in, float* s_thr, int32_t* s_add) {
   const int s0 = a.seg[s].first_slot, ns = a.seg[s].nslots;
   if (int(threadIdx.x) < ns) {
     s_in[threadIdx.x] = a.slot[s0 + threadIdx.x].in;
     s_thr[threadIdx.x] = a.slot[s0 + threadIdx.x].thr;
     s_add[threadIdx.x] = a.slot[s0 + threadIdx.x].add;
   }
+  return ns;
+}
+__device__ __forceinline__ int multi_slots(const SArgs& a, int s, const uint8_t** s_in, float* s_thr, int32_t* s_add) {
+  const int ns = a.seg[s].nslots;
+  if (int(threadIdx.x) < ns) {
+    s_in[threadIdx.x] = a.seg[s].in0 + int64_t(threadIdx.x) * a.seg[s].stride;
+    s_thr[threadIdx.x] = a.seg[s].thr;
+    s_add[threadIdx.x] = threadIdx.x == 0 ? int32_t(a.seg[s].add0) : 1;
+  }
+  return ns;
+}
+
+template <typename Args>
+__global__ __launch_bounds__(kThreads) void tbq_decode_multi_kernel(const Args a) {
+  __shared__ const uint8_t* s_in[kMultiSlotsPerSeg];
+  __shared__ float s_thr[kMultiSlotsPerSeg];
+  __shared__ int32_t s_add[kMultiSlotsPerSeg];
+  const int tile = blockIdx.x;
+  const int s = multi_segment(a, tile);
+  float* __restrict__ op = a.seg[s].out;
+  const uint32_t n = static_cast<uint32_t>(a.seg[s].n);
+  const int ns = multi_slots(a, s, s_in, s_thr, s_add);
   __syncthreads();
   const bool need_old = s_add[0] != 0;
   const uint32_t full = n >> 2;
@@ -532,6 +571,42 @@ std::vector<MultiGroup> plan_multi_launch(int count, float* const* outs, const i
   return groups;
 }
 
+// Fills the table of the fixed-distance form when the whole call fits it: at most kStrideSegs tensors, every
+// tensor's messages (in call order) at one distance from each other, with one threshold, and all but the first
+// added.  Arguments have been checked.
+bool plan_strided(int count, float* const* outs, const int32_t* sizes, const uint8_t* const* ins, const float* thresholds,
+                  const int32_t* is_add_tos, SArgs& a) {
+  std::unordered_map<float*, int> index;
+  std::vector<const uint8_t*> last(kStrideSegs, nullptr);
+  a.nseg = 0;
+  for (int j = 0; j < count; j++) {
+    if (sizes[j] == 0) continue;
+    auto it = index.find(outs[j]);
+    if (it == index.end()) {
+      if (a.nseg == kStrideSegs) return false;
+      index[outs[j]] = a.nseg;
+      a.seg[a.nseg] = SSeg{outs[j], ins[j], 0, sizes[j], thresholds[j], 1, int16_t(is_add_tos[j] != 0), 0};
+      last[a.nseg] = ins[j];
+      a.nseg++;
+      continue;
+    }
+    SSeg& g = a.seg[it->second];
+    const int64_t step = ins[j] - last[it->second];
+    if (g.nslots == kMultiSlotsPerSeg || is_add_tos[j] == 0 || thresholds[j] != g.thr || sizes[j] != g.n) return false;
+    if (g.nslots == 1) g.stride = step; else if (step != g.stride) return false;
+    last[it->second] = ins[j];
+    g.nslots++;
+  }
+  int64_t tiles = 0;
+  a.tile_start[0] = 0;
+  for (int k = 0; k < a.nseg; k++) {
+    tiles += tiles_for(a.seg[k].n);
+    if (tiles > INT32_MAX) return false;
+    a.tile_start[k + 1] = int32_t(tiles);
+  }
+  return a.nseg > 0;
+}
+
 int launch_decode_multi(int count, float* const* outs, const int32_t* sizes, const uint8_t* const* ins,
                         const float* thresholds, const int32_t* is_add_tos, hipStream_t st) {
   std::vector<char> done(count, 0);
@@ -541,6 +616,15 @@ int launch_decode_multi(int count, float* const* outs, const int32_t* sizes, con
     if (sizes[j] == 0) { done[j] = 1; continue; }
     HPX_ARG(outs[j] && ins[j], "hpx_tbq_decode: tensor %d has a null pointer", j);
     left++;
+  }
+  if (left == 0) return HPX_OK;
+  {
+    SArgs sa;
+    if (plan_strided(count, outs, sizes, ins, thresholds, is_add_tos, sa)) {
+      HPX_LAUNCH("tbq_decode_multi_kernel", tbq_decode_multi_kernel<SArgs>, dim3(sa.tile_start[sa.nseg]), dim3(kThreads), st, sa);
+      HPX_HIP(hipGetLastError());
+      return HPX_OK;
+    }
   }
   MArgs a;
   while (left > 0) {
@@ -556,7 +640,7 @@ int launch_decode_multi(int count, float* const* outs, const int32_t* sizes, con
     }
     if (nslots == 0) { hpx::set_error("hpx_tbq_decode: could not place the remaining messages"); return HPX_ERR_ARG; }
     left -= nslots;
-    HPX_LAUNCH("tbq_decode_multi_kernel", tbq_decode_multi_kernel, dim3(a.tile_start[a.nseg]), dim3(kThreads), st, a);
+    HPX_LAUNCH("tbq_decode_multi_kernel", tbq_decode_multi_kernel<MArgs>, dim3(a.tile_start[a.nseg]), dim3(kThreads), st, a);
     HPX_HIP(hipGetLastError());
   }
   return HPX_OK;
