@@ -443,6 +443,36 @@ def x_terngrad_resnet50(torch, np, capi, L, stream, gen, res):
         "ms_per_step_with_the_two_launch_encode": round(sec_tiled * 1e3, 4),
         "roofline": kernel_roofline(kt, {"terngrad_resident_multi_kernel": 4.0 * N_TERNGRAD + msg_bytes,
                                          "terngrad_decode_kernel": 4.0 * N_TERNGRAD + msg_bytes})}
+    # ---- the root's gather-decode of that bucket: 7 gathered messages per tensor, the slots of the tensor's piece of
+    # the communication buffer one after the other (hp_cuda.cpp:421-439), accumulate into the 161 gradients ----
+    slots = 7
+    bufs = []
+    for m_, x_ in zip(ms_, xs):
+        nb = m_.numel()
+        b_ = torch.zeros(slots * nb, dtype=torch.uint8, device="cuda")
+        one = [b_[j * nb:(j + 1) * nb] for j in range(slots)]
+        rc = L.hpx_terngrad_encode(slots, capi.ptr_array([x_.data_ptr()] * slots), capi.i32_array([x_.numel()] * slots),
+                                   capi.ptr_array([o_.data_ptr() for o_ in one]), capi.i32_array([nb] * slots), capi.u8_array([2] * slots),
+                                   capi.i32_array([1] * slots), capi.u64_array(list(range(1, slots + 1))), stream)
+        assert rc == 0, capi.last_error()
+        bufs.append(one)
+    outs_r, ins_r, sizes_r, insz_r = [], [], [], []
+    for j in range(slots):
+        outs_r += [t_.data_ptr() for t_ in ds_]
+        ins_r += [bufs[i_][j].data_ptr() for i_ in range(k_)]
+        sizes_r += r50
+        insz_r += [t_.numel() for t_ in ms_]
+    for t_ in ds_:
+        t_.zero_()
+    root = Call(L.hpx_terngrad_decode, slots * k_, capi.ptr_array(outs_r), capi.i32_array(sizes_r), capi.ptr_array(ins_r),
+                capi.i32_array(insz_r), capi.i32_array([1] * (slots * k_)), stream)
+    sec_root = timed(torch, root, 30, 5)
+    kt_root = kernel_times(torch, capi, root, ["terngrad_decode_multi_kernel"], reps=10)
+    alg_root = (8.0 + 0.25 * slots) * N_TERNGRAD
+    res["terngrad_root_decode_add_7_messages_resnet50_161_tensors"] = {
+        "ms": round(sec_root * 1e3, 4), "algorithmic_bytes": alg_root, "frac_of_hbm_peak": round(alg_root / sec_root / 1e9 / HBM_PEAK_GBS, 4),
+        "launches_per_call": 1,
+        "roofline": kernel_roofline(kt_root, {"terngrad_decode_multi_kernel": alg_root})}
 
 
 GD_KERNELS = ["gd_sample_kernel", "gd_select_kernel", "gd_threshold_kernel", "gd_stream_kernel", "gd_scan_kernel",

@@ -223,6 +223,41 @@ def test_several_two_bit_messages_into_one_tensor(tg, oracle_cpu, n, count):
     assert tg.status() == 0
 
 
+@pytest.mark.parametrize("ntensors,slots,first_add", [(3, 7, 1), (161, 7, 1), (208, 3, 0), (209, 3, 1), (4, 32, 1), (4, 33, 1)])
+def test_messages_at_a_fixed_distance(tg, oracle_cpu, ntensors, slots, first_add):
+    # The gathered slots of the reference's communication buffer: the messages of a tensor lie at one distance from
+    # each other and have one size.  Up to 208 tensors with up to 32 such messages each are one launch with a
+    # 40-byte table entry per tensor; one tensor or message more, and the call takes the general table again.
+    rng = np.random.default_rng(ntensors * 100 + slots)
+    sizes = [int(v) for v in rng.integers(1, 9000, ntensors)]
+    sizes[0] = 5 * 16384 + 4096 + 17
+    outs, refs, keep, ins, souts, adds = [], [], [], [], [], []
+    for t, n in enumerate(sizes):
+        nb = 10 + (n + 3) // 4
+        slot = nb + int(rng.integers(0, 7))                       # distance between this tensor's messages
+        buf = np.zeros(slot * slots + 3, np.uint8)
+        base = rng.normal(0, 1, n).astype(np.float32)
+        ref = base.copy()
+        for k in range(slots):
+            x = rng.normal(0, 1e-2 * (k + 1), n).astype(np.float32)
+            rc, m = oracle_cpu.terngrad_encode(x, 2, 1, 7000 + 31 * t + k)
+            assert rc == 0 and m.size == nb
+            buf[1 + k * slot:1 + k * slot + nb] = m
+            rc, ref = oracle_cpu.terngrad_decode(m, n, ref, 1 if (k or first_add) else 0)
+        db = dev(buf)
+        keep.append(db)
+        out = dev(base)
+        outs.append(out); refs.append(ref)
+        for k in range(slots):
+            ins.append(db[1 + k * slot:1 + k * slot + nb]); souts.append(out); adds.append(1 if (k or first_add) else 0)
+    order = [t * slots + k for k in range(slots) for t in range(ntensors)]   # slot k of every tensor, then slot k + 1
+    tg.decode([ins[i] for i in order], [souts[i] for i in order], [adds[i] for i in order])
+    torch.cuda.synchronize()
+    for t in range(ntensors):
+        assert_bits_equal(host(outs[t]), refs[t], f"tensor {t} of {ntensors}, n={sizes[t]}, {slots} messages")
+    assert tg.status() == 0
+
+
 def test_many_tensors_each_with_several_messages(tg, oracle_cpu):
     rng = np.random.default_rng(78)
     sizes = [int(s) for s in np.exp(rng.uniform(np.log(5), np.log(20000), 70))]

@@ -1163,6 +1163,43 @@ struct MArgs {
   uint32_t* status;
 };
 static_assert(sizeof(MArgs) <= 9600, "kernel-argument budget");
+// The same for tensors whose messages lie at a fixed distance from each other, have one size and are all added
+// (the first one may also overwrite): the gathered slots of the reference's communication buffer
+// (hp_cuda.cpp:421-439).  A tensor then takes 40 bytes of table whatever its number of messages, and ResNet-50's
+// 161 tensors with 7 messages each are ONE launch instead of three.
+constexpr int kStrideSegs = 208;
+struct SSeg {
+  float* out;
+  const uint8_t* in0;  // the first message
+  int64_t stride;      // bytes from one message to the next
+  int32_t out_size;
+  int32_t in_size;
+  int16_t nslots;
+  int16_t add0;        // the first message is added to what the tensor holds
+  int32_t pad;
+};
+struct SArgs {
+  int32_t nseg;
+  int32_t tile_start[kStrideSegs + 1];
+  SSeg seg[kStrideSegs];
+  uint32_t* status;
+};
+static_assert(sizeof(SSeg) == 40 && sizeof(SArgs) <= 9600, "kernel-argument budget");
+// What the kernel asks of either table: the tensor of a tile, its number of messages, and message j of it.
+struct MultiMsg {
+  const uint8_t* in;
+  int32_t in_size;
+  int32_t add;
+};
+__device__ __forceinline__ int multi_segment(const MArgs& a, int tile) { return find_segment<kMultiSegs>(a.tile_start, a.nseg, tile); }
+__device__ __forceinline__ int multi_segment(const SArgs& a, int tile) { return find_segment<kStrideSegs>(a.tile_start, a.nseg, tile); }
+__device__ __forceinline__ MultiMsg multi_message(const MArgs& a, int s, int j) {
+  const MSlot& m = a.slot[a.seg[s].first_slot + j];
+  return MultiMsg{m.in, m.in_size, m.add};
+}
+__device__ __forceinline__ MultiMsg multi_message(const SArgs& a, int s, int j) {
+  return MultiMsg{a.seg[s].in0 + int64_t(j) * a.seg[s].stride, a.seg[s].in_size, j == 0 ? int32_t(a.seg[s].add0) : 1};
+}
 
 __device__ __forceinline__ uint32_t code_at(const uint8_t* __restrict__ pay, size_t i, uint32_t bits) {
   const uint32_t dpb = 8u / bits;
@@ -1257,18 +1294,20 @@ __device__ __forceinline__ uint32_t decode_two_bit_whole(float* __restrict__ op,
   return nfull;
 }
 
-__global__ __launch_bounds__(kThreads) void terngrad_decode_multi_kernel(const MArgs a) {
+template <typename Args>
+__global__ __launch_bounds__(kThreads) void terngrad_decode_multi_kernel(const Args a) {
   __shared__ float s_mn[kMultiSlotsPerSeg], s_gap[kMultiSlotsPerSeg];
   __shared__ uint32_t s_cnt[kMultiSlotsPerSeg], s_bits[kMultiSlotsPerSeg];
   __shared__ int32_t s_add[kMultiSlotsPerSeg];
   __shared__ const uint8_t* s_pay[kMultiSlotsPerSeg];
   const int tile = blockIdx.x;
-  const int s = find_segment<kMultiSegs>(a.tile_start, a.nseg, tile);
+  const int s = multi_segment(a, tile);
   float* __restrict__ op = a.seg[s].out;
-  const int s0 = a.seg[s].first_slot, ns = a.seg[s].nslots;
+  const int ns = a.seg[s].nslots;
   if (int(threadIdx.x) < ns) {
     const int j = threadIdx.x;
-    const uint8_t* in = a.slot[s0 + j].in;
+    const MultiMsg msg = multi_message(a, s, j);
+    const uint8_t* in = msg.in;
     const uint32_t bits = in[0], tail = in[1];
     uint32_t mb = 0, xb = 0;
     for (int i = 0; i < 4; i++) {
@@ -1279,7 +1318,7 @@ __global__ __launch_bounds__(kThreads) void terngrad_decode_multi_kernel(const M
     float gap = 0.f;
     if (bits == 1 || bits == 2 || bits == 4 || bits == 8) {
       gap = (__uint_as_float(xb) - __uint_as_float(mb)) / (float(1 << bits) - 1.0f);
-      int64_t c = int64_t(a.slot[s0 + j].in_size - 10) * int64_t(8 / bits) - int64_t(tail);
+      int64_t c = int64_t(msg.in_size - 10) * int64_t(8 / bits) - int64_t(tail);
       if (c > a.seg[s].out_size) c = a.seg[s].out_size;
       cnt = c > 0 ? uint32_t(c) : 0u;
     } else if (tile == a.tile_start[s]) {
@@ -1289,7 +1328,7 @@ __global__ __launch_bounds__(kThreads) void terngrad_decode_multi_kernel(const M
     s_gap[j] = gap;
     s_cnt[j] = cnt;
     s_bits[j] = cnt ? bits : 8u;
-    s_add[j] = a.slot[s0 + j].add;
+    s_add[j] = msg.add;
     s_pay[j] = in + 10;
   }
   __syncthreads();
@@ -1850,9 +1889,51 @@ int launch_decode_multi(int count, float* const* outs, const int32_t* out_sizes,
     HPX_ARG(outs[j] && ins[j], "hpx_terngrad_decode: message %d has a null pointer", j);
     left++;
   }
+  if (left == 0) return HPX_OK;
+  auto tiles_of = [](int32_t n) { return ceil_div(n, kDecTile * kMultiRep); };
+  {
+    // The fixed-distance form when the whole call fits it: at most kStrideSegs tensors, every tensor's messages (in
+    // call order) at one distance from each other, of one size, and all but the first added.
+    SArgs sa;
+    sa.status = status;
+    sa.nseg = 0;
+    std::unordered_map<float*, int> index;
+    std::vector<const uint8_t*> last(kStrideSegs, nullptr);
+    bool fits = true;
+    for (int j = 0; j < count && fits; j++) {
+      if (out_sizes[j] == 0) continue;
+      auto it = index.find(outs[j]);
+      if (it == index.end()) {
+        if (sa.nseg == kStrideSegs) { fits = false; break; }
+        index[outs[j]] = sa.nseg;
+        sa.seg[sa.nseg] = SSeg{outs[j], ins[j], 0, out_sizes[j], in_sizes[j], 1, int16_t(is_add_tos[j] != 0), 0};
+        last[sa.nseg] = ins[j];
+        sa.nseg++;
+        continue;
+      }
+      SSeg& g = sa.seg[it->second];
+      const int64_t step = ins[j] - last[it->second];
+      if (g.nslots == kMultiSlotsPerSeg || is_add_tos[j] == 0 || in_sizes[j] != g.in_size || out_sizes[j] != g.out_size) fits = false;
+      else if (g.nslots == 1) g.stride = step;
+      else if (step != g.stride) fits = false;
+      last[it->second] = ins[j];
+      g.nslots++;
+    }
+    int64_t tiles = 0;
+    sa.tile_start[0] = 0;
+    for (int k = 0; k < sa.nseg && fits; k++) {
+      tiles += tiles_of(sa.seg[k].out_size);
+      if (tiles > INT32_MAX) fits = false;
+      sa.tile_start[k + 1] = int32_t(tiles);
+    }
+    if (fits && sa.nseg > 0) {
+      HPX_LAUNCH("terngrad_decode_multi_kernel", terngrad_decode_multi_kernel<SArgs>, dim3(sa.tile_start[sa.nseg]), dim3(kThreads), st, sa);
+      HPX_HIP(hipGetLastError());
+      return HPX_OK;
+    }
+  }
   MArgs a;
   a.status = status;
-  auto tiles_of = [](int32_t n) { return ceil_div(n, kDecTile * kMultiRep); };
   while (left > 0) {
     const std::vector<MultiGroup> groups = plan_multi_launch(count, outs, out_sizes, done, tiles_of);
     a.nseg = 0;
@@ -1866,7 +1947,7 @@ int launch_decode_multi(int count, float* const* outs, const int32_t* out_sizes,
     }
     if (nslots == 0) { hpx::set_error("hpx_terngrad_decode: could not place the remaining messages"); return HPX_ERR_ARG; }
     left -= nslots;
-    HPX_LAUNCH("terngrad_decode_multi_kernel", terngrad_decode_multi_kernel, dim3(a.tile_start[a.nseg]), dim3(kThreads), st, a);
+    HPX_LAUNCH("terngrad_decode_multi_kernel", terngrad_decode_multi_kernel<MArgs>, dim3(a.tile_start[a.nseg]), dim3(kThreads), st, a);
     HPX_HIP(hipGetLastError());
   }
   return HPX_OK;
