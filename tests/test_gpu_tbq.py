@@ -260,6 +260,37 @@ def test_messages_at_a_fixed_distance(tbq, oracle_cpu, ntensors, slots, first_ad
         assert_bits_equal(host(outs[t]), refs[t], f"tensor {t} of {ntensors}, n={sizes[t]}, {slots} messages")
 
 
+@pytest.mark.parametrize("size,own", [(8, 0), (8, 1), (8, 4), (8, 7), (3, 1), (2, 0), (4, 2)])
+def test_gathered_slots_without_the_roots_own(tbq, oracle_cpu, size, own):
+    # What a root decodes (hp_cuda.cpp:241-259): the `size` slots of its piece of the communication buffer except
+    # the one of its own rank, so the messages lie at one distance with one gap; also two gaps, which the
+    # fixed-distance table does not describe and the general one takes.
+    rng = np.random.default_rng(size * 10 + own)
+    for gaps in ([own], [own, (own + 2) % size] if size >= 5 else [own]):
+        sizes = [3 * 4096 + 1027, 77, 4096, 9001]
+        keep, outs, refs, ins, souts, thrs = [], [], [], [], [], []
+        for n in sizes:
+            thr = float(np.float32(rng.uniform(1e-3, 5e-3)))
+            slot = (n + 3) // 4 + int(rng.integers(0, 5))
+            buf = np.zeros(slot * size + 2, np.uint8)
+            base = rng.normal(0, 1, n).astype(np.float32)
+            ref = base.copy()
+            for k in range(size):
+                m = oracle_cpu.tbq_encode(rng.normal(0, 2e-3, n).astype(np.float32), np.zeros(n, np.float32), thr)
+                buf[k * slot:k * slot + m.size] = m
+                if k not in gaps:
+                    ref = oracle_cpu.tbq_decode(m, n, thr, ref, 1)
+            db = dev(buf); keep.append(db)
+            out = dev(base); outs.append(out); refs.append(ref)
+            for k in range(size):
+                if k not in gaps:
+                    ins.append(db[k * slot:k * slot + (n + 3) // 4]); souts.append(out); thrs.append(thr)
+        tbq.decode(ins, souts, thrs, [1] * len(ins))
+        torch.cuda.synchronize()
+        for t in range(len(sizes)):
+            assert_bits_equal(host(outs[t]), refs[t], f"tensor {t}, {size} slots without {gaps}")
+
+
 @pytest.mark.parametrize("count", [2, 3, 5, 8, 9])
 def test_message_counts_of_the_straight_line_path(tbq, oracle_cpu, count):
     # whole tiles with 2 to 8 messages take code generated per message count; payloads start at odd addresses

@@ -258,6 +258,39 @@ def test_messages_at_a_fixed_distance(tg, oracle_cpu, ntensors, slots, first_add
     assert tg.status() == 0
 
 
+@pytest.mark.parametrize("size,own", [(8, 0), (8, 1), (8, 4), (8, 7), (3, 1), (2, 0), (4, 2)])
+def test_gathered_slots_without_the_roots_own(tg, oracle_cpu, size, own):
+    # What a root decodes (hp_cuda.cpp:421-439): the `size` slots of its piece of the communication buffer except
+    # the one of its own rank, so the messages lie at one distance with one gap; also two gaps, which the
+    # fixed-distance table does not describe and the general one takes.
+    rng = np.random.default_rng(size * 10 + own)
+    for gaps in ([own], [own, (own + 2) % size] if size >= 5 else [own]):
+        sizes = [5 * 16384 + 4096 + 17, 77, 4096, 9001]
+        keep, outs, refs, ins, souts = [], [], [], [], []
+        for t, n in enumerate(sizes):
+            nb = 10 + (n + 3) // 4
+            slot = nb + int(rng.integers(0, 5))
+            buf = np.zeros(slot * size + 2, np.uint8)
+            base = rng.normal(0, 1, n).astype(np.float32)
+            ref = base.copy()
+            for k in range(size):
+                rc, m = oracle_cpu.terngrad_encode(rng.normal(0, 1e-2 * (k + 1), n).astype(np.float32), 2, 1, 900 + 17 * t + k)
+                assert rc == 0
+                buf[k * slot:k * slot + nb] = m
+                if k not in gaps:
+                    rc, ref = oracle_cpu.terngrad_decode(m, n, ref, 1)
+            db = dev(buf); keep.append(db)
+            out = dev(base); outs.append(out); refs.append(ref)
+            for k in range(size):
+                if k not in gaps:
+                    ins.append(db[k * slot:k * slot + nb]); souts.append(out)
+        tg.decode(ins, souts, [1] * len(ins))
+        torch.cuda.synchronize()
+        for t in range(len(sizes)):
+            assert_bits_equal(host(outs[t]), refs[t], f"tensor {t}, {size} slots without {gaps}")
+    assert tg.status() == 0
+
+
 def test_many_tensors_each_with_several_messages(tg, oracle_cpu):
     rng = np.random.default_rng(78)
     sizes = [int(s) for s in np.exp(rng.uniform(np.log(5), np.log(20000), 70))]

@@ -297,7 +297,7 @@ struct MArgs {
 static_assert(sizeof(MArgs) <= 9600, "kernel-argument budget");
 // The same for tensors whose messages lie at a fixed distance from each other, share one threshold and are all
 // added (the first one may also overwrite): the gathered slots of the reference's communication buffer
-// (hp_cuda.cpp:241-259).  A tensor then takes 40 bytes of table whatever its number of messages, and a bucket of
+// (hp_cuda.cpp:241-259), of which the root leaves out its own - one gap of twice the distance is part of the form.  A tensor then takes 40 bytes of table whatever its number of messages, and a bucket of
 // 200 tensors with 7 messages each is ONE launch instead of four.
 constexpr int kStrideSegs = 208;
 struct SSeg {
@@ -308,7 +308,8 @@ struct SSeg {
   float thr;
   int16_t nslots;
   int16_t add0;        // the first message is added to what the tensor holds
-  int32_t pad;
+  int16_t skip;        // messages from this one on lie one distance further (the root's own slot is left out); -1: none
+  int16_t pad;
 };
 struct SArgs {
   int32_t nseg;
@@ -332,7 +333,8 @@ __device__ __forceinline__ int multi_slots(const MArgs& a, int s, const uint8_t*
 __device__ __forceinline__ int multi_slots(const SArgs& a, int s, const uint8_t** s_in, float* s_thr, int32_t* s_add) {
   const int ns = a.seg[s].nslots;
   if (int(threadIdx.x) < ns) {
-    s_in[threadIdx.x] = a.seg[s].in0 + int64_t(threadIdx.x) * a.seg[s].stride;
+    const int skip = a.seg[s].skip;
+    s_in[threadIdx.x] = a.seg[s].in0 + int64_t(int(threadIdx.x) + ((skip >= 0 && int(threadIdx.x) >= skip) ? 1 : 0)) * a.seg[s].stride;
     s_thr[threadIdx.x] = a.seg[s].thr;
     s_add[threadIdx.x] = threadIdx.x == 0 ? int32_t(a.seg[s].add0) : 1;
   }
@@ -585,7 +587,7 @@ bool plan_strided(int count, float* const* outs, const int32_t* sizes, const uin
     if (it == index.end()) {
       if (a.nseg == kStrideSegs) return false;
       index[outs[j]] = a.nseg;
-      a.seg[a.nseg] = SSeg{outs[j], ins[j], 0, sizes[j], thresholds[j], 1, int16_t(is_add_tos[j] != 0), 0};
+      a.seg[a.nseg] = SSeg{outs[j], ins[j], 0, sizes[j], thresholds[j], 1, int16_t(is_add_tos[j] != 0), -1, 0};
       last[a.nseg] = ins[j];
       a.nseg++;
       continue;
@@ -593,7 +595,11 @@ bool plan_strided(int count, float* const* outs, const int32_t* sizes, const uin
     SSeg& g = a.seg[it->second];
     const int64_t step = ins[j] - last[it->second];
     if (g.nslots == kMultiSlotsPerSeg || is_add_tos[j] == 0 || thresholds[j] != g.thr || sizes[j] != g.n) return false;
-    if (g.nslots == 1) g.stride = step; else if (step != g.stride) return false;
+    if (g.nslots == 1) g.stride = step;
+    else if (step == g.stride) {}
+    else if (g.skip < 0 && step == 2 * g.stride) g.skip = g.nslots;                                   // the gap
+    else if (g.skip < 0 && g.nslots == 2 && 2 * step == g.stride) { g.stride = step; g.skip = 1; }    // the gap came first
+    else return false;
     last[it->second] = ins[j];
     g.nslots++;
   }

@@ -1165,7 +1165,7 @@ struct MArgs {
 static_assert(sizeof(MArgs) <= 9600, "kernel-argument budget");
 // The same for tensors whose messages lie at a fixed distance from each other, have one size and are all added
 // (the first one may also overwrite): the gathered slots of the reference's communication buffer
-// (hp_cuda.cpp:421-439).  A tensor then takes 40 bytes of table whatever its number of messages, and ResNet-50's
+// (hp_cuda.cpp:421-439), of which the root leaves out its own - one gap of twice the distance is part of the form.  A tensor then takes 40 bytes of table whatever its number of messages, and ResNet-50's
 // 161 tensors with 7 messages each are ONE launch instead of three.
 constexpr int kStrideSegs = 208;
 struct SSeg {
@@ -1176,7 +1176,8 @@ struct SSeg {
   int32_t in_size;
   int16_t nslots;
   int16_t add0;        // the first message is added to what the tensor holds
-  int32_t pad;
+  int16_t skip;        // messages from this one on lie one distance further (the root's own slot is left out); -1: none
+  int16_t pad;
 };
 struct SArgs {
   int32_t nseg;
@@ -1198,7 +1199,9 @@ __device__ __forceinline__ MultiMsg multi_message(const MArgs& a, int s, int j) 
   return MultiMsg{m.in, m.in_size, m.add};
 }
 __device__ __forceinline__ MultiMsg multi_message(const SArgs& a, int s, int j) {
-  return MultiMsg{a.seg[s].in0 + int64_t(j) * a.seg[s].stride, a.seg[s].in_size, j == 0 ? int32_t(a.seg[s].add0) : 1};
+  const int skip = a.seg[s].skip;
+  return MultiMsg{a.seg[s].in0 + int64_t(j + ((skip >= 0 && j >= skip) ? 1 : 0)) * a.seg[s].stride, a.seg[s].in_size,
+                  j == 0 ? int32_t(a.seg[s].add0) : 1};
 }
 
 __device__ __forceinline__ uint32_t code_at(const uint8_t* __restrict__ pay, size_t i, uint32_t bits) {
@@ -1906,7 +1909,7 @@ int launch_decode_multi(int count, float* const* outs, const int32_t* out_sizes,
       if (it == index.end()) {
         if (sa.nseg == kStrideSegs) { fits = false; break; }
         index[outs[j]] = sa.nseg;
-        sa.seg[sa.nseg] = SSeg{outs[j], ins[j], 0, out_sizes[j], in_sizes[j], 1, int16_t(is_add_tos[j] != 0), 0};
+        sa.seg[sa.nseg] = SSeg{outs[j], ins[j], 0, out_sizes[j], in_sizes[j], 1, int16_t(is_add_tos[j] != 0), -1, 0};
         last[sa.nseg] = ins[j];
         sa.nseg++;
         continue;
@@ -1915,7 +1918,10 @@ int launch_decode_multi(int count, float* const* outs, const int32_t* out_sizes,
       const int64_t step = ins[j] - last[it->second];
       if (g.nslots == kMultiSlotsPerSeg || is_add_tos[j] == 0 || in_sizes[j] != g.in_size || out_sizes[j] != g.out_size) fits = false;
       else if (g.nslots == 1) g.stride = step;
-      else if (step != g.stride) fits = false;
+      else if (step == g.stride) {}
+      else if (g.skip < 0 && step == 2 * g.stride) g.skip = g.nslots;                                   // the gap
+      else if (g.skip < 0 && g.nslots == 2 && 2 * step == g.stride) { g.stride = step; g.skip = 1; }    // the gap came first
+      else fits = false;
       last[it->second] = ins[j];
       g.nslots++;
     }
