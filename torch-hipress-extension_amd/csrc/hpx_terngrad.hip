@@ -1059,17 +1059,23 @@ __device__ __forceinline__ void decode_tile(const DecSeg& sg, float mn, float ga
   const uint8_t* __restrict__ pay = sg.in + 10;
   const uint32_t g0 = tile_in_seg * uint32_t(kThreads * kDIters) + threadIdx.x;  // groups of 4 elements
   if (uint64_t(g0 - threadIdx.x + kThreads * kDIters) * 4 <= cnt) {
-    // Whole tile inside the tensor.  Each step's store is kept behind its own
-    // load (the barrier stops the compiler from batching the four stores):
-    // streaming stores issued back to back run about 35 % slower here.
+    // Whole tile inside the tensor.  All code loads of the lane are requested first (one after the other,
+    // each behind the store before it, a workgroup lived through four memory latencies and the grid was
+    // close to waiting for loads rather than for its stores); the stores then follow one per step, kept
+    // apart by the barrier (streaming stores issued back to back run about 35 % slower here).
+    uint32_t q[kDIters];
+#pragma unroll
+    for (int k = 0; k < kDIters; k++) q[k] = group_bits<B>(pay, size_t(g0 + k * kThreads) * 4);
+    float4 o[kDIters];
+    if (ADD) {
+#pragma unroll
+      for (int k = 0; k < kDIters; k++) o[k] = ld4_stream(op + size_t(g0 + k * kThreads) * 4);
+    }
 #pragma unroll
     for (int k = 0; k < kDIters; k++) {
       const size_t e = size_t(g0 + k * kThreads) * 4;
-      float4 v = group_values<B>(group_bits<B>(pay, e), gap, mn);
-      if (ADD) {
-        const float4 o = ld4_stream(op + e);
-        v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w;
-      }
+      float4 v = group_values<B>(q[k], gap, mn);
+      if (ADD) { v.x += o[k].x; v.y += o[k].y; v.z += o[k].z; v.w += o[k].w; }
       if (ADD || STREAM) st4_stream(op + e, v); else st4(op + e, v);
       __asm__ volatile("" ::: "memory");
     }
