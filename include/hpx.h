@@ -116,7 +116,10 @@ int hpx_tbq_encode(int count, const float* const* grads, const int32_t* sizes,
  * (the reference's root path decodes every gathered message into one tensor,
  * hp_cuda.cpp:241-259): they are applied in call order, and when the outputs are
  * exact duplicates all messages of a tensor are applied in a single pass over
- * it with the same sequence of fp32 additions. */
+ * it with the same sequence of fp32 additions.  (When the messages of each
+ * tensor lie at one distance from each other - the slots of a gathered buffer,
+ * with or without the one slot a root leaves out - a call with up to 208
+ * tensors is a single launch.) */
 int hpx_tbq_decode(int count, float* const* outs, const int32_t* sizes,
                    const uint8_t* const* ins, const float* thresholds,
                    const int32_t* is_add_tos, hpx_stream_t stream);
@@ -204,7 +207,9 @@ int hpx_terngrad_encode_noalloc(int count, const float* const* ins, const int32_
  * decodes to nothing and raises the sticky flag hpx_terngrad_decode_status
  * reports.  Several messages may name the same output (hp_cuda.cpp:421-439);
  * they are applied in call order, in a single pass over the tensor when the
- * outputs are exact duplicates. */
+ * outputs are exact duplicates (and a call with up to 208 tensors whose
+ * messages lie at one distance from each other is a single launch, as for
+ * hpx_tbq_decode). */
 int hpx_terngrad_decode(int count, float* const* outs, const int32_t* out_sizes,
                         const uint8_t* const* ins, const int32_t* in_sizes,
                         const int32_t* is_add_tos, hpx_stream_t stream);
