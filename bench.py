@@ -482,6 +482,9 @@ GD_KERNELS = ["gd_sample_kernel", "gd_select_kernel", "gd_threshold_kernel", "gd
 def x_dgc(torch, np, capi, L, stream, gen, res):
     # ---- DGC / GradDrop top-0.1 %: 138,357,544 elements --------------------------------------
     n = N_DGC
+    # A generator of its own: which seeds below have to sort and cut depends on the gradient drawn here (each does
+    # with probability about one half), and the section's mean should not move with what other sections drew before it.
+    gen = torch.Generator(device="cuda").manual_seed(138_357_544)
     u = torch.rand(n, device="cuda", generator=gen) - 0.5
     # Laplace(0, 1e-3) by inversion; |u| is kept below 1/2 (a draw of exactly 0 would otherwise become an
     # infinite gradient, which the configuration's float64 Laplace sampler never produces)
@@ -554,6 +557,7 @@ def x_dgc(torch, np, capi, L, stream, gen, res):
 
 def x_dgc_bucket(torch, np, capi, L, stream, gen, res):
     # ---- GradDrop over the 200-tensor bucket (110 M elements): one call against one call per tensor -------------
+    gen = torch.Generator(device="cuda").manual_seed(110_000_000)   # as above: a draw of its own
     sizes = bucket_sizes(np)
     tot = sum(sizes)
     gs = [torch.randn(s, device="cuda", generator=gen) * 5e-3 for s in sizes]
