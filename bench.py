@@ -610,8 +610,8 @@ def x_dgc_bucket(torch, np, capi, L, stream, gen, res):
         "algorithmic_bytes": 12.0 * tot, "frac_of_hbm_peak": round(12.0 * tot / sec / 1e9 / HBM_PEAK_GBS, 4),
         "kernel_us_per_launch": {k_: round(v * 1e6, 1) for k_, v in kt.items() if v},
         "launches_per_call": {k_: n_ for k_, (ms_, n_) in per_call.items() if n_},
-        # the stream pass runs once per table of 128 tensors: both launches of the call together against all its bytes
-        "roofline": {"bound": "hbm", "kernel": "gd_stream_kernel (both launches of the call)", "avg_launch_us": round(stream_s * 1e6, 2),
+        # the stream pass runs once per table of 256 tensors: all its launches of a call together against all its bytes
+        "roofline": {"bound": "hbm", "kernel": "gd_stream_kernel (all launches of the call: one per table of 256 tensors)", "avg_launch_us": round(stream_s * 1e6, 2),
                      "algorithmic_bytes": 12.0 * tot, "achieved": round(12.0 * tot / stream_s / 1e9, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(12.0 * tot / stream_s / 1e9 / HBM_PEAK_GBS, 4)}}
 

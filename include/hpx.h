@@ -234,7 +234,7 @@ int hpx_terngrad_decode_status(hpx_stream_t stream);
  * (scratch lives in the library workspace), so outs[t] needs only
  * 4 + 8*ceil(N*(1-drop)) bytes.
  * All tensors of a call go through each phase together (one launch per phase
- * for up to 128 tensors), so hand over whole buckets, as the reference's
+ * for up to 256 tensors), so hand over whole buckets, as the reference's
  * scheduler does (hp_cuda.cpp:284-301).  The reference waits for the stream
  * three times per tensor; this call never waits for the stream: it polls
  * pinned host words in which a kernel reports the candidate count of every

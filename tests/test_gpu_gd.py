@@ -198,13 +198,14 @@ def test_several_tensors_and_messages(gd, oracle_cpu):
 
 
 def test_bucket_of_ragged_tensors_in_one_call(gd, oracle_cpu, capi):
-    # The scheduler hands hpx_gd_encode whole batches (hp_cuda.cpp:284-301).  160 tensors - more than one launch
+    # The scheduler hands hpx_gd_encode whole batches (hp_cuda.cpp:284-301).  260 tensors - more than one launch
     # table holds - of ragged sizes in ONE call: every phase is one launch for a table of tensors, the host
     # learns all counts at once, and only the tensors that overshoot are sorted and cut afterwards.  Among them:
     # tensors that are cut and tensors that are not, one that selects nothing, one whose candidates are far
     # more than the space reserved for the cut, single-element and tile-edge sizes.
     rng = np.random.default_rng(60)
     sizes = [int(np.exp(rng.uniform(np.log(50), np.log(400_000)))) for _ in range(150)]
+    sizes += [int(np.exp(rng.uniform(np.log(50), np.log(20_000)))) for _ in range(100)]
     sizes += [1, 2, 4095, 4096, 4097, 8191, 65_536, 262_145, 1_000_003, 400_003]
     srs = [float(rng.choice([0.01, 0.05, 0.2, 0.5])) for _ in sizes]
     drs = [float(rng.choice([0.9, 0.99, 0.999])) for _ in sizes]
@@ -235,7 +236,7 @@ def test_bucket_of_ragged_tensors_in_one_call(gd, oracle_cpu, capi):
         stream_launches = capi.profile_query("gd_stream_kernel")[1]
     finally:
         L.hpx_profile_enable(0); L.hpx_profile_reset()
-    assert stream_launches == 2, stream_launches                  # 160 tensors: two launch tables, not 160 launches
+    assert stream_launches == 2, stream_launches                  # 260 tensors: two launch tables, not 260 launches
     cut = kept_all = 0
     for i, n in enumerate(sizes):
         r_ref = rs[i].copy()

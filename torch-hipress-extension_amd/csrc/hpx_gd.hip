@@ -47,7 +47,7 @@ constexpr int kSelThreads = 1024;
 constexpr int kSelBlocksMax = 128;               // few blocks: their bins meet in global atomics
 constexpr int kBins1 = 2048, kBins2 = 2048, kBins3 = 1024;  // key = d1:11 | d2:11 | d3:10
 constexpr int kHistWords = kBins1 + kBins2 + kBins3;
-constexpr int kCapLarge = 128;                   // tensors per launch table (8.7 KiB of kernel arguments)
+constexpr int kCapLarge = 256;                   // tensors per launch table (17 KiB of kernel arguments)
 constexpr int kCapSmall = 4;                     // calls with a few tensors pass a table of a few hundred bytes
 
 struct GdState {
@@ -129,7 +129,7 @@ struct GdArgs {
   GdSeg seg[CAP];
   uint32_t* report;             // pinned host memory, kReportWords per tensor of this table
 };
-static_assert(sizeof(GdArgs<kCapLarge>) <= 9600, "kernel-argument budget");
+static_assert(sizeof(GdArgs<kCapLarge>) <= 18000, "kernel-argument budget");
 
 __device__ __forceinline__ GdState* seg_state(const GdSeg& sg) { return reinterpret_cast<GdState*>(sg.ws); }
 
@@ -586,7 +586,7 @@ struct SortArgs {
   int32_t tile_start[CAP + 1];
   SortSeg seg[CAP];
 };
-static_assert(sizeof(SortArgs<kCapLarge>) <= 9600, "kernel-argument budget");
+static_assert(sizeof(SortArgs<kCapLarge>) <= 18000, "kernel-argument budget");
 
 // generate_S_value, gd_body.h:80-99, plus the header (gd_body.h:193-201), for
 // messages whose k indices are already in place (the cut path).  A launch of its

@@ -593,7 +593,7 @@ bool plan_strided(int count, float* const* outs, const int32_t* sizes, const uin
       continue;
     }
     SSeg& g = a.seg[it->second];
-    const int64_t step = ins[j] - last[it->second];
+    const int64_t step = static_cast<int64_t>(reinterpret_cast<intptr_t>(ins[j]) - reinterpret_cast<intptr_t>(last[it->second]));  // addresses, not elements of one array
     if (g.nslots == kMultiSlotsPerSeg || is_add_tos[j] == 0 || thresholds[j] != g.thr || sizes[j] != g.n) return false;
     if (g.nslots == 1) g.stride = step;
     else if (step == g.stride) {}

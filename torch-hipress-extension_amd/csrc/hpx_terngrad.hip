@@ -1921,7 +1921,7 @@ int launch_decode_multi(int count, float* const* outs, const int32_t* out_sizes,
         continue;
       }
       SSeg& g = sa.seg[it->second];
-      const int64_t step = ins[j] - last[it->second];
+      const int64_t step = static_cast<int64_t>(reinterpret_cast<intptr_t>(ins[j]) - reinterpret_cast<intptr_t>(last[it->second]));  // addresses, not elements of one array
       if (g.nslots == kMultiSlotsPerSeg || is_add_tos[j] == 0 || in_sizes[j] != g.in_size || out_sizes[j] != g.out_size) fits = false;
       else if (g.nslots == 1) g.stride = step;
       else if (step == g.stride) {}
