@@ -84,8 +84,8 @@ __host__ __device__ inline GdLayout gd_layout(uint32_t n, uint32_t sample_cnt) {
 }
 // The cut path's buffers for up to `pairs` candidates: two copies of keys and indices, and the sort's counts.
 constexpr int kSortThreads = 1024;
-constexpr int kSortPer = 8;
-constexpr int kSortTile = kSortThreads * kSortPer;   // tiles of 8192 pairs
+constexpr int kSortPer = 4;
+constexpr int kSortTile = kSortThreads * kSortPer;   // tiles of 4096 pairs (8192: each launch of a pass 3 us longer)
 constexpr int kSortWaves = kSortThreads / kWave;
 constexpr int kSortBinsMax = 512;                    // bins of the widest digit the sort uses (9 bits)
 struct CutLayout {
@@ -555,8 +555,8 @@ __global__ __launch_bounds__(kThreads) void gd_expand_kernel(const GdArgs<CAP> a
 // Stable LSD radix sort of (key, index) pairs, 8 or 9 bits per pass (9 when that
 // saves a pass: keys of 25 to 27 bits, as the configuration's heavy-tailed gradient
 // gives, take three passes instead of four), descending (bin = BINS - 1 - digit).
-// A pass is a count launch and a scatter launch over tiles of 8192 pairs
-// (1024 lanes x 8), counts[tile * BINS + bin]; the last pass writes
+// A pass is a count launch and a scatter launch over tiles of 4096 pairs
+// (1024 lanes x 4), counts[tile * BINS + bin]; the last pass writes
 // the message's index block instead of a sorted list.  All tensors of a call that
 // have to be cut share these launches (a table of tensors in the kernel arguments);
 // the number of passes is that of the tensor with the largest key (a pass over a
@@ -659,7 +659,7 @@ __global__ __launch_bounds__(kSortThreads) void gd_sort_count_kernel(const SortA
   if (t < BINS) counts[size_t(ltile) * BINS + t] = s_hist[t];
 }
 
-// A wave owns 512 consecutive pairs of the tile and takes them 64 at a time, so
+// A wave owns 256 consecutive pairs of the tile and takes them 64 at a time, so
 // the order wave, round, lane is the input order and equal digits keep it.  Per
 // round the lanes of a wave that share a bin are found with ballots; the wave
 // keeps its own running count per bin in its row of s_cnt (no workgroup barrier
@@ -703,10 +703,10 @@ __global__ __launch_bounds__(kSortThreads) void gd_sort_pass_kernel(const SortAr
     id[j] = x < n ? idx_in[x] : 0;
   }
   // bin t (first BINS lanes): pairs in all tiles, in the tiles before this one, in this one.
-  // The first 32 tiles are read with independent loads.
+  // The first 40 tiles (163,840 pairs) are read with independent loads.
   uint32_t total = 0, before = 0, mine = 0;
   if (t < BINS) {
-    constexpr uint32_t kFlat = 32;
+    constexpr uint32_t kFlat = 40;
     uint32_t c[kFlat];
 #pragma unroll
     for (uint32_t q = 0; q < kFlat; q++) c[q] = q < nblk ? counts[size_t(q) * BINS + t] : 0u;
