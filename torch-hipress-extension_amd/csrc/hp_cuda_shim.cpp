@@ -35,7 +35,7 @@ SHIM_API void hp_cuda_terngradr(std::vector<float*>& out_floats, std::vector<int
   int ret = hpx_terngrad_decode(static_cast<int>(out_floats.size()), out_floats.data(), out_float_sizes.data(),
                                 cptrs(in_uint8_ts), in_uint8_t_sizes.data(), adds.data(), stream);
   // The reference parses the header on the host and fails there; here the check
-  // ran on the device, so ask for its verdict (waits for the stream, as the
+  // ran on the device, so ask for its result (waits for the stream, as the
   // reference's own header copy does, terngrad_body.h:334-340).
   if (!ret) ret = hpx_terngrad_decode_status(stream);
   if (ret) printf("ret=%d %s\n", ret, hpx_last_error());  // hp_cuda_kernel.cu:229
