@@ -256,6 +256,40 @@ def test_bucket_of_ragged_tensors_in_one_call(gd, oracle_cpu, capi):
     assert cut >= 10 and kept_all >= 10, (cut, kept_all)
 
 
+def test_more_tensors_than_one_round_of_reports(gd, oracle_cpu):
+    # The host learns the candidate counts from a block of pinned words that holds 4092 tensors' reports; a call
+    # with more tensors goes through the phases, the wait and the cut once per such round (and through seventeen
+    # launch tables).  4200 small tensors as views of one buffer, both branches among them.
+    rng = np.random.default_rng(62)
+    count = 4200
+    sizes = [int(x) for x in rng.integers(40, 400, count)]
+    starts = np.concatenate([[0], np.cumsum(sizes)])
+    g_all = rng.laplace(0, 1e-3, int(starts[-1])).astype(np.float32)
+    r_all = rng.normal(0, 1e-4, int(starts[-1])).astype(np.float32)
+    dg_all, dr_all = dev(g_all), dev(r_all)
+    dgs = [dg_all[starts[i]:starts[i + 1]] for i in range(count)]
+    drs_ = [dr_all[starts[i]:starts[i + 1]] for i in range(count)]
+    obytes = [(_out_bytes(n, 0.9) + 3) // 4 * 4 for n in sizes]
+    ostarts = np.concatenate([[0], np.cumsum(obytes)])
+    out_all = torch.full((int(ostarts[-1]),), 0xEE, dtype=torch.uint8, device="cuda")
+    outs = [out_all[ostarts[i]:ostarts[i + 1]] for i in range(count)]
+    seeds = [int(x) for x in rng.integers(0, 2**63, count)]
+    gd.encode(dgs, drs_, outs, [0.5] * count, [0.9] * count, seeds)
+    torch.cuda.synchronize()
+    got_all, r_got = host(out_all), host(dr_all)
+    assert_bits_equal(host(dg_all), g_all, "gradients untouched")
+    cut = 0
+    for i, n in enumerate(sizes):
+        r_ref = r_all[starts[i]:starts[i + 1]].copy()
+        msg, info = oracle_cpu.gd_encode(g_all[starts[i]:starts[i + 1]], r_ref, 0.5, 0.9, seeds[i])
+        got = got_all[ostarts[i]:ostarts[i + 1]]
+        assert_bits_equal(got[:msg.size], msg, f"message[{i}] n={n} info={info}")
+        assert np.all(got[_out_bytes(n, 0.9):] == 0xEE), f"tensor {i}: wrote past its message"
+        assert_bits_equal(r_got[starts[i]:starts[i + 1]], r_ref, f"residual[{i}]")
+        cut += info["candidates"] > info["kept"]
+    assert 100 < cut < count - 100, cut
+
+
 def test_bad_tensor_in_a_bucket_is_reported_and_skipped(gd, oracle_cpu):
     # like the reference driver, which prints and goes on (hp_cuda_kernel.cu:90-92): the call returns the failure,
     # the other tensors are encoded
