@@ -85,7 +85,7 @@ def timed(torch, fn, steps, warmup):
 
 
 def kernel_times(torch, capi, fn, names, reps=10):
-    """Average duration (s) of each named kernel, HIP events on the launch stream."""
+    """Average duration (s) of each named kernel: HIP events attached to each launch on its stream (begin and end of the kernel itself)."""
     L = capi.load()
     torch.cuda.synchronize()
     L.hpx_profile_reset()

@@ -87,11 +87,13 @@ int hpx_get_option(const char* name, int64_t* value);
 
 /* ---- measurement aid ------------------------------------------------------
  * No counterpart in the reference.  While enabled, every kernel the library
- * launches is bracketed by a pair of HIP events recorded on the stream of the
- * launch; hpx_profile_query waits for them and returns the summed duration and
- * the number of launches of the kernel with that name (e.g.
+ * launches carries a pair of HIP events that take the kernel's own begin and
+ * end times on the stream of the launch (hipExtLaunchKernelGGL), so the
+ * durations are those a kernel trace shows, without the hand-over between
+ * launches; hpx_profile_query waits for them and returns the summed duration
+ * and the number of launches of the kernel with that name (e.g.
  * "terngrad_decode_kernel").  hpx_profile_reset forgets what was recorded.
- * Off by default; enabling it inserts events between kernels. */
+ * Off by default. */
 int hpx_profile_enable(int on);
 int hpx_profile_reset(void);
 int hpx_profile_query(const char* kernel, double* total_ms, int64_t* launches);

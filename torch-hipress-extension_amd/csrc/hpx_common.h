@@ -1,6 +1,7 @@
 // Shared host/device helpers of the hpx kernel library (gfx950, wave64).
 #pragma once
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
 
 #include <mutex>
@@ -35,17 +36,25 @@ void clear_error();
 
 // ---- per-kernel timing (measurement aid, off by default) ---------------------
 extern bool g_prof_on;
-void prof_begin(const char* name, hipStream_t st);
-void prof_end(hipStream_t st);
+// A new record under `name` and its two events, not yet recorded.
+void prof_events(const char* name, hipEvent_t* start, hipEvent_t* stop);
 
-// Every kernel goes out through this macro so that hpx_profile_* can bracket it
-// with HIP events on the stream it is launched on.
-#define HPX_LAUNCH(NAME, KERNEL, GRID, BLOCK, STREAM, ...)            \
-  do {                                                                \
-    if (hpx::g_prof_on) hpx::prof_begin(NAME, STREAM);                \
-    hipLaunchKernelGGL(KERNEL, GRID, BLOCK, 0, STREAM, __VA_ARGS__);  \
-    if (hpx::g_prof_on) hpx::prof_end(STREAM);                        \
+// Every kernel goes out through these macros.  With hpx_profile_enable(1) a launch carries two HIP events that
+// take the kernel's own begin and end times (hipExtLaunchKernelGGL), so hpx_profile_query reports the durations a
+// kernel trace shows; events recorded on the stream around a launch would add the hand-over between launches
+// (1-2 us) to every kernel.
+#define HPX_LAUNCH_LDS(NAME, PROF, KERNEL, GRID, BLOCK, LDS, STREAM, ...)                        \
+  do {                                                                                           \
+    if (PROF) {                                                                                  \
+      hipEvent_t hpx_e0_ = nullptr, hpx_e1_ = nullptr;                                           \
+      hpx::prof_events(NAME, &hpx_e0_, &hpx_e1_);                                                \
+      hipExtLaunchKernelGGL(KERNEL, GRID, BLOCK, LDS, STREAM, hpx_e0_, hpx_e1_, 0, __VA_ARGS__); \
+    } else {                                                                                     \
+      hipLaunchKernelGGL(KERNEL, GRID, BLOCK, LDS, STREAM, __VA_ARGS__);                         \
+    }                                                                                            \
   } while (0)
+#define HPX_LAUNCH(NAME, KERNEL, GRID, BLOCK, STREAM, ...) \
+  HPX_LAUNCH_LDS(NAME, hpx::g_prof_on, KERNEL, GRID, BLOCK, 0, STREAM, __VA_ARGS__)
 
 // ---- per-(device, stream) workspace ----------------------------------------
 // `dev` is grow-only scratch whose contents are meaningless between calls.

@@ -857,12 +857,8 @@ int sort_passes(SortArgs<CAP>& a, int passes, hipStream_t st) {
     a.shift = pass * BITS;
     a.parity = pass & 1;
     a.last = pass == passes - 1;
-    if (hpx::g_prof_on) hpx::prof_begin("gd_sort_count_kernel", st);
-    hipLaunchKernelGGL((gd_sort_count_kernel<CAP, BITS>), grid, dim3(kSortThreads), 0, st, a);
-    if (hpx::g_prof_on) hpx::prof_end(st);
-    if (hpx::g_prof_on) hpx::prof_begin("gd_sort_pass_kernel", st);
-    hipLaunchKernelGGL((gd_sort_pass_kernel<CAP, BITS>), grid, dim3(kSortThreads), kStageBytes, st, a);
-    if (hpx::g_prof_on) hpx::prof_end(st);
+    HPX_LAUNCH("gd_sort_count_kernel", (gd_sort_count_kernel<CAP, BITS>), grid, dim3(kSortThreads), st, a);
+    HPX_LAUNCH_LDS("gd_sort_pass_kernel", hpx::g_prof_on, (gd_sort_pass_kernel<CAP, BITS>), grid, dim3(kSortThreads), kStageBytes, st, a);
     HPX_HIP(hipGetLastError());
   }
   return HPX_OK;

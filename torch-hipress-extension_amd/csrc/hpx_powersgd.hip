@@ -567,9 +567,7 @@ HPX_API int hpx_powersgd_encode2(int count, float* const* Ps, const float* const
       const size_t lds = size_t(max_nr) * sizeof(float);
       HPX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(psgd_orth_lds_kernel),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, int(lds)));
-      if (hpx::g_prof_on) hpx::prof_begin("psgd_orth_kernel", st);
-      hipLaunchKernelGGL(psgd_orth_lds_kernel, dim3(a.nseg), dim3(kOrthThreads), lds, st, a);
-      if (hpx::g_prof_on) hpx::prof_end(st);
+      HPX_LAUNCH_LDS("psgd_orth_kernel", hpx::g_prof_on, psgd_orth_lds_kernel, dim3(a.nseg), dim3(kOrthThreads), lds, st, a);
     } else {
       HPX_LAUNCH("psgd_orth_kernel", psgd_orth_kernel, dim3(a.nseg), dim3(kOrthThreads), st, a);
     }

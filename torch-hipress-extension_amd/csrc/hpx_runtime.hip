@@ -101,15 +101,12 @@ hipEvent_t prof_event() {
 }
 }  // namespace
 
-void prof_begin(const char* name, hipStream_t st) {
+void prof_events(const char* name, hipEvent_t* start, hipEvent_t* stop) {
   std::lock_guard<std::mutex> g(g_prof_mu);
   ProfRec r{name, prof_event(), prof_event()};
-  (void)hipEventRecord(r.start, st);
   g_prof_recs.push_back(r);
-}
-void prof_end(hipStream_t st) {
-  std::lock_guard<std::mutex> g(g_prof_mu);
-  if (!g_prof_recs.empty()) (void)hipEventRecord(g_prof_recs.back().stop, st);
+  *start = r.start;
+  *stop = r.stop;
 }
 
 int ensure_slots(Workspace* ws, size_t words) {

@@ -1617,9 +1617,8 @@ int launch_resident_as(const ResArgs& ra, int num_cus, hipStream_t st) {
     }
   }
   const size_t lds = size_t(ra.lds_rows + PRE) * H * kResThreads * sizeof(float4);
-  if (hpx::g_prof_on) hpx::prof_begin("terngrad_resident_kernel", st);
-  hipLaunchKernelGGL((terngrad_resident_kernel<B, RANDOM, PRE>), dim3(num_cus), dim3(kResThreads), lds, st, ra);
-  if (hpx::g_prof_on) hpx::prof_end(st);
+  HPX_LAUNCH_LDS("terngrad_resident_kernel", hpx::g_prof_on, (terngrad_resident_kernel<B, RANDOM, PRE>), dim3(num_cus),
+                 dim3(kResThreads), lds, st, ra);
   HPX_HIP(hipGetLastError());
   return HPX_OK;
 }
@@ -1738,9 +1737,8 @@ int launch_resident_multi_as(const ResMultiArgs& ma, int num_cus, hipStream_t st
     }
   }
   const size_t lds = size_t(ma.lds_rows + PRE) * H * kResThreads * sizeof(float4);
-  if (hpx::g_prof_on) hpx::prof_begin("terngrad_resident_multi_kernel", st);
-  hipLaunchKernelGGL((terngrad_resident_multi_kernel<B, RANDOM, PRE>), dim3(num_cus), dim3(kResThreads), lds, st, ma);
-  if (hpx::g_prof_on) hpx::prof_end(st);
+  HPX_LAUNCH_LDS("terngrad_resident_multi_kernel", hpx::g_prof_on, (terngrad_resident_multi_kernel<B, RANDOM, PRE>),
+                 dim3(num_cus), dim3(kResThreads), lds, st, ma);
   HPX_HIP(hipGetLastError());
   return HPX_OK;
 }
@@ -1802,14 +1800,10 @@ int launch_encode(int count, const float* const* ins, const int32_t* in_sizes, u
       a.nseg++;
       i++;
     }
-    if (prof) hpx::prof_begin("terngrad_minmax_kernel", st);
-    hipLaunchKernelGGL(terngrad_minmax_kernel<CAP>, dim3(a.tile_start[a.nseg]), dim3(kThreads), 0, st, a);
-    if (prof) hpx::prof_end(st);
+    HPX_LAUNCH_LDS("terngrad_minmax_kernel", prof, terngrad_minmax_kernel<CAP>, dim3(a.tile_start[a.nseg]), dim3(kThreads), 0, st, a);
     HPX_HIP(hipGetLastError());
     for (int k = 0; k <= a.nseg; k++) a.tile_start[k] = qstart[k];
-    if (prof) hpx::prof_begin("terngrad_quant_kernel", st);
-    hipLaunchKernelGGL(terngrad_quant_kernel<CAP>, dim3(a.tile_start[a.nseg]), dim3(kThreads), 0, st, a);
-    if (prof) hpx::prof_end(st);
+    HPX_LAUNCH_LDS("terngrad_quant_kernel", prof, terngrad_quant_kernel<CAP>, dim3(a.tile_start[a.nseg]), dim3(kThreads), 0, st, a);
     HPX_HIP(hipGetLastError());
   }
   return HPX_OK;
