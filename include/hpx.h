@@ -93,7 +93,8 @@ int hpx_get_option(const char* name, int64_t* value);
  * launches; hpx_profile_query waits for them and returns the summed duration
  * and the number of launches of the kernel with that name (e.g.
  * "terngrad_decode_kernel").  hpx_profile_reset forgets what was recorded.
- * Off by default. */
+ * Off by default; leave it off while a stream is being captured into a graph
+ * (a launch with events is not something a graph can record). */
 int hpx_profile_enable(int on);
 int hpx_profile_reset(void);
 int hpx_profile_query(const char* kernel, double* total_ms, int64_t* launches);
