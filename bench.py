@@ -218,12 +218,14 @@ def main():
 
 def plain_streams(torch, stream, n):
     """What the memory system gives the simplest kernels of the codecs' shapes (bench_probe.hip, built beside this
-    file; not part of the product library), measured the way the headline is: buffers rotate over distinct sets,
-    events on the launch stream around each kernel.  The TernGrad step reads 4*n bytes once and writes 4*n bytes
-    once, so read + write of 4*n bytes is the time below which no encode+decode of this tensor can go on this part."""
+    file; not part of the product library), measured the way the headline's kernels are: buffers rotate over
+    distinct sets, every launch carries a pair of events that take the kernel's own begin and end.  The TernGrad
+    step reads 4*n bytes once and writes 4*n bytes once, so read + write of 4*n bytes is the kernel time below which
+    no encode+decode of this tensor can go on this part."""
     import __graft_entry__
     probe = C.CDLL(__graft_entry__.BENCH_PROBE)
-    probe.bench_probe_stream.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]
+    probe.bench_probe_stream_timed.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_int]
+    probe.bench_probe_elapsed_us.restype = C.c_double
     names = {0: "read", 1: "write_streaming", 2: "write_plain", 3: "read_read_write"}
     out = {}
     for label, elems, nsets in (("headline_tensor", n, 6), ("440MB", 110_000_000, 3)):
@@ -234,22 +236,21 @@ def plain_streams(torch, stream, n):
         for kind, name in names.items():
             i = [0]
 
-            def f():
+            def f(slot=-1):
                 i[0] += 1
-                rc = probe.bench_probe_stream(kind, a[i[0] % nsets].data_ptr(), b.data_ptr(), nbytes, stream)
+                rc = probe.bench_probe_stream_timed(kind, a[i[0] % nsets].data_ptr(), b.data_ptr(), nbytes, stream, slot)
                 assert rc == 0, rc
 
             for _ in range(2 * nsets):   # untimed: clocks up, the zero fill's dirty lines out of the caches
                 f()
             reps = 24
-            evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
             torch.cuda.synchronize()
-            for e0, e1 in evs:           # the launches go out on torch's current stream, which `stream` is
-                e0.record()
-                f()
-                e1.record()
+            for r in range(reps):        # back to back; every launch carries its own pair of events
+                f(r)
             torch.cuda.synchronize()
-            kt = sum(e0.elapsed_time(e1) for e0, e1 in evs) / reps * 1e-3
+            us = [probe.bench_probe_elapsed_us(r) for r in range(reps)]
+            assert min(us) > 0, us
+            kt = sum(us) / reps * 1e-6
             traffic = nbytes * (3 if kind == 3 else 1)
             res[name] = {"us": round(kt * 1e6, 2), "GBps": round(traffic / kt / 1e9, 1),
                          "frac_of_hbm_peak": round(traffic / kt / 1e9 / HBM_PEAK_GBS, 4)}

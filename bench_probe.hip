@@ -7,7 +7,10 @@
 //   kind 3  a = a + b over `bytes` each  (read, read, write in place; non-temporal)
 // a and b are device pointers, 16-byte aligned; bytes is rounded down to a multiple of 16 KiB.
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
+
+#include <vector>
 
 namespace {
 constexpr int kWave = 64;
@@ -57,10 +60,27 @@ __global__ __launch_bounds__(kThreads) void probe_stream_kernel(float* __restric
 }
 }  // namespace
 
-// 0 on success, -3 for a bad argument, -2 for a HIP error.
-extern "C" __attribute__((visibility("default"))) int bench_probe_stream(int kind, void* a, const void* b, int64_t bytes,
-                                                                        void* stream) {
-  if (kind < 0 || kind > 3 || !a || (kind == 3 && !b)) return -3;
+namespace {
+// Event pairs for timed launches: a launch carries its pair, which takes the kernel's own begin and end times
+// (the way the library's hpx_profile_* measures its kernels), not the hand-over between launches.
+std::vector<hipEvent_t> g_events;
+bool event_pair(int slot, hipEvent_t* e0, hipEvent_t* e1) {
+  while (g_events.size() < size_t(2 * slot + 2)) {
+    hipEvent_t e = nullptr;
+    if (hipEventCreate(&e) != hipSuccess) return false;
+    g_events.push_back(e);
+  }
+  *e0 = g_events[2 * slot];
+  *e1 = g_events[2 * slot + 1];
+  return true;
+}
+}  // namespace
+
+// 0 on success, -3 for a bad argument, -2 for a HIP error.  slot < 0: an ordinary launch; slot >= 0: the launch
+// carries event pair `slot`, read back with bench_probe_elapsed_us once the stream has drained.
+extern "C" __attribute__((visibility("default"))) int bench_probe_stream_timed(int kind, void* a, const void* b,
+                                                                              int64_t bytes, void* stream, int slot) {
+  if (kind < 0 || kind > 3 || !a || (kind == 3 && !b) || slot > 4095) return -3;
   if ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15) return -3;
   constexpr int64_t kTile = int64_t(kThreads) * kIters * 16;
   const int64_t tiles = bytes / kTile;
@@ -69,11 +89,31 @@ extern "C" __attribute__((visibility("default"))) int bench_probe_stream(int kin
   float* fa = static_cast<float*>(a);
   const float* fb = static_cast<const float*>(b);
   const dim3 grid(static_cast<uint32_t>(tiles)), block(kThreads);
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  if (slot >= 0 && !event_pair(slot, &e0, &e1)) return -2;
+#define PROBE_LAUNCH(K)                                                                              \
+  if (slot >= 0) hipExtLaunchKernelGGL(probe_stream_kernel<K>, grid, block, 0, st, e0, e1, 0, fa, fb); \
+  else hipLaunchKernelGGL(probe_stream_kernel<K>, grid, block, 0, st, fa, fb)
   switch (kind) {
-    case 0: hipLaunchKernelGGL(probe_stream_kernel<0>, grid, block, 0, st, fa, fb); break;
-    case 1: hipLaunchKernelGGL(probe_stream_kernel<1>, grid, block, 0, st, fa, fb); break;
-    case 2: hipLaunchKernelGGL(probe_stream_kernel<2>, grid, block, 0, st, fa, fb); break;
-    default: hipLaunchKernelGGL(probe_stream_kernel<3>, grid, block, 0, st, fa, fb); break;
+    case 0: PROBE_LAUNCH(0); break;
+    case 1: PROBE_LAUNCH(1); break;
+    case 2: PROBE_LAUNCH(2); break;
+    default: PROBE_LAUNCH(3); break;
   }
+#undef PROBE_LAUNCH
   return hipGetLastError() == hipSuccess ? 0 : -2;
+}
+
+extern "C" __attribute__((visibility("default"))) int bench_probe_stream(int kind, void* a, const void* b, int64_t bytes,
+                                                                        void* stream) {
+  return bench_probe_stream_timed(kind, a, b, bytes, stream, -1);
+}
+
+// Duration of the launch that carried event pair `slot`, in microseconds; negative on failure.
+extern "C" __attribute__((visibility("default"))) double bench_probe_elapsed_us(int slot) {
+  if (slot < 0 || size_t(2 * slot + 1) >= g_events.size()) return -1.0;
+  float ms = 0.f;
+  if (hipEventSynchronize(g_events[2 * slot + 1]) != hipSuccess) return -1.0;
+  if (hipEventElapsedTime(&ms, g_events[2 * slot], g_events[2 * slot + 1]) != hipSuccess) return -1.0;
+  return double(ms) * 1e3;
 }
