@@ -127,6 +127,22 @@ def test_ragged_shapes_ranks_and_padding(psgd):
         _run_case(psgd, [shape], rng)
 
 
+@pytest.mark.parametrize("seed", [11, 12])
+def test_random_batches_of_shapes(psgd, seed):
+    # batches of 1 ... 12 matrices with random n, m (1 ... 1500, log-uniform), rank 1 ... 16 (never above min(n, m)) and
+    # padding, two iterations each now and then
+    rng = np.random.default_rng(seed)
+    for it in range(12):
+        shapes = []
+        for _ in range(int(rng.integers(1, 13))):
+            n = int(np.exp(rng.uniform(0, np.log(1500))))
+            m = int(np.exp(rng.uniform(0, np.log(1500))))
+            r = int(rng.integers(1, min(16, n, m) + 1))
+            pad = int(rng.integers(0, min(m, 13))) if rng.integers(0, 2) else 0
+            shapes.append((n, m, r, min(pad, n * m - 1)))
+        _run_case(psgd, shapes, rng, iterations=2 if it % 4 == 0 else 1)
+
+
 def test_two_iterations_exercise_error_feedback(psgd):
     rng = np.random.default_rng(2)
     _run_case(psgd, [(256, 512, 4, 0), (512, 256, 4, 0), (300, 300, 4, 9)], rng, iterations=2)
