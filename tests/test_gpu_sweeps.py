@@ -158,3 +158,48 @@ def test_decode_calls_with_random_message_layouts(capi, oracle_cpu, seed):
         torch.cuda.synchronize()
         for t in range(ntens):
             assert_bits_equal(host(outs[t]), refs[t], f"call {it} ({codec}, {ntens} tensors x {nslot} messages, layout {layout}, order {order_mode}) tensor {t}")
+
+
+@pytest.mark.parametrize("seed", [1, 2])
+def test_tbq_calls_with_random_buckets(capi, oracle_cpu, seed):
+    # hpx_tbq_encode / hpx_tbq_decode over buckets of 1 ... 700 tensors that start at any element of their buffers,
+    # thresholds per tensor (zero and negative ones among them, which the reference accepts: tbq_body.h:70-84),
+    # residuals carried over a second step, decode written or added.
+    rng = np.random.default_rng(seed)
+    tbq = Tbq(capi)
+    for it in range(20):
+        count = int(np.exp(rng.uniform(0, np.log(700))))
+        hi = 3_000_000 if count < 20 else 100_000 if count < 200 else 10_000
+        sizes = [int(np.exp(rng.uniform(0, np.log(hi)))) for _ in range(count)]
+        offs = [int(rng.integers(0, 9)) for _ in sizes]
+        thrs = [float(np.float32(rng.choice([2e-3, 1e-3, 5e-2, 0.0, -1e-3]))) for _ in sizes]
+        span = [n + 16 for n in sizes]
+        starts = np.concatenate([[0], np.cumsum(span)])
+        g_all, r_all, o_all = (torch.zeros(int(starts[-1]), device="cuda") for _ in range(3))
+        view = lambda buf: [buf[starts[i] + offs[i]:starts[i] + offs[i] + sizes[i]] for i in range(count)]
+        dg, dr, do = view(g_all), view(r_all), view(o_all)
+        rs = [rng.normal(0, 1e-3, n).astype(np.float32) for n in sizes]
+        for a, b in zip(dr, rs):
+            a.copy_(dev(b))
+        for step in range(2):
+            gs = [rng.normal(0, 2e-3, n).astype(np.float32) for n in sizes]
+            bases = [rng.normal(0, 1, n).astype(np.float32) for n in sizes]
+            adds = [int(rng.integers(0, 2)) for _ in sizes]
+            for a, b in zip(dg, gs):
+                a.copy_(dev(b))
+            for a, b in zip(do, bases):
+                a.copy_(dev(b))
+            packed = tbq.encode(dg, dr, thrs)
+            tbq.decode(packed, do, thrs, adds)
+            torch.cuda.synchronize()
+            for i, n in enumerate(sizes):
+                what = f"call {it} step {step} tensor {i}: n={n} offset={offs[i]} thr={thrs[i]} add={adds[i]}"
+                pr = oracle_cpu.tbq_encode(gs[i], rs[i], thrs[i])          # rs[i] is updated in place: the next step's residual
+                assert_bits_equal(host(packed[i]), pr, "codes, " + what)
+                assert_bits_equal(host(dr[i]), rs[i], "residual, " + what)
+                assert_bits_equal(host(do[i]), oracle_cpu.tbq_decode(pr, n, thrs[i], bases[i].copy(), adds[i]), "decoded, " + what)
+        inside = np.zeros(int(starts[-1]), bool)
+        for i, n in enumerate(sizes):
+            inside[starts[i] + offs[i]:starts[i] + offs[i] + n] = True
+        for name, buf in (("gradients", g_all), ("residuals", r_all), ("decoded tensors", o_all)):
+            assert not host(buf)[~inside].any(), f"call {it}: wrote between the {name}"
