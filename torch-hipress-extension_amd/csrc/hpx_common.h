@@ -176,13 +176,19 @@ __device__ __forceinline__ void st4_stream(float* p, float4 v) {
   __builtin_nontemporal_store(v.w, &q->w);
 }
 
-// Output policy of the write-only decoders.  A pure write stream that fits the
-// 256 MB Infinity Cache would otherwise finish with its lines dirty in the cache
-// and leave the write-back to whichever kernel runs next; the streaming store
-// makes the decoder pay for its own traffic at no cost to itself.  Past that
-// size the write-back happens inside the kernel anyway and the plain store is
-// measurably faster.
-constexpr size_t kStreamStoreMaxBytes = size_t(128) << 20;
+// Output policy of the write-only decoders: streaming (non-temporal) stores whatever the size of the output.  A
+// pure write stream that fits the 256 MB Infinity Cache would otherwise finish with its lines dirty in the cache
+// and leave the write-back to whichever kernel runs next; a larger one is simply written faster (110 M elements:
+// 73 us against 91 with plain stores in the TernGrad decode, 73 against 85 in TBQ's).  The option stays for
+// callers whose next kernel reads the decoded tensor straight back.
+constexpr size_t kStreamStoreMaxBytes = size_t(1) << 62;
+// A write stream of streaming stores runs faster with few workgroups per CU (their stores then reach memory as a
+// compact front): launches of the write-mode decoders ask for this much LDS they never touch, which holds a CU to
+// three (52 KiB) or four (40 KiB) workgroups of 256 lanes.  TBQ decode of 110 M elements: 73 -> 62 us at three
+// (66 at four, 80 at two); TernGrad decode: 73 -> 65 us at four (72 at three).  Kernels that also read what they
+// write (the add-mode decoders, the encoders' in-place residual update, GradDrop's stream pass) gain nothing.
+constexpr int kWriteStreamPadLds3 = 52 * 1024;
+constexpr int kWriteStreamPadLds4 = 40 * 1024;
 // The limit in force: option "stream_store_max_bytes".
 size_t stream_store_max_bytes();
 

@@ -1821,6 +1821,7 @@ int launch_decode(int count, float* const* outs, const int32_t* out_sizes, const
   while (i < count) {
     a.nseg = 0;
     a.tile_start[0] = 0;
+    bool any_add = false;
     while (i < count && a.nseg < CAP) {
       HPX_ARG(out_sizes[i] >= 0 && in_sizes[i] >= 10, "hpx_terngrad_decode: message %d: out_size %d, in_size %d", i,
               out_sizes[i], in_sizes[i]);
@@ -1829,13 +1830,16 @@ int launch_decode(int count, float* const* outs, const int32_t* out_sizes, const
         const int32_t t = ceil_div(out_sizes[i], kDecTile);
         if (int64_t(a.tile_start[a.nseg]) + t > INT32_MAX) break;
         a.seg[a.nseg] = DecSeg{outs[i], ins[i], out_sizes[i], in_sizes[i], is_add_tos[i] != 0, 0};
+        any_add = any_add || is_add_tos[i] != 0;
         a.tile_start[a.nseg + 1] = a.tile_start[a.nseg] + t;
         a.nseg++;
       }
       i++;
     }
     if (a.nseg == 0) continue;
-    HPX_LAUNCH("terngrad_decode_kernel", terngrad_decode_kernel<CAP>, dim3(a.tile_start[a.nseg]), dim3(kThreads), st, a);
+    // write mode throughout: a pure write stream, held to four workgroups per CU (hpx_common.h)
+    const int pad = (a.stream_store && !any_add) ? hpx::kWriteStreamPadLds4 : 0;
+    HPX_LAUNCH_LDS("terngrad_decode_kernel", hpx::g_prof_on, terngrad_decode_kernel<CAP>, dim3(a.tile_start[a.nseg]), dim3(kThreads), pad, st, a);
     HPX_HIP(hipGetLastError());
   }
   return HPX_OK;
