@@ -187,6 +187,7 @@ constexpr size_t kStreamStoreMaxBytes = size_t(1) << 62;
 // three (52 KiB) or four (40 KiB) workgroups of 256 lanes.  TBQ decode of 110 M elements: 73 -> 62 us at three
 // (66 at four, 80 at two); TernGrad decode: 73 -> 65 us at four (72 at three).  Kernels that also read what they
 // write (the add-mode decoders, the encoders' in-place residual update, GradDrop's stream pass) gain nothing.
+constexpr int kWriteStreamPadLds2 = 64 * 1024;  // two per CU: the PowerSGD decode (one read, three writes: 792 -> 755 us)
 constexpr int kWriteStreamPadLds3 = 52 * 1024;
 constexpr int kWriteStreamPadLds4 = 40 * 1024;
 // The limit in force: option "stream_store_max_bytes".

@@ -807,11 +807,13 @@ __global__ __launch_bounds__(kSortThreads) void gd_sort_pass_kernel(const SortAr
 }
 
 // ---- decode -----------------------------------------------------------------
+// The fill of a written tensor is a pure write stream: streaming stores, three workgroups per CU (hpx_common.h;
+// 138 M elements: 119 -> 95 us for the whole call, 103 without the limit on the workgroups).
 __global__ __launch_bounds__(kThreads) void gd_zero_kernel(float* __restrict__ out, uint32_t n) {
   const uint32_t stride = gridDim.x * kThreads * 4;
   for (uint32_t e = (blockIdx.x * kThreads + threadIdx.x) * 4; e < n; e += stride) {
     if (n - e >= 4) {
-      st4(out + e, make_float4(0.f, 0.f, 0.f, 0.f));
+      st4_stream(out + e, make_float4(0.f, 0.f, 0.f, 0.f));
     } else {
       for (uint32_t i = e; i < n; i++) out[i] = 0.f;
     }
@@ -1179,7 +1181,7 @@ int decode_messages(int count, const uint8_t* const* ins, const int32_t* in_size
       const uint32_t n = static_cast<uint32_t>(out_sizes[i]);
       if (n && zero_fill) {
         uint32_t blocks = cdiv(n, kThreads * 4);
-        HPX_LAUNCH("gd_zero_kernel", gd_zero_kernel, dim3(blocks), dim3(kThreads), st, outs[i], n);
+        HPX_LAUNCH_LDS("gd_zero_kernel", hpx::g_prof_on, gd_zero_kernel, dim3(blocks), dim3(kThreads), hpx::kWriteStreamPadLds3, st, outs[i], n);
       }
       if (k) HPX_LAUNCH("gd_scatter_kernel", gd_scatter_kernel<false>, dim3(cdiv(k, kThreads)), dim3(kThreads), st, idx, val, k, outs[i]);
     } else if (k) {

@@ -470,13 +470,14 @@ int check_dims(const char* who, const Batch& b, int* max_cg) {
   return HPX_OK;
 }
 
-#define PSGD_LAUNCH_CG(KERNEL, cg, grid, st, args)                                              \
-  switch (cg) {                                                                                 \
-    case 1: HPX_LAUNCH(#KERNEL, KERNEL<1>, dim3(grid), dim3(kThreads), st, args); break;      \
-    case 2: HPX_LAUNCH(#KERNEL, KERNEL<2>, dim3(grid), dim3(kThreads), st, args); break;      \
-    case 3: HPX_LAUNCH(#KERNEL, KERNEL<3>, dim3(grid), dim3(kThreads), st, args); break;      \
-    default: HPX_LAUNCH(#KERNEL, KERNEL<4>, dim3(grid), dim3(kThreads), st, args); break;     \
+#define PSGD_LAUNCH_CG_LDS(KERNEL, cg, grid, lds, st, args)                                                         \
+  switch (cg) {                                                                                                     \
+    case 1: HPX_LAUNCH_LDS(#KERNEL, hpx::g_prof_on, KERNEL<1>, dim3(grid), dim3(kThreads), lds, st, args); break;  \
+    case 2: HPX_LAUNCH_LDS(#KERNEL, hpx::g_prof_on, KERNEL<2>, dim3(grid), dim3(kThreads), lds, st, args); break;  \
+    case 3: HPX_LAUNCH_LDS(#KERNEL, hpx::g_prof_on, KERNEL<3>, dim3(grid), dim3(kThreads), lds, st, args); break;  \
+    default: HPX_LAUNCH_LDS(#KERNEL, hpx::g_prof_on, KERNEL<4>, dim3(grid), dim3(kThreads), lds, st, args); break; \
   }
+#define PSGD_LAUNCH_CG(KERNEL, cg, grid, st, args) PSGD_LAUNCH_CG_LDS(KERNEL, cg, grid, 0, st, args)
 
 }  // namespace
 
@@ -611,7 +612,9 @@ HPX_API int hpx_powersgd_decode(int count, const float* const* Ps, const float* 
       a.nseg++;
       i++;
     }
-    PSGD_LAUNCH_CG(psgd_decode_kernel, cg, a.tile_start[a.nseg], st, a);
+    // One read and three writes per element: held to two workgroups per CU (LDS the kernel never touches,
+    // hpx_common.h), the 36 matrices of the configuration decode in 755 us instead of 792 (three per CU: 776).
+    PSGD_LAUNCH_CG_LDS(psgd_decode_kernel, cg, a.tile_start[a.nseg], hpx::kWriteStreamPadLds2, st, a);
     HPX_HIP(hipGetLastError());
   }
   return HPX_OK;
