@@ -63,7 +63,9 @@ int hpx_release_stream(hpx_stream_t stream);
  * variable HPX_<NAME IN CAPITALS> when that is set, else from its default, and
  * can be changed at any time (it applies to calls made afterwards):
  *   "stream_store_max_bytes"  total output size up to which the write-only
- *                             decoders use streaming stores (default 128 MiB)
+ *                             decoders use streaming stores (default: no
+ *                             limit; lower it if the next kernel reads the
+ *                             decoded tensor straight back)
  *   "terngrad_resident_min"   smallest tensor, in elements, that
  *                             hpx_terngrad_encode sends through its
  *                             single-launch resident kernel (default 5 * 2^20,
