@@ -83,6 +83,12 @@ int hpx_release_stream(hpx_stream_t stream);
  *                             that may only use some of the CUs (a CU mask)
  *                             must set it to that number: the workgroups of a
  *                             resident launch wait for each other
+ *   "clock_seed"              what an encoder uses when it is called with
+ *                             seeds == NULL; negative (default): the wall
+ *                             clock, as the reference's bodies
+ *                             (terngrad_body.h:247-251, gd_body.h:138-140).
+ *                             Lets the C++ drivers, whose signatures carry no
+ *                             seed, produce reproducible messages
  * Unknown names return HPX_ERR_ARG. */
 int hpx_set_option(const char* name, int64_t value);
 int hpx_get_option(const char* name, int64_t* value);
@@ -174,16 +180,21 @@ int hpx_terngrad_encode(int count, const float* const* ins, const int32_t* in_si
                         const uint8_t* bitwidths, const int32_t* enable_randoms,
                         const uint64_t* seeds, hpx_stream_t stream);
 
-/* The completion contract of hp_cuda_terngrad (hp_cuda_kernel.cu:30-65 returns
- * only once terngrad_body has synchronised and the message is complete,
- * terngrad_body.h:195, :273).  Returns 0 at once if no grid-barrier launch of
- * hpx_terngrad_encode is outstanding on `stream` (the two-launch path cannot
- * fail).  Otherwise waits for the stream; if a barrier wait expired, encodes the
- * tensors of those launches again through the two-launch path on the same
- * stream and waits for that too.  On return 0 every message of every
- * hpx_terngrad_encode call made on the stream so far is valid; -2 if the repair
- * itself failed.  hpx_terngrad_repaired counts the tensors ever encoded again
- * on the stream (a diagnostic). */
+/* One half of the completion contract of hp_cuda_terngrad (hp_cuda_kernel.cu:30-65
+ * returns only once terngrad_body has synchronised after its last quantise
+ * launch, terngrad_body.h:285, so every message is complete and the reference's
+ * scheduler reads it on another stream at once, hp_cuda.cpp:464-468).  This call
+ * settles the launches that meet at a grid barrier, the only ones that can leave
+ * a message unwritten: it returns 0 at once if none is outstanding on `stream`
+ * - it does NOT wait for two-launch encodes, which cannot fail but may still be
+ * queued or running; a caller that needs them finished waits for the stream
+ * itself, as the C++ driver hp_cuda_terngrad (csrc/hp_cuda_shim.cpp) does after
+ * this call.  Otherwise it waits for the stream; if a barrier wait expired, it
+ * encodes the tensors of those launches again through the two-launch path on
+ * the same stream and waits for that too.  On return 0 no message of any
+ * hpx_terngrad_encode call made on the stream so far will be left unwritten;
+ * -2 if the repair itself failed.  hpx_terngrad_repaired counts the tensors
+ * ever encoded again on the stream (a diagnostic). */
 int hpx_terngrad_encode_status(hpx_stream_t stream);
 int64_t hpx_terngrad_repaired(hpx_stream_t stream);
 
@@ -195,7 +206,11 @@ int64_t hpx_terngrad_repaired(hpx_stream_t stream);
  * hipMalloc / hipFree, takes no workspace, never waits for the stream and puts
  * no per-call tag into its kernels (it clears the slots it uses with a small
  * kernel first), which also makes it recordable into a graph (seeds == NULL then
- * freezes the clock value of the capture).  Limits: at most 192 tensors per call
+ * freezes the clock value of the capture: every replay rounds with the same
+ * draws).  The first call on a device looks up the array's address
+ * (hipGetDevice, hipGetSymbolAddress), which a capture in a non-relaxed mode
+ * does not allow: make one eager call per device - any size - before capturing.
+ * Limits: at most 192 tensors per call
  * (-3 beyond that).  Every call on a GPU shares that GPU's array: calls that
  * overlap in time on one GPU - on any streams - race; order them. */
 int hpx_terngrad_encode_noalloc(int count, const float* const* ins, const int32_t* in_sizes,

@@ -155,3 +155,163 @@ def test_powersgd_drivers_equal_the_c_abi_path(drv, pkg):
         for i in range(len(shapes)):
             assert_bits_equal(host(a[i]).ravel(), host(b[i]).ravel(), f"{what}[{i}]")
     del gen
+
+
+# ---- the drivers used the way the reference's scheduler uses them ---------------------------------------------
+# hp_cuda.cpp runs a driver on one pool stream and consumes its output on ANOTHER pool stream straight afterwards,
+# with no event between the two (TernGrad: driver on the compute stream, `C.copy_(B)` on the data stream,
+# hp_cuda.cpp:464-468; GradDrop: hp_cuda_gdr on the compute stream, hp_cuda_gd over the same root tensors on the
+# null stream, then the copies on the data stream, hp_cuda.cpp:284-313; pool streams are non-blocking, so the null
+# stream orders nothing either).  That only works because the reference's drivers return with their work done
+# (terngrad_body.h:285, gd_body.h:161,201,313).  The tests below repeat those sequences on torch's pool streams
+# (non-blocking, as the reference's) and hold the result to the oracle bit for bit; the option "clock_seed" stands
+# in for the wall clock the drivers seed from.
+
+@pytest.fixture()
+def fixed_clock(capi):
+    old = capi.set_option("clock_seed", 77)
+    yield 77
+    capi.set_option("clock_seed", old)
+
+
+def _pinned_like(t):
+    return torch.empty(t.shape, dtype=t.dtype, pin_memory=True)
+
+
+@pytest.mark.parametrize("resident", [False, True])
+def test_terngrad_message_is_complete_for_a_consumer_on_another_stream(drv, oracle_cpu, capi, fixed_clock, resident):
+    rng = np.random.default_rng(50)
+    ns = [20_000_003, 18_000_000, 16_000_001] if not resident else [25_557_032]
+    xs = [rng.normal(0, 1e-2, n).astype(np.float32) for n in ns]
+    old = capi.set_option("terngrad_resident_min", (5 << 20) if resident else -1)   # -1: every tensor takes two launches
+    try:
+        dx = [dev(x) for x in xs]
+        Bs = [torch.full((oracle_cpu.terngrad_packed_size(n, 2),), 0x5A, dtype=torch.uint8, device="cuda") for n in ns]
+        Cs = [_pinned_like(b) for b in Bs]
+        compute, data = torch.cuda.Stream(), torch.cuda.Stream()
+        torch.cuda.synchronize()
+        with torch.cuda.stream(compute):
+            drv.hp_cuda_terngrad(dx, Bs, [2] * len(ns), [1] * len(ns))
+        with torch.cuda.stream(data):                       # hp_cuda.cpp:466-468, no event, no wait in between
+            for b, c in zip(Bs, Cs):
+                c.copy_(b, non_blocking=True)
+        data.synchronize()                                   # hp_cuda.cpp:485
+        for i, x in enumerate(xs):
+            rc, ref = oracle_cpu.terngrad_encode(x, 2, 1, fixed_clock)
+            assert rc == 0
+            assert_bits_equal(Cs[i].numpy(), ref, f"message[{i}] as the data stream saw it")
+    finally:
+        capi.set_option("terngrad_resident_min", old)
+        torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("drop_ratio", [0.999, 0.99])
+def test_graddrop_batch_is_complete_for_a_consumer_on_another_stream(drv, oracle_cpu, fixed_clock, drop_ratio):
+    # one call over a batch on the null stream (hp_cuda.cpp:292-301), B -> C on the data stream (:304-315); over
+    # the seeds and sizes below some tensors overshoot `expected` and are cut, others are not (asserted at the end)
+    rng = np.random.default_rng(51)
+    ns, sr = [9_000_001, 7_000_000, 3_000_003, 1_200_000, 600_000], 0.01
+    gs = [rng.laplace(0, 1e-3, n).astype(np.float32) for n in ns]
+    rs = [rng.normal(0, 1e-4, n).astype(np.float32) for n in ns]
+    dg, dres = [dev(g) for g in gs], [dev(r) for r in rs]
+    sizes = [4 + 8 * oracle_cpu.gd_sizes(n, sr, drop_ratio)[1] for n in ns]
+    Bs = [torch.full((s,), 0xEE, dtype=torch.uint8, device="cuda") for s in sizes]
+    Cs = [_pinned_like(b) for b in Bs]
+    data = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(torch.cuda.default_stream()):
+        drv.hp_cuda_gd(dg, dres, Bs, [sr] * len(ns), [drop_ratio] * len(ns))
+    with torch.cuda.stream(data):
+        for b, c in zip(Bs, Cs):
+            c.copy_(b, non_blocking=True)
+        res_seen = [r.clone() for r in dres]
+    data.synchronize()
+    cut = []
+    for i, n in enumerate(ns):
+        r_ref = rs[i].copy()
+        msg, info = oracle_cpu.gd_encode(gs[i], r_ref, sr, drop_ratio, fixed_clock)
+        assert_bits_equal(Cs[i].numpy()[:msg.size], msg, f"message[{i}] as the data stream saw it")
+        assert_bits_equal(host(res_seen[i]), r_ref, f"residual[{i}] as the data stream saw it")
+        cut.append(info["candidates"] > info["kept"])
+    assert any(cut) and not all(cut), cut                   # the batch holds both branches
+
+
+def test_graddrop_root_decode_then_encode_on_different_streams(drv, oracle_cpu, fixed_clock):
+    # A root task: hp_cuda_gdr adds the gathered messages into the gradient on the compute stream, hp_cuda_gd encodes
+    # that gradient on the null stream, the message is copied out on the data stream (hp_cuda.cpp:241-259, 284-313).
+    rng = np.random.default_rng(52)
+    n, sr, dr_ = 12_000_001, 0.01, 0.999
+    expected = oracle_cpu.gd_sizes(n, sr, dr_)[1]
+    grad = rng.laplace(0, 1e-3, n).astype(np.float32)
+    res = rng.normal(0, 1e-4, n).astype(np.float32)
+    peers = []
+    for p in range(3):                                       # three gathered slots from other ranks
+        gp = rng.laplace(0, 1e-3, n).astype(np.float32)
+        rp = np.zeros(n, np.float32)
+        m, _ = oracle_cpu.gd_encode(gp, rp, sr, dr_, 1000 + p)
+        peers.append(m)
+    dgrad, dres = dev(grad), dev(res)
+    dmsgs = [dev(m) for m in peers]
+    B = torch.full((4 + 8 * expected,), 0xEE, dtype=torch.uint8, device="cuda")
+    C = _pinned_like(B)
+    compute, data = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(compute):
+        drv.hp_cuda_gdr(dmsgs, [m.size for m in peers], [dgrad] * 3, [1, 1, 1])
+    with torch.cuda.stream(torch.cuda.default_stream()):
+        drv.hp_cuda_gd([dgrad], [dres], [B], [sr], [dr_])
+    with torch.cuda.stream(data):
+        C.copy_(B, non_blocking=True)
+    data.synchronize()
+    want = grad.copy()
+    for m in peers:
+        oracle_cpu.gd_decode(m, want, 1)
+    r_ref = res.copy()
+    msg, _ = oracle_cpu.gd_encode(want, r_ref, sr, dr_, fixed_clock)
+    assert_bits_equal(C.numpy()[:msg.size], msg, "the root's message as the data stream saw it")
+    torch.cuda.synchronize()
+    assert_bits_equal(host(dgrad), want, "gradient after the gathered messages")
+    assert_bits_equal(host(dres), r_ref, "residual after the root's encode")
+
+
+def test_powersgd_phases_are_complete_for_a_consumer_on_another_stream(drv, pkg):
+    # hp_cuda.cpp:729-768: the three drivers on the compute stream, names published after waiting for the data
+    # stream only; a consumer then reads P, Q and the gradient on a stream of its own.
+    shapes, rk = [(4096, 4096), (1024, 4096), (4096, 1024)] * 3, 4
+    def fresh():
+        g = torch.Generator(device="cuda").manual_seed(8)
+        G = [torch.randn(a * b, device="cuda", generator=g) * 1e-2 for a, b in shapes]
+        R = [torch.randn(a * b, device="cuda", generator=g) * 1e-3 for a, b in shapes]
+        Q = [torch.randn(b, rk, device="cuda", generator=g) for a, b in shapes]
+        M = [torch.zeros(a, b, device="cuda") for a, b in shapes]
+        P = [torch.zeros(a, rk, device="cuda") for a, b in shapes]
+        return G, R, Q, M, P
+    G1, R1, Q1, M1, P1 = fresh()
+    compute, other = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    seen = {}
+    with torch.cuda.stream(compute):
+        drv.hp_cuda_powersgd_encode1(G1, R1, Q1, M1, P1)
+    with torch.cuda.stream(other):
+        seen["P0"] = [p.clone() for p in P1]
+    with torch.cuda.stream(compute):
+        drv.hp_cuda_powersgd_encode2(P1, M1, Q1)
+    with torch.cuda.stream(other):
+        seen["P"] = [p.clone() for p in P1]
+        seen["Q"] = [q.clone() for q in Q1]
+    with torch.cuda.stream(compute):
+        drv.hp_cuda_powersgd_decode(P1, Q1, M1, R1, G1)
+    with torch.cuda.stream(other):
+        seen["G"] = [g.clone() for g in G1]
+        seen["R"] = [r.clone() for r in R1]
+    other.synchronize()
+    G2, R2, Q2, M2, P2 = fresh()
+    assert pkg.hp_cuda_powersgd_encode1(G2, R2, Q2, M2, P2) == 0
+    torch.cuda.synchronize()
+    P0 = [p.clone() for p in P2]
+    assert pkg.hp_cuda_powersgd_encode2(P2, M2, Q2) == 0
+    assert pkg.hp_cuda_powersgd_decode(P2, Q2, M2, R2, G2) == 0
+    torch.cuda.synchronize()
+    for key, ref in (("P0", P0), ("P", P2), ("Q", Q2), ("G", G2), ("R", R2)):
+        for i in range(len(shapes)):
+            assert_bits_equal(host(seen[key][i]).ravel(), host(ref[i]).ravel(), f"{key}[{i}] as the other stream saw it")

@@ -312,7 +312,7 @@ def test_many_tensors_each_with_several_messages(tg, oracle_cpu):
 # ---- the single-launch resident encode (tensor kept on chip between the two passes) ----
 @pytest.fixture
 def resident_from_2m(capi):
-    """By default only tensors of 10 * 2^20 elements and more take the resident encode; these tests want it at 2^21
+    """By default only tensors of 5 * 2^20 elements and more take the resident encode; these tests want it at 2^21
     (and every tensor looked at on its own: the one-launch encode of a whole call has its own tests below)."""
     old = capi.set_option("terngrad_resident_min", 1 << 21)
     old_b = capi.set_option("terngrad_resident_bucket", 0)

@@ -12,6 +12,8 @@ namespace {
 template <typename T>
 const T* const* cptrs(std::vector<T*>& v) { return const_cast<const T* const*>(v.data()); }
 std::vector<int32_t> to_i32(const std::vector<int>& v) { return std::vector<int32_t>(v.begin(), v.end()); }
+// The completion contract of the reference's drivers: what a driver queued on `stream` has run when it returns.
+int finished(hipStream_t stream) { return hipStreamSynchronize(stream) == hipSuccess ? 0 : HPX_ERR_HIP; }
 }  // namespace
 
 SHIM_API void hp_cuda_terngrad(std::vector<float*>& in_floats, std::vector<int32_t>& in_float_sizes,
@@ -21,10 +23,12 @@ SHIM_API void hp_cuda_terngrad(std::vector<float*>& in_floats, std::vector<int32
   int ret = hpx_terngrad_encode(static_cast<int>(in_floats.size()), cptrs(in_floats), in_float_sizes.data(),
                                 out_uint8_ts.data(), out_uint8_t_sizes.data(), bitwidths.data(),
                                 enable_randoms.data(), nullptr, stream);
-  // The reference returns with complete messages (terngrad_body synchronises, terngrad_body.h:195, :273).
-  // Here only a launch that waits at a grid barrier can fail to write one; the status call waits for such
-  // launches and encodes again what an expired barrier left unwritten.
+  // The reference returns with complete messages: terngrad_body waits for the stream after its last quantise
+  // launch (terngrad_body.h:285), and its scheduler copies B on another stream straight afterwards with no event
+  // in between (hp_cuda.cpp:464-468).  The status call waits for launches that meet at a grid barrier and encodes
+  // again what an expired barrier left unwritten; finished() then waits for everything else queued here.
   if (!ret) ret = hpx_terngrad_encode_status(stream);
+  if (!ret) ret = finished(stream);
   if (ret) printf("ret=%d %s\n", ret, hpx_last_error());  // hp_cuda_kernel.cu:63
 }
 
@@ -67,6 +71,10 @@ SHIM_API void hp_cuda_gd(std::vector<float*>& in_floats, std::vector<int32_t>& N
                          std::vector<double>& sample_rates, std::vector<double>& drop_ratios, hipStream_t stream) {
   int ret = hpx_gd_encode(static_cast<int>(in_floats.size()), cptrs(in_floats), Ns.data(), residuals.data(),
                           out_uint8_ts.data(), sample_rates.data(), drop_ratios.data(), nullptr, stream);
+  // gd_body's launches are blocking Thrust calls and it waits for the stream at gd_body.h:161 and :201, so the
+  // reference's scheduler copies B on its data stream right after this call, which it makes on the null
+  // stream (hp_cuda.cpp:292-313).
+  if (!ret) ret = finished(stream);
   if (ret) std::cout << "Call gd_body failed, ret = " << ret << ". " << hpx_last_error() << std::endl;
 }
 
@@ -76,5 +84,8 @@ SHIM_API void hp_cuda_gdr(std::vector<uint8_t*>& in_uint8_ts, std::vector<int32_
   std::vector<int32_t> adds = to_i32(is_add_tos);
   int ret = hpx_gd_decode(static_cast<int>(in_uint8_ts.size()), cptrs(in_uint8_ts), in_uint8_t_sizes.data(),
                           out_floats.data(), out_float_sizes.data(), adds.data(), stream);
+  // The scheduler encodes the tensors decoded here next, on ANOTHER stream (hp_cuda.cpp:284-301: hp_cuda_gdr on
+  // the compute stream, hp_cuda_gd on the null stream; pool streams do not wait for the null stream).
+  if (!ret) ret = finished(stream);
   if (ret) std::cout << "Call gdr_body failed, ret = " << ret << ". " << hpx_last_error() << std::endl;
 }

@@ -4,6 +4,7 @@
 // `c10::cuda::CUDAStream` being the HIP stream wrapper there.  M is n x m,
 // Q is m x r, P is n x r, all contiguous fp32 device tensors.
 #pragma once
+#include <hip/hip_runtime_api.h>
 #include <torch/extension.h>
 
 #include <iostream>
@@ -36,6 +37,10 @@ inline std::vector<int64_t> numels(TensorList& ts) {
 }
 template <typename T>
 const T* const* cp(std::vector<T*>& v) { return const_cast<const T* const*>(v.data()); }
+// A driver returns when what it queued has run: the reference's scheduler publishes a task's name right after
+// the calls, having waited for its data stream only (hp_cuda.cpp:729-768), and its consumers read P, Q and the gradient on streams of their own.
+template <typename Stream>
+int finished(Stream& stream) { return hipStreamSynchronize(stream.stream()) == hipSuccess ? 0 : HPX_ERR_HIP; }
 }  // namespace hp_cuda_shim_detail
 
 template <typename Stream>
@@ -50,6 +55,7 @@ void hp_cuda_powersgd_encode1(std::vector<std::shared_ptr<torch::Tensor>>& grads
   auto ne = numels(grads);
   int ret = hpx_powersgd_encode1(static_cast<int>(g.size()), cp(g), ne.data(), cp(r), cp(q), m.data(), p.data(),
                                  d.n.data(), d.m.data(), d.r.data(), stream.stream());
+  if (!ret) ret = finished(stream);
   if (ret) std::cout << "Call powersgd encode1 failed, ret = " << ret << ". " << hpx_last_error() << std::endl;
 }
 
@@ -62,6 +68,7 @@ void hp_cuda_powersgd_encode2(std::vector<std::shared_ptr<torch::Tensor>>& Ps,
   auto p = ptrs(Ps), m = ptrs(Ms), q = ptrs(Qs);
   int ret = hpx_powersgd_encode2(static_cast<int>(p.size()), p.data(), cp(m), q.data(), d.n.data(), d.m.data(),
                                  d.r.data(), stream.stream());
+  if (!ret) ret = finished(stream);
   if (ret) std::cout << "Call powersgd encode2 failed, ret = " << ret << ". " << hpx_last_error() << std::endl;
 }
 
@@ -77,5 +84,6 @@ void hp_cuda_powersgd_decode(std::vector<std::shared_ptr<torch::Tensor>>& Ps,
   auto ne = numels(grads);
   int ret = hpx_powersgd_decode(static_cast<int>(p.size()), cp(p), cp(q), m.data(), r.data(), g.data(), ne.data(),
                                 d.n.data(), d.m.data(), d.r.data(), stream.stream());
+  if (!ret) ret = finished(stream);
   if (ret) std::cout << "Call powersgd decode failed, ret = " << ret << ". " << hpx_last_error() << std::endl;
 }

@@ -207,6 +207,9 @@ enum Option {
   kOptTerngradResidentWorkgroups,  // "terngrad_resident_workgroups": workgroups of a resident launch; 0 (default) = one per CU.
                                    // For a process that may only use some of the CUs (a CU mask), which the device's CU
                                    // count does not show: a resident launch needs all its workgroups running at once.
+  kOptClockSeed,                // "clock_seed": what an encoder called with seeds == NULL uses in place of the wall clock
+                                // (terngrad_body.h:247-251, gd_body.h:138-140); negative (default) = read the clock.
+                                // Makes the C++ drivers, which cannot pass seeds, reproducible.
   kOptCount
 };
 int64_t option(Option o);

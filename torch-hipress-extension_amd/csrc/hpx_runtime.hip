@@ -190,6 +190,7 @@ const OptionDef kOptions[kOptCount] = {
     {"terngrad_barrier_ms", "HPX_TERNGRAD_BARRIER_MS", 2000},
     {"terngrad_resident_bucket", "HPX_TERNGRAD_RESIDENT_BUCKET", 1},
     {"terngrad_resident_workgroups", "HPX_TERNGRAD_RESIDENT_WORKGROUPS", 0},
+    {"clock_seed", "HPX_CLOCK_SEED", -1},
 };
 std::atomic<int64_t> g_opt[kOptCount];
 std::once_flag g_opt_once;
@@ -324,6 +325,8 @@ int reject_capture(hipStream_t stream, const char* who) {
 }
 
 uint64_t clock_seed() {
+  const int64_t fixed = option(kOptClockSeed);
+  if (fixed >= 0) return static_cast<uint64_t>(fixed);
   return static_cast<uint64_t>(
       std::chrono::high_resolution_clock::now().time_since_epoch().count());
 }
