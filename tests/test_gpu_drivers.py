@@ -178,28 +178,47 @@ def _pinned_like(t):
     return torch.empty(t.shape, dtype=t.dtype, pin_memory=True)
 
 
+def _other_streams(k=4):
+    # HIP multiplexes its streams onto a few hardware queues, and two streams that share a queue are ordered by
+    # accident; consecutive pool streams go to different queues, so among four at least one runs beside `compute`.
+    return [torch.cuda.Stream() for _ in range(k)]
+
+
+def _peek(streams, tensors):
+    """Clones of `tensors` (last first) taken on each of `streams`, with no wait on anything."""
+    seen = []
+    for s in streams:
+        with torch.cuda.stream(s):
+            seen.append([t.clone() for t in reversed(tensors)][::-1])
+    return seen
+
+
 @pytest.mark.parametrize("resident", [False, True])
 def test_terngrad_message_is_complete_for_a_consumer_on_another_stream(drv, oracle_cpu, capi, fixed_clock, resident):
     rng = np.random.default_rng(50)
-    ns = [20_000_003, 18_000_000, 16_000_001] if not resident else [25_557_032]
+    ns = [30_000_003, 28_000_000, 26_000_001, 30_000_000, 29_000_002, 27_000_001] if not resident else [25_557_032]
     xs = [rng.normal(0, 1e-2, n).astype(np.float32) for n in ns]
     old = capi.set_option("terngrad_resident_min", (5 << 20) if resident else -1)   # -1: every tensor takes two launches
     try:
         dx = [dev(x) for x in xs]
         Bs = [torch.full((oracle_cpu.terngrad_packed_size(n, 2),), 0x5A, dtype=torch.uint8, device="cuda") for n in ns]
         Cs = [_pinned_like(b) for b in Bs]
-        compute, data = torch.cuda.Stream(), torch.cuda.Stream()
+        compute, data, others = torch.cuda.Stream(), torch.cuda.Stream(), _other_streams()
         torch.cuda.synchronize()
         with torch.cuda.stream(compute):
             drv.hp_cuda_terngrad(dx, Bs, [2] * len(ns), [1] * len(ns))
+        seen = _peek(others, Bs)
         with torch.cuda.stream(data):                       # hp_cuda.cpp:466-468, no event, no wait in between
             for b, c in zip(Bs, Cs):
                 c.copy_(b, non_blocking=True)
         data.synchronize()                                   # hp_cuda.cpp:485
+        torch.cuda.synchronize()
         for i, x in enumerate(xs):
             rc, ref = oracle_cpu.terngrad_encode(x, 2, 1, fixed_clock)
             assert rc == 0
-            assert_bits_equal(Cs[i].numpy(), ref, f"message[{i}] as the data stream saw it")
+            for k, sk in enumerate(seen):
+                assert_bits_equal(host(sk[i]), ref, f"message[{i}] as a kernel on side stream {k} saw it")
+            assert_bits_equal(Cs[i].numpy(), ref, f"message[{i}] as the copy on the data stream saw it")
     finally:
         capi.set_option("terngrad_resident_min", old)
         torch.cuda.synchronize()
@@ -217,10 +236,11 @@ def test_graddrop_batch_is_complete_for_a_consumer_on_another_stream(drv, oracle
     sizes = [4 + 8 * oracle_cpu.gd_sizes(n, sr, drop_ratio)[1] for n in ns]
     Bs = [torch.full((s,), 0xEE, dtype=torch.uint8, device="cuda") for s in sizes]
     Cs = [_pinned_like(b) for b in Bs]
-    data = torch.cuda.Stream()
+    data, others = torch.cuda.Stream(), _other_streams()
     torch.cuda.synchronize()
     with torch.cuda.stream(torch.cuda.default_stream()):
         drv.hp_cuda_gd(dg, dres, Bs, [sr] * len(ns), [drop_ratio] * len(ns))
+    seen = _peek(others, Bs)
     with torch.cuda.stream(data):
         for b, c in zip(Bs, Cs):
             c.copy_(b, non_blocking=True)
@@ -231,6 +251,8 @@ def test_graddrop_batch_is_complete_for_a_consumer_on_another_stream(drv, oracle
         r_ref = rs[i].copy()
         msg, info = oracle_cpu.gd_encode(gs[i], r_ref, sr, drop_ratio, fixed_clock)
         assert_bits_equal(Cs[i].numpy()[:msg.size], msg, f"message[{i}] as the data stream saw it")
+        for k, sk in enumerate(seen):
+            assert_bits_equal(host(sk[i])[:msg.size], msg, f"message[{i}] as a kernel on side stream {k} saw it")
         assert_bits_equal(host(res_seen[i]), r_ref, f"residual[{i}] as the data stream saw it")
         cut.append(info["candidates"] > info["kept"])
     assert any(cut) and not all(cut), cut                   # the batch holds both branches
