@@ -479,6 +479,45 @@ def test_resident_barrier_expiry_is_repaired(tg, oracle_cpu, capi, resident_from
         assert capi.load().hpx_release_workspaces() == 0
 
 
+def test_repair_leaves_the_buffers_of_finished_calls_alone(tg, oracle_cpu, capi, resident_from_2m):
+    # Two single-launch encodes that finish well, no status call; their buffers are then overwritten, as a caller
+    # whose allocator hands the memory on would.  A third encode's barrier expires.  The repair must encode the third
+    # call's tensor only: the records of the first two were dropped when the third call found their events reached
+    # with the expiry flag down.
+    rng = np.random.default_rng(15)
+    n = 3_000_000
+    xs = [rng.normal(0, 1e-2, n).astype(np.float32) for _ in range(3)]
+    refs = [oracle_cpu.terngrad_encode(x, 2, 1, 20 + i)[1] for i, x in enumerate(xs)]
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    assert capi.load().hpx_release_workspaces() == 0
+    prev = None
+    try:
+        with torch.cuda.stream(side):
+            dxs = [dev(x) for x in xs]
+            outs = [torch.full((tg.packed_size(n, 2),), 0x5A, dtype=torch.uint8, device="cuda") for _ in range(3)]
+            for i in range(2):
+                tg.encode([dxs[i]], [2], [1], [20 + i], outs=[outs[i]])
+            side.synchronize()
+            for i in range(2):
+                assert_bits_equal(host(outs[i]), refs[i], f"message of good call {i}")
+            # the caller reuses the memory of the finished calls
+            outs[0].fill_(0x11); outs[1].fill_(0x22); dxs[0].zero_(); dxs[1].zero_()
+            side.synchronize()
+            prev = capi.set_option("terngrad_barrier_ms", 0)
+            tg.encode([dxs[2]], [2], [1], [22], outs=[outs[2]])
+            assert tg.encode_status() == 0, capi.last_error()
+            capi.set_option("terngrad_barrier_ms", prev); prev = None
+            assert tg.repaired() == 1                          # only the call whose barrier expired
+            assert_bits_equal(host(outs[2]), refs[2], "the expired call's message after the repair")
+            assert bool((outs[0] == 0x11).all()) and bool((outs[1] == 0x22).all()), "buffers of finished calls were written again"
+    finally:
+        if prev is not None:
+            capi.set_option("terngrad_barrier_ms", prev)
+        torch.cuda.synchronize()
+        assert capi.load().hpx_release_workspaces() == 0
+
+
 def test_release_stream_hands_the_resident_kernel_on(tg, oracle_cpu, capi, resident_from_2m):
     # The first stream that encodes a large tensor owns the barrier kernels; once it has been released
     # (as the scheduler's worker does before it destroys its stream) another stream gets them.

@@ -8,6 +8,7 @@
 #include <vector>
 
 #include "hpx.h"
+#include "hpx_completion_log.h"
 
 #define HPX_API extern "C" __attribute__((visibility("default")))
 
@@ -92,7 +93,11 @@ struct Workspace {
     uint64_t seed;
     uint8_t bits, random;
   };
-  std::vector<ResidentRec> resident_log;
+  // A call records an event behind its barrier launches; the next call drops the records of every call whose
+  // event has been reached while the expiry flag is down, so the log only ever names buffers of calls that
+  // may still be running (hpx_completion_log.h).
+  CompletionLog<ResidentRec, hipEvent_t> resident_log;
+  std::vector<hipEvent_t> event_pool;  // events to reuse for those marks
   uint64_t repaired = 0;  // tensors encoded again after an expired barrier, ever
 };
 constexpr size_t kStateWords = 4096;       // 16 KiB

@@ -265,6 +265,8 @@ HPX_API int hpx_ecq_encode(int count, const float* const* Gs, const int32_t* Ns,
             out_sizes[i]);
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
+  // the workspace may have to grow (a wait for the stream, hipFree, hipMalloc): not something a graph can record
+  if (const int rcc = hpx::reject_capture(st, "hpx_ecq_encode")) return rcc;
   hpx::Workspace* ws = hpx::workspace_record(st);
   if (!ws) return HPX_ERR_HIP;
   std::lock_guard<std::mutex> lock(ws->mu);

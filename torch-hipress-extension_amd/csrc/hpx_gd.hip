@@ -1148,8 +1148,9 @@ int decode_messages(int count, const uint8_t* const* ins, const int32_t* in_size
   HPX_ARG(count >= 0, "hpx_gd_decode: negative count");
   if (count == 0) return HPX_OK;
   HPX_ARG(ins && in_sizes && outs && out_sizes && is_add_tos, "hpx_gd_decode: null argument array");
-  HPX_ARG(size_t(count) * sizeof(int32_t) <= hpx::kPinnedBytes, "hpx_gd_decode: more than %zu messages in one call",
-          hpx::kPinnedBytes / sizeof(int32_t));
+  // the headers are read back into the pinned block, whose last words belong to the barrier kernels' expiry flag
+  HPX_ARG(size_t(count) * sizeof(int32_t) <= hpx::kPinnedFlagOffset, "hpx_gd_decode: more than %zu messages in one call",
+          hpx::kPinnedFlagOffset / sizeof(int32_t));
   for (int i = 0; i < count; i++) {
     HPX_ARG(ins[i] && outs[i] && out_sizes[i] >= 0, "hpx_gd_decode: message %d has a null pointer or negative size", i);
     HPX_ARG((reinterpret_cast<uintptr_t>(ins[i]) & 3) == 0, "hpx_gd_decode: message %d is not 4-byte aligned", i);

@@ -145,6 +145,10 @@ int free_workspace(Workspace* ws) {
   if (ws->slots && hipFree(ws->slots) != hipSuccess) rc = HPX_ERR_HIP;
   if (ws->bar && hipFree(ws->bar) != hipSuccess) rc = HPX_ERR_HIP;
   if (ws->pinned && hipHostFree(ws->pinned) != hipSuccess) rc = HPX_ERR_HIP;
+  ws->resident_log.clear([ws](hipEvent_t e) { if (e) ws->event_pool.push_back(e); });
+  for (hipEvent_t e : ws->event_pool)
+    if (hipEventDestroy(e) != hipSuccess) rc = HPX_ERR_HIP;
+  ws->event_pool.clear();
   ws->dev = nullptr; ws->aux = nullptr; ws->state = nullptr; ws->slots = nullptr; ws->bar = nullptr; ws->pinned = nullptr;
   return rc;
 }

@@ -206,7 +206,7 @@ __device__ __forceinline__ void tbq_decode_tile(const DecSeg& sg, uint32_t t) {
     // consecutive bytes of codes, which it fetches with ONE load (a dword per lane); the lanes pick their
     // bytes out of it with cross-lane reads.  (A byte load per group and lane, the workgroup walking the
     // tile 4 KiB at a time, took 84 us for 110 M elements where this takes 66.)
-    static_assert(kIters * 4 <= kWave, "a wave's bytes must fit one dword per lane");
+    static_assert(kIters * kWave == kWave * 4, "a wave fetches exactly 256 code bytes, one dword per lane: four groups of four elements per lane");
     const uint32_t lane = threadIdx.x & (kWave - 1);
     const uint32_t gw = gbeg + (threadIdx.x / kWave) * uint32_t(kIters * kWave);  // the wave's first group
     const uint32_t dw = as_global(reinterpret_cast<const u32u*>(ip + gw + lane * 4))->v;  // messages start at any byte
@@ -369,7 +369,7 @@ __global__ __launch_bounds__(kThreads) void tbq_decode_multi_kernel(const Args a
     // group and message (28 loads per lane for 7 messages; the address pipeline, not memory,
     // was the limit).  The old values and up to 8 messages are requested together, then folded in
     // message order.
-    static_assert(kIters * 4 <= kWave, "a wave's bytes of one message must fit one dword per lane");
+    static_assert(kIters * kWave == kWave * 4, "a wave fetches exactly 256 code bytes of a message, one dword per lane");
     const uint32_t lane = threadIdx.x & (kWave - 1);
     const uint32_t gw = g0 - threadIdx.x + (threadIdx.x / kWave) * uint32_t(kIters * kWave);  // the wave's first group
     float4 acc[kIters];

@@ -1981,6 +1981,11 @@ int encode_tiled(hpx::Workspace* ws, hipStream_t st, int count, const float* con
 // A barrier kernel on this stream gave up waiting (ws->mu held): barrier kernels are switched off for the
 // stream and every tensor they have encoded since the stream was last known to be good is queued again
 // through the tiled kernels, with the seed it was given the first time, so the same message comes out.
+// Hands an event of a mark back to the workspace's pool.
+inline auto recycle_into(hpx::Workspace* ws) {
+  return [ws](hipEvent_t e) { if (e) ws->event_pool.push_back(e); };
+}
+
 int repair_resident_log(hpx::Workspace* ws, hipStream_t st) {
   ws->barrier_broken = true;
   if (ws->resident_log.empty()) return HPX_OK;
@@ -1991,14 +1996,38 @@ int repair_resident_log(hpx::Workspace* ws, hipStream_t st) {
   std::vector<uint8_t> t_bits(m);
   std::vector<uint64_t> t_seed(m);
   for (int k = 0; k < m; k++) {
-    const hpx::Workspace::ResidentRec& r = ws->resident_log[k];
+    const hpx::Workspace::ResidentRec& r = ws->resident_log.records()[k];
     t_in[k] = r.x; t_out[k] = r.out; t_isz[k] = r.n; t_osz[k] = r.out_size;
     t_rnd[k] = r.random; t_bits[k] = r.bits; t_seed[k] = r.seed;
   }
-  ws->resident_log.clear();
+  ws->resident_log.clear(recycle_into(ws));
   ws->repaired += uint64_t(m);
   return encode_tiled(ws, st, m, t_in.data(), t_isz.data(), t_out.data(), t_osz.data(), t_bits.data(), t_rnd.data(),
                       t_seed.data());
+}
+
+// Drops the records of earlier calls whose barrier launches have finished with the expiry flag down: their
+// buffers are the caller's again and must not be named by a later repair (ws->mu held, workspace ensured).
+void prune_resident_log(hpx::Workspace* ws) {
+  ws->resident_log.prune([](hipEvent_t e) { return hipEventQuery(e) == hipSuccess; },
+                         [ws] { return !hpx::barrier_expired(ws); }, recycle_into(ws));
+}
+
+// Records an event behind the barrier launches a call has queued and marks the log with it (ws->mu held).
+void mark_resident_log(hpx::Workspace* ws, hipStream_t st) {
+  if (ws->resident_log.empty()) return;
+  hipEvent_t e = nullptr;
+  if (!ws->event_pool.empty()) {
+    e = ws->event_pool.back();
+    ws->event_pool.pop_back();
+  } else if (hipEventCreateWithFlags(&e, hipEventDisableTiming) != hipSuccess) {
+    return;  // no mark: the records stay until a later mark or a wait for the stream covers them
+  }
+  if (hipEventRecord(e, st) != hipSuccess) {
+    ws->event_pool.push_back(e);
+    return;
+  }
+  ws->resident_log.mark(e, recycle_into(ws));
 }
 
 // Waits for the stream and settles the log of barrier-kernel encodes: cleared if they all got through, encoded
@@ -2006,7 +2035,7 @@ int repair_resident_log(hpx::Workspace* ws, hipStream_t st) {
 int settle_resident_log(hpx::Workspace* ws, hipStream_t st) {
   HPX_HIP(hipStreamSynchronize(st));
   if (!hpx::barrier_expired(ws)) {
-    ws->resident_log.clear();
+    ws->resident_log.clear(recycle_into(ws));
     return HPX_OK;
   }
   // every kernel of the stream has finished: nothing can raise the flag again behind this
@@ -2089,10 +2118,16 @@ HPX_API int hpx_terngrad_encode(int count, const float* const* ins, const int32_
   // through the tiled kernels before this call's work, and this call takes the tiled kernels too.  (The
   // flag stays up until hpx_terngrad_encode_status has waited for the stream: workgroups of that
   // kernel may still be on their way out.)
+  prune_resident_log(ws);
   if (!ws->barrier_broken && hpx::barrier_expired(ws)) {
     rc = repair_resident_log(ws, st);
     if (rc != HPX_OK) return rc;
   }
+  // whatever this call logs is marked when it returns, on every path
+  struct MarkOnExit {
+    hpx::Workspace* ws; hipStream_t st;
+    ~MarkOnExit() { mark_resident_log(ws, st); }
+  } mark_on_exit{ws, st};
   if (ws->resident_log.size() + size_t(count) > kResidentLogMax) {
     rc = settle_resident_log(ws, st);
     if (rc != HPX_OK) return rc;
@@ -2106,7 +2141,7 @@ HPX_API int hpx_terngrad_encode(int count, const float* const* ins, const int32_
   const bool buckets = count >= 2 && hpx::option(hpx::kOptTerngradResidentBucket) != 0 &&
                        hpx::option(hpx::kOptTerngradResidentMin) >= 0;
   auto log_resident = [&](const EncSeg& sg, uint64_t seed) {
-    ws->resident_log.push_back(hpx::Workspace::ResidentRec{sg.x, sg.out, sg.n, sg.out_size, seed, sg.bits, sg.random});
+    ws->resident_log.add(hpx::Workspace::ResidentRec{sg.x, sg.out, sg.n, sg.out_size, seed, sg.bits, sg.random});
   };
   int i = 0;
   while (i < count) {
