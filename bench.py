@@ -84,6 +84,71 @@ def timed(torch, fn, steps, warmup):
     return (time.perf_counter() - t0) / steps
 
 
+def event_pairs(torch, fn, steps, warmup=3):
+    """Per-step durations (s) from a pair of events recorded on the stream around each step (the launches are on
+    torch's current stream): what the GPU spends between the start of a step's first kernel and the end of its last,
+    hand-overs between the launches included, host launch time excluded as long as the queue stays ahead."""
+    for _ in range(warmup):
+        fn()
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    torch.cuda.synchronize()
+    for a, b in pairs:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    return sorted(a.elapsed_time(b) * 1e-3 for a, b in pairs)
+
+
+def quantiles(xs_sorted, scale=1e3, digits=5):
+    n = len(xs_sorted)
+    pick = lambda q: xs_sorted[min(n - 1, int(q * n))]
+    return {"median": round(pick(0.5) * scale, digits), "p10": round(pick(0.1) * scale, digits),
+            "p90": round(pick(0.9) * scale, digits), "min": round(xs_sorted[0] * scale, digits), "n": n}
+
+
+def terngrad_phases(torch, np, L, fn, workgroups, launches=20):
+    """Per-phase breakdown of the resident encode from the four wall-clock stamps each workgroup leaves
+    (hpx_terngrad_phase_stamps; 100 MHz, so 0.01 us steps): for each launch, times are taken from the earliest entry
+    stamp of the grid; reported are medians over `launches` launches of the min / median / max over workgroups."""
+    buf = torch.zeros(4 * workgroups, dtype=torch.int64, device="cuda")
+    rows = {k: [] for k in ("entry", "loaded_and_reduced", "exchange_passed", "last_store",
+                            "load_phase", "exchange_phase", "quantise_phase")}
+    try:
+        if L.hpx_terngrad_phase_stamps(buf.data_ptr(), workgroups):
+            return None
+        for _ in range(3):
+            fn()
+        for _ in range(launches):
+            buf.zero_()
+            torch.cuda.synchronize()
+            fn()
+            torch.cuda.synchronize()
+            t = buf.cpu().numpy().reshape(workgroups, 4).astype(np.float64)
+            t = t[(t > 0).all(axis=1)]
+            if not len(t):
+                continue
+            t0 = t[:, 0].min()
+            rel = (t - t0) / 100.0    # us
+            cols = {"entry": rel[:, 0], "loaded_and_reduced": rel[:, 1], "exchange_passed": rel[:, 2], "last_store": rel[:, 3],
+                    "load_phase": rel[:, 1] - rel[:, 0], "exchange_phase": rel[:, 2] - rel[:, 1],
+                    "quantise_phase": rel[:, 3] - rel[:, 2]}
+            for k, v in cols.items():
+                rows[k].append((v.min(), np.median(v), v.max()))
+    finally:
+        L.hpx_terngrad_phase_stamps(None, 0)
+        torch.cuda.synchronize()
+    if not rows["entry"]:
+        return None
+    out = {"unit": "us", "clock": "100 MHz wall clock, stamps per workgroup, time 0 = earliest entry of the launch",
+           "launches": len(rows["entry"]), "workgroups": workgroups,
+           "columns": "median over launches of [min, median, max] over workgroups"}
+    for k, v in rows.items():
+        a = np.median(np.array(v), axis=0)
+        out[k] = [round(float(x), 2) for x in a]
+    return out
+
+
 def kernel_times(torch, capi, fn, names, reps=10):
     """Average duration (s) of each named kernel: HIP events attached to each launch on its stream (begin and end of the kernel itself)."""
     L = capi.load()
@@ -173,6 +238,11 @@ def main():
 
     sec_enc = timed(torch, only(3), max(20, args.steps // 4), 5)
     sec_dec = timed(torch, only(4), max(20, args.steps // 4), 5)
+    pairs = event_pairs(torch, step, max(20, min(args.steps, 200)))
+    pairs_enc = event_pairs(torch, only(3), 40)
+    pairs_dec = event_pairs(torch, only(4), 40)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    phases = terngrad_phases(torch, np, L, only(3), cus)
 
     kt = kernel_times(torch, capi, step,
                       ["terngrad_resident_kernel", "terngrad_minmax_kernel", "terngrad_quant_kernel", "terngrad_decode_kernel"])
@@ -194,7 +264,11 @@ def main():
     path = {"algorithmic_bytes_per_step": path_alg, "achieved_GBps": round(path_alg / sec / 1e9, 1),
             "frac_of_hbm_peak": round(path_alg / sec / 1e9 / HBM_PEAK_GBS, 4),
             "warm_cache_ms_per_step": round(sec_warm * 1e3, 4), "encode_ms": round(sec_enc * 1e3, 4),
-            "decode_ms": round(sec_dec * 1e3, 4), "buffer_sets": len(sets)}
+            "decode_ms": round(sec_dec * 1e3, 4), "buffer_sets": len(sets),
+            "wall_clock_mean_ms_per_step": round(sec * 1e3, 5),
+            "event_pair_ms_per_step": quantiles(pairs), "event_pair_encode_ms": quantiles(pairs_enc),
+            "event_pair_decode_ms": quantiles(pairs_dec),
+            "frac_of_hbm_peak_event_pair_median": round(path_alg / quantiles(pairs, 1.0, 9)["median"] / 1e9 / HBM_PEAK_GBS, 4)}
 
     result = {
         "metric": "encode+decode GB/s of fp32 gradient (TernGrad 2-bit, 1 GPU)", "value": round(value, 2), "unit": "GB/s",
@@ -213,6 +287,8 @@ def main():
         result["cpu_baseline"] = cpu_baseline(np, n, args.cpu_seconds)
     if not args.no_extra:
         result["extra"] = extra(torch, np, capi, L, stream, gen)
+    if phases:
+        result.setdefault("extra", {})["terngrad_phases_us"] = phases
     print(json.dumps(result), flush=True)
 
 

@@ -198,6 +198,18 @@ int hpx_terngrad_encode(int count, const float* const* ins, const int32_t* in_si
 int hpx_terngrad_encode_status(hpx_stream_t stream);
 int64_t hpx_terngrad_repaired(hpx_stream_t stream);
 
+/* Measurement aid, no counterpart in the reference.  While a device buffer of
+ * 4 * workgroups 64-bit words is set, every workgroup b of a single-launch
+ * (resident) encode leaves four readings of the GPU's 100 MHz wall clock in
+ * words 4b .. 4b+3: on entry, before its first load is requested; when its
+ * whole share is loaded and reduced; when it has the global extremes (the
+ * grid-wide exchange is behind it); when its last store has been issued.
+ * bench.py turns them into the per-phase breakdown of the headline kernel.
+ * Launches with more workgroups than the buffer holds leave nothing.  NULL or
+ * 0 switches it off (the default); the caller keeps the buffer alive until
+ * then and until the launches that saw it have finished. */
+int hpx_terngrad_phase_stamps(uint64_t* device_words, int32_t workgroups);
+
 /* hpx_terngrad_encode for callers that cannot allocate: code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart
  * in the reference.  Same arguments, same bytes out; always the two-launch path

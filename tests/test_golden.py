@@ -1,6 +1,8 @@
-"""Golden vectors produced by the reference's own code (tests/golden/make_fixtures.py, which compiles the
-reference's header bodies for the host) against (a) the CPU oracle and (b) the HIP kernels through the
-C ABI.  Bit-exact throughout."""
+"""Regression vectors written by the CPU oracle (tests/golden/make_fixtures.py; `--check` reproduces the committed
+file) held against (a) the oracle as it is now and (b) the HIP kernels through the C ABI, bit for bit.  They keep the
+two from drifting apart or changing unnoticed; they do NOT pin either to the reference, whose code had no part in
+writing them - that is the job of the hand-derived known answers (tests/kat_vectors.py, tests/test_oracle_kat.py,
+tests/test_gpu_kat.py) and of the brute-force and closed-form checks in tests/test_oracle_*.py."""
 import os
 
 import numpy as np
@@ -25,7 +27,7 @@ def _eq(a, b, what):
     assert np.array_equal(a.view(np.uint8), b.view(np.uint8)), what
 
 
-# ---- (a) the CPU oracle reproduces the reference's answers ---------------------------------------
+# ---- (a) the CPU oracle still produces the vectors it wrote --------------------------------------
 def test_oracle_tbq_against_golden(gold, oracle_cpu):
     for k in range(int(gold["tbq_count"])):
         g, r, thr = gold[f"tbq_{k}_g"], gold[f"tbq_{k}_r0"].copy(), float(gold[f"tbq_{k}_thr"])
@@ -80,7 +82,7 @@ def test_oracle_lcg_against_golden(gold, oracle_cpu):
     assert gold["lcg_draws"][0][:4].tolist() == [3554416254, 2802067423, 3596950572, 229283573]
 
 
-# ---- (b) the HIP kernels reproduce the reference's answers -----------------------------------------
+# ---- (b) the HIP kernels produce the same vectors ---------------------------------------------------
 @pytest.mark.gpu
 def test_gpu_against_golden(gold, capi):
     import torch

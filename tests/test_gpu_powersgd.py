@@ -175,35 +175,51 @@ def test_rank_above_limit_is_rejected(psgd):
 
 
 def test_config4_layer_set(psgd):
-    # 12 x (4096x4096), 12 x (1024x4096), 12 x (4096x1024), entries ~N(0,1e-2), Q ~N(0,1), rank 4:
-    # checked against the oracle on one matrix of each shape (the fp64 oracle takes seconds per large matrix)
+    # 12 x (4096x4096), 12 x (1024x4096), 12 x (4096x1024), entries ~N(0,1e-2), Q ~N(0,1), rank 4, TWO iterations
+    # (the second starts from the first one's residual and warm-started Q, so the error feedback runs at full size).
+    # Per iteration: four matrices of each shape against the fp64 oracle (the first, the last and two in between),
+    # and all 36 through invariants evaluated on the device.
     gen = torch.Generator(device="cuda").manual_seed(0)
     shapes = [(4096, 4096)] * 12 + [(1024, 4096)] * 12 + [(4096, 1024)] * 12
     r = 4
-    G = [torch.randn(n * m, device="cuda", generator=gen) * 1e-2 for n, m in shapes]
     R = [torch.zeros(n * m, device="cuda") for n, m in shapes]
     Q = [torch.randn(m, r, device="cuda", generator=gen) for n, m in shapes]
     M = [torch.zeros(n, m, device="cuda") for n, m in shapes]
     P = [torch.zeros(n, r, device="cuda") for n, m in shapes]
-    picks = (0, 12, 24, 35)
-    G0 = {i: host(G[i]).copy() for i in picks}
-    Q0 = {i: host(Q[i]).copy() for i in picks}
-    psgd.encode1(G, R, Q, M, P)
-    psgd.encode2(P, M, Q)
-    psgd.decode(P, Q, M, R, G)
-    torch.cuda.synchronize()
-    for i in picks:
-        n, m = shapes[i]
-        Mref, Pref = ps.encode1(G0[i], np.zeros(n * m, np.float32), Q0[i], np.zeros((n, m), np.float32))
-        Po, Qn = ps.encode2(Pref, Mref)
-        Mn, Rn, Gn = ps.decode(Po, Qn, G0[i])
-        Pg = host(P[i]).astype(np.float64)
-        sign = np.sign(np.sum(Pg * Po, axis=0))
-        assert np.linalg.norm(Pg.T @ Pg - np.eye(r)) < 1e-5
-        assert ps.rel_fro(Pg * sign, Po) < TOL and ps.rel_fro(host(Q[i]) * sign, Qn) < TOL
-        assert ps.rel_fro(host(M[i]), Mn) < TOL and ps.rel_fro(host(G[i]), Gn) < TOL
-        assert np.linalg.norm(host(R[i]).astype(np.float64) - Rn) / np.linalg.norm(G0[i].astype(np.float64)) < TOL
-    # every matrix: grad_new + residual_new == grad_old up to one fp32 rounding, checked on the device
-    for i in (1, 13, 25):
-        n, m = shapes[i]
-        assert bool((G[i] == M[i].reshape(-1)).all())
+    picks = (0, 3, 7, 11, 12, 16, 20, 23, 24, 27, 31, 35)
+    eye = torch.eye(r, device="cuda", dtype=torch.float64)
+    for it in range(2):
+        G = [torch.randn(n * m, device="cuda", generator=gen) * 1e-2 for n, m in shapes]
+        G0 = {i: host(G[i]).copy() for i in picks}
+        R0 = {i: host(R[i]).copy() for i in picks}
+        Q0 = {i: host(Q[i]).copy() for i in picks}
+        Gin = [g.clone() for g in G]
+        Rin = [x.clone() for x in R]
+        psgd.encode1(G, R, Q, M, P)
+        torch.cuda.synchronize()
+        Min = [x.clone() for x in M]                                       # M = G + R, before decode overwrites it
+        psgd.encode2(P, M, Q)
+        psgd.decode(P, Q, M, R, G)
+        torch.cuda.synchronize()
+        for i in picks:
+            n, m = shapes[i]
+            Mref, Pref = ps.encode1(G0[i], R0[i], Q0[i], np.zeros((n, m), np.float32))
+            assert_bits_equal(host(Min[i]).ravel(), Mref.ravel(), f"iteration {it} M[{i}] = G + R")
+            Po, Qn = ps.encode2(Pref, Mref)
+            Mn, Rn, Gn = ps.decode(Po, Qn, G0[i])                          # residual = grad - P Q^T (powersgd_body.h:72)
+            Pg = host(P[i]).astype(np.float64)
+            sign = np.sign(np.sum(Pg * Po, axis=0))
+            assert ps.rel_fro(Pg * sign, Po) < TOL and ps.rel_fro(host(Q[i]) * sign, Qn) < TOL, (it, i)
+            assert ps.rel_fro(host(M[i]), Mn) < TOL and ps.rel_fro(host(G[i]), Gn) < TOL, (it, i)
+            assert np.linalg.norm(host(R[i]).astype(np.float64) - Rn) / np.linalg.norm(G0[i].astype(np.float64)) < TOL, (it, i)
+        for i, (n, m) in enumerate(shapes):
+            Pd, Qd, Md = P[i].double(), Q[i].double(), Min[i].double()
+            assert float((Pd.T @ Pd - eye).norm()) < 1e-5, (it, i)        # orthonormal columns
+            assert float((Qd - Md.T @ Pd).norm() / Qd.norm()) < TOL, (it, i)   # Q = M^T P
+            assert bool((G[i] == M[i].reshape(-1)).all()), (it, i)        # the gradient handed on is P Q^T
+            assert bool((Min[i].reshape(-1) == Gin[i] + Rin[i]).all()), (it, i)  # M was G + R, one fp32 add
+            # what the approximation leaves out of the gradient went into the residual: grad_new + residual_new ==
+            # grad_old to one fp32 rounding
+            back = (G[i].double() + R[i].double() - Gin[i].double()).abs().max()
+            assert float(back) <= 2.0 ** -23 * float(Gin[i].abs().max()) * 2, (it, i, float(back))
+        del Gin, Rin, Min

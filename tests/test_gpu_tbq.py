@@ -164,8 +164,8 @@ def test_bucket_of_many_tensors(tbq, oracle_cpu):
         assert_bits_equal(host(outs[i]), oracle_cpu.tbq_decode(host(packed[i]), n, thrs[i]), f"decoded[{i}]")
 
 
-def test_full_size_bucket_properties(tbq):
-    # 110M-element bucket (BERT-base-like): size-independent properties only.
+def test_full_size_bucket_two_steps(tbq):
+    # 110M-element bucket (BERT-base-like): size-independent properties, then all 200 tensors against the oracle.
     rng = np.random.default_rng(0)
     sizes = np.exp(rng.uniform(np.log(768), np.log(3e7), 200))
     sizes = np.clip(np.floor(sizes * 110e6 / sizes.sum()), 768, 3e7).astype(np.int64)
@@ -191,15 +191,22 @@ def test_full_size_bucket_properties(tbq):
         codes = packed[i]
         assert int(((codes >> 0) & 3 == 3).sum() + ((codes >> 2) & 3 == 3).sum()) == 0
     assert [float(g.double().sum()) for g in gs[:5]] == g_sum  # gradients untouched
-    # bit-exact against the oracle on the largest and a few other tensors of the bucket
+    # Two consecutive steps, every one of the 200 tensors bit-exact against the oracle: packed bytes, residual
+    # (the second step starts from the first one's residuals: the error feedback at full size) and decoded tensor.
     from oracle import cpu
-    for i in (0, 7, int(np.argmax(sizes)), len(gs) - 1):
-        gh = host(gs[i])
-        rh = np.zeros_like(gh)
-        p_ref = cpu.tbq_encode(gh, rh, thr)
-        assert_bits_equal(host(packed[i]), p_ref, f"bucket packed[{i}]")
-        assert_bits_equal(host(rs[i]), rh, f"bucket residual[{i}]")
-        assert_bits_equal(host(outs[i]), cpu.tbq_decode(p_ref, gh.size, thr), f"bucket decoded[{i}]")
+    r_host = [np.zeros(int(n), np.float32) for n in sizes]
+    for step in range(2):
+        if step == 1:
+            gs = [torch.randn(int(n), device="cuda", generator=gen) * 5e-3 for n in sizes]
+            packed = tbq.encode(gs, rs, [thr] * len(gs))
+            tbq.decode(packed, outs, [thr] * len(gs), [0] * len(gs))
+            torch.cuda.synchronize()
+        for i in range(len(gs)):
+            gh = host(gs[i])
+            p_ref = cpu.tbq_encode(gh, r_host[i], thr)
+            assert_bits_equal(host(packed[i]), p_ref, f"step {step} bucket packed[{i}]")
+            assert_bits_equal(host(rs[i]), r_host[i], f"step {step} bucket residual[{i}]")
+            assert_bits_equal(host(outs[i]), cpu.tbq_decode(p_ref, gh.size, thr), f"step {step} bucket decoded[{i}]")
 
 
 @pytest.mark.parametrize("n", [7, 4096, 10007, 300001])

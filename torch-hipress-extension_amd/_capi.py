@@ -25,6 +25,7 @@ SYMBOLS = (
     "hpx_terngrad_encode",
     "hpx_terngrad_encode_status",
     "hpx_terngrad_repaired",
+    "hpx_terngrad_phase_stamps",
     "hpx_terngrad_encode_noalloc",
     "hpx_terngrad_decode",
     "hpx_terngrad_decode_status",
@@ -98,6 +99,7 @@ def load():
     L.hpx_terngrad_encode_status.argtypes = [p]
     L.hpx_terngrad_repaired.argtypes = [p]
     L.hpx_terngrad_repaired.restype = C.c_int64
+    L.hpx_terngrad_phase_stamps.argtypes = [p, i32]
     L.hpx_release_stream.argtypes = [p]
     L.hpx_terngrad_decode.argtypes = [i32, pp, p, pp, p, p, p]
     L.hpx_terngrad_decode_status.argtypes = [p]

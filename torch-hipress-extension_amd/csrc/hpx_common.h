@@ -93,11 +93,17 @@ struct Workspace {
     uint64_t seed;
     uint8_t bits, random;
   };
-  // A call records an event behind its barrier launches; the next call drops the records of every call whose
-  // event has been reached while the expiry flag is down, so the log only ever names buffers of calls that
-  // may still be running (hpx_completion_log.h).
-  CompletionLog<ResidentRec, hipEvent_t> resident_log;
-  std::vector<hipEvent_t> event_pool;  // events to reuse for those marks
+  // Every workgroup of a barrier launch that gets through its barrier stores the launch's generation into its
+  // word of `done` (pinned host memory); a launch is marked in the log by its generation and grid, and the next
+  // call drops the records of every launch whose workgroups have all reported while the expiry flag is down, so
+  // the log only ever names buffers of launches that may still have to be repeated (hpx_completion_log.h).  No
+  // event, nothing extra on the stream.
+  struct ResidentMark {
+    uint32_t gen;
+    int32_t grid;
+  };
+  CompletionLog<ResidentRec, ResidentMark> resident_log;
+  uint32_t* done = nullptr;  // kBarMaxWorkgroups words, see ensure_barrier
   uint64_t repaired = 0;  // tensors encoded again after an expired barrier, ever
 };
 constexpr size_t kStateWords = 4096;       // 16 KiB

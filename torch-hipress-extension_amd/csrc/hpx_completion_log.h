@@ -1,6 +1,6 @@
 // A log of work records that is pruned by completion marks.  Host-only, no HIP types: the mark is whatever the
-// owner uses to ask "has everything queued before this point finished?" (a HIP event in the library, an integer
-// in the unit test).
+// owner uses to ask "has everything queued before this point finished?" (in the library the generation and grid
+// of a barrier launch, checked against the words its workgroups leave in host memory; an integer in the unit test).
 //
 // Use: add() a record for each piece of queued work that may have to be repeated, mark() after the launches of a
 // call, prune() at the start of the next call.  prune() asks, oldest mark first, whether the mark has been

@@ -145,10 +145,9 @@ int free_workspace(Workspace* ws) {
   if (ws->slots && hipFree(ws->slots) != hipSuccess) rc = HPX_ERR_HIP;
   if (ws->bar && hipFree(ws->bar) != hipSuccess) rc = HPX_ERR_HIP;
   if (ws->pinned && hipHostFree(ws->pinned) != hipSuccess) rc = HPX_ERR_HIP;
-  ws->resident_log.clear([ws](hipEvent_t e) { if (e) ws->event_pool.push_back(e); });
-  for (hipEvent_t e : ws->event_pool)
-    if (hipEventDestroy(e) != hipSuccess) rc = HPX_ERR_HIP;
-  ws->event_pool.clear();
+  if (ws->done && hipHostFree(ws->done) != hipSuccess) rc = HPX_ERR_HIP;
+  ws->done = nullptr;
+  ws->resident_log.clear([](Workspace::ResidentMark) {});
   ws->dev = nullptr; ws->aux = nullptr; ws->state = nullptr; ws->slots = nullptr; ws->bar = nullptr; ws->pinned = nullptr;
   return rc;
 }
@@ -179,6 +178,9 @@ int ensure_barrier(Workspace* ws) {
   HPX_HIP(hipMalloc(reinterpret_cast<void**>(&ws->bar), kBarWords * sizeof(uint32_t)));
   HPX_HIP(hipMemset(ws->bar, 0, kBarWords * sizeof(uint32_t)));
   ws->bar_gen = 0;
+  // one word per workgroup of a barrier launch, written by the GPU with system scope, read by the host at any time
+  HPX_HIP(hipHostMalloc(reinterpret_cast<void**>(&ws->done), kBarMaxWorkgroups * sizeof(uint32_t), hipHostMallocCoherent));
+  std::memset(ws->done, 0, kBarMaxWorkgroups * sizeof(uint32_t));
   return HPX_OK;
 }
 

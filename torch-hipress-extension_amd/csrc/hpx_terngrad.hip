@@ -27,6 +27,7 @@
 //   * min and max are the FIRST smallest / largest element as
 //     thrust::minmax_element returns them, which only matters for the sign of
 //     a zero extreme; it is recovered from the first zero of the tensor.
+#include <atomic>
 #include <cstdlib>
 #include <mutex>
 #include <type_traits>
@@ -516,7 +517,17 @@ struct ResArgs {
   uint64_t* bar;         // exchange memory (kBarTotalWords); only ever holds (gen << 32 | key) words
   uint32_t* host_flag;   // pinned host word, set to 1 when the barrier wait expires
   uint64_t spin_limit;
+  uint64_t* stamps;      // measurement aid, normally null: four wall-clock readings per workgroup (phase_stamp below)
+  uint32_t* done;        // pinned host words, one per workgroup: set to `gen` by a workgroup that got through the barrier
 };
+
+// Measurement aid (hpx_terngrad_phase_stamps): while a buffer is set, every workgroup of a resident launch leaves
+// four readings of the 100 MHz wall clock in it: [0] on entry, before its first load is requested; [1] when all its
+// waves have their share loaded and reduced; [2] when it has the global extremes (the grid-wide exchange is behind
+// it); [3] when all its waves have issued their last store.  One scalar branch per reading when no buffer is set.
+__device__ __forceinline__ void phase_stamp(uint64_t* stamps, int k) {
+  if (stamps && threadIdx.x == 0) stamps[size_t(blockIdx.x) * 4 + k] = wall_clock64();
+}
 
 __device__ __forceinline__ void acc_zero(float v, uint32_t idx, float& mn, float& mx, uint32_t& fz) {
   mn = v < mn ? v : mn;
@@ -561,6 +572,7 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
   __shared__ uint32_t s_fz[kWaves];
   __shared__ uint32_t s_q[kBarWaves][4];  // per quarter of the grid: the three keys, then 1 if its wait ended in time
 
+  phase_stamp(a.stamps, 0);
   const float* __restrict__ xp = a.seg.x;
   const uint32_t n = static_cast<uint32_t>(a.seg.n);
   const uint32_t full_units = n / UNIT;
@@ -666,6 +678,7 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
     s_mn[threadIdx.x / kWave] = mn; s_mx[threadIdx.x / kWave] = mx; s_fz[threadIdx.x / kWave] = fz;
   }
   __syncthreads();
+  phase_stamp(a.stamps, 1);
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   if (wave < uint32_t(kBarWaves)) {
     // Each wave that takes part in the exchange folds the workgroup's sixteen results for itself.
@@ -693,6 +706,9 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
     oks &= s_q[q][3];
   }
   if (oks == 0u) return;
+  // this workgroup will write its part of the message: the host may forget the launch once all have said so
+  if (threadIdx.x == 0) __hip_atomic_store(a.done + blockIdx.x, a.gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  phase_stamp(a.stamps, 2);
 
   // ---- pass 2: quantise from registers -------------------------------------------
   mx = from_okey(kx);
@@ -771,6 +787,10 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
     }
     quant_unit_ragged<B, RANDOM>(a.seg, mn, gi, full_units, d);
   }
+  if (a.stamps) {  // uniform
+    __syncthreads();
+    phase_stamp(a.stamps, 3);
+  }
 }
 
 // ---- resident encode of a bucket -------------------------------------------------
@@ -800,6 +820,8 @@ struct ResMultiArgs {
   uint64_t* bar;
   uint32_t* host_flag;
   uint64_t spin_limit;
+  uint64_t* stamps;    // measurement aid, normally null (phase_stamp)
+  uint32_t* done;      // pinned host words, one per workgroup: set to `gen` by a workgroup that got through the barrier
 };
 static_assert(sizeof(ResMultiArgs) <= 9600, "kernel-argument budget");
 
@@ -817,6 +839,7 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_multi_kernel(co
 
   // The wave index is the same in every lane: taken from the first lane, it and all that is derived from it
   // (piece, tensor, bounds) live in scalar registers.
+  phase_stamp(a.stamps, 0);
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x & (kWave - 1);
   const int total = a.piece_start[a.nseg];
   const int my_piece = int(blockIdx.x) * kWaves + int(wave);
@@ -926,6 +949,7 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_multi_kernel(co
     __asm__ volatile("" ::"v"(old));
   }
   __syncthreads();
+  phase_stamp(a.stamps, 1);
   if (wave < uint32_t(kBarWaves)) {
     uint32_t k0 = 0u, k1 = 0u, k2 = 0u;  // the exchange only serves as the barrier here
     const bool ok = grid_exchange(a.bar, a.gen, a.spin_limit, wave, k0, k1, k2);
@@ -938,7 +962,10 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_multi_kernel(co
   uint32_t oks = 1u;
 #pragma unroll
   for (int q = 0; q < kBarWaves; q++) oks &= s_ok[q];
-  if (oks == 0u || !active) return;
+  if (oks == 0u) return;
+  if (threadIdx.x == 0) __hip_atomic_store(a.done + blockIdx.x, a.gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+  if (!active) return;
+  phase_stamp(a.stamps, 2);
 
   // ---- pass 2: the tensor's extremes, then quantise from registers ----------------
   {
@@ -1030,6 +1057,7 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_multi_kernel(co
     }
     quant_unit_ragged<B, RANDOM>(sg, mn, gi, full_units, d);
   }
+  phase_stamp(a.stamps, 3);  // the workgroup's first wave is through (the others hold pieces of the same length)
 }
 
 // The 4*B bits holding the codes of the 4-element group that starts at element e.
@@ -1645,6 +1673,9 @@ int next_barrier_generation(hpx::Workspace* ws, hipStream_t st) {
     // The 32-bit generation wrapped: start over from cleared exchange memory.
     HPX_HIP(hipStreamSynchronize(st));
     HPX_HIP(hipMemset(ws->bar, 0, hpx::kBarWords * sizeof(uint32_t)));
+    // the stream is idle: whatever the log still held has finished, and the workgroups' words start over too
+    if (!hpx::barrier_expired(ws)) ws->resident_log.clear([](hpx::Workspace::ResidentMark) {});
+    for (int w = 0; w < hpx::kBarMaxWorkgroups; w++) ws->done[w] = 0;
     ws->bar_gen = 1;
   }
   return HPX_OK;
@@ -1981,9 +2012,8 @@ int encode_tiled(hpx::Workspace* ws, hipStream_t st, int count, const float* con
 // A barrier kernel on this stream gave up waiting (ws->mu held): barrier kernels are switched off for the
 // stream and every tensor they have encoded since the stream was last known to be good is queued again
 // through the tiled kernels, with the seed it was given the first time, so the same message comes out.
-// Hands an event of a mark back to the workspace's pool.
-inline auto recycle_into(hpx::Workspace* ws) {
-  return [ws](hipEvent_t e) { if (e) ws->event_pool.push_back(e); };
+inline auto recycle_into(hpx::Workspace*) {
+  return [](hpx::Workspace::ResidentMark) {};  // marks own nothing
 }
 
 int repair_resident_log(hpx::Workspace* ws, hipStream_t st) {
@@ -2006,28 +2036,24 @@ int repair_resident_log(hpx::Workspace* ws, hipStream_t st) {
                       t_seed.data());
 }
 
-// Drops the records of earlier calls whose barrier launches have finished with the expiry flag down: their
-// buffers are the caller's again and must not be named by a later repair (ws->mu held, workspace ensured).
+// Drops the records of earlier launches whose workgroups have all come through their barrier, while the
+// expiry flag is down: such a launch will never have to be repeated, its buffers are the caller's again and must
+// not be named by a later repair (ws->mu held, barrier memory ensured).
 void prune_resident_log(hpx::Workspace* ws) {
-  ws->resident_log.prune([](hipEvent_t e) { return hipEventQuery(e) == hipSuccess; },
-                         [ws] { return !hpx::barrier_expired(ws); }, recycle_into(ws));
+  if (!ws->done) return;
+  const volatile uint32_t* done = ws->done;
+  ws->resident_log.prune(
+      [done](hpx::Workspace::ResidentMark m) {
+        for (int w = 0; w < m.grid; w++)
+          if (int32_t(done[w] - m.gen) < 0) return false;  // generations only grow (a wrap clears the words)
+        return true;
+      },
+      [ws] { return !hpx::barrier_expired(ws); }, recycle_into(ws));
 }
 
-// Records an event behind the barrier launches a call has queued and marks the log with it (ws->mu held).
-void mark_resident_log(hpx::Workspace* ws, hipStream_t st) {
-  if (ws->resident_log.empty()) return;
-  hipEvent_t e = nullptr;
-  if (!ws->event_pool.empty()) {
-    e = ws->event_pool.back();
-    ws->event_pool.pop_back();
-  } else if (hipEventCreateWithFlags(&e, hipEventDisableTiming) != hipSuccess) {
-    return;  // no mark: the records stay until a later mark or a wait for the stream covers them
-  }
-  if (hipEventRecord(e, st) != hipSuccess) {
-    ws->event_pool.push_back(e);
-    return;
-  }
-  ws->resident_log.mark(e, recycle_into(ws));
+// Marks the log behind a barrier launch that has just been queued (ws->mu held).
+void mark_resident_log(hpx::Workspace* ws, uint32_t gen, int grid) {
+  ws->resident_log.mark(hpx::Workspace::ResidentMark{gen, grid}, recycle_into(ws));
 }
 
 // Waits for the stream and settles the log of barrier-kernel encodes: cleared if they all got through, encoded
@@ -2074,6 +2100,14 @@ int scratch_address(unsigned long long** out) {
   }
   *out = ptr[dev];
   return HPX_OK;
+}
+
+// Measurement aid: where resident launches leave their phase stamps (null: nowhere).
+std::atomic<uint64_t*> g_phase_stamps{nullptr};
+std::atomic<int32_t> g_phase_capacity{0};
+uint64_t* phase_stamps_for(int grid) {
+  uint64_t* p = g_phase_stamps.load(std::memory_order_relaxed);
+  return p && grid <= g_phase_capacity.load(std::memory_order_relaxed) ? p : nullptr;
 }
 
 constexpr size_t kResidentLogMax = 4096;  // records kept before hpx_terngrad_encode settles the log itself
@@ -2123,11 +2157,6 @@ HPX_API int hpx_terngrad_encode(int count, const float* const* ins, const int32_
     rc = repair_resident_log(ws, st);
     if (rc != HPX_OK) return rc;
   }
-  // whatever this call logs is marked when it returns, on every path
-  struct MarkOnExit {
-    hpx::Workspace* ws; hipStream_t st;
-    ~MarkOnExit() { mark_resident_log(ws, st); }
-  } mark_on_exit{ws, st};
   if (ws->resident_log.size() + size_t(count) > kResidentLogMax) {
     rc = settle_resident_log(ws, st);
     if (rc != HPX_OK) return rc;
@@ -2168,8 +2197,11 @@ HPX_API int hpx_terngrad_encode(int count, const float* const* ins, const int32_
         ma.bar = reinterpret_cast<uint64_t*>(ws->bar);
         ma.host_flag = expired;
         ma.spin_limit = resident_spin_limit();
+        ma.stamps = phase_stamps_for(resident_grid(ws));
+        ma.done = ws->done;
         rc = launch_resident_multi(ma, bitwidths[i], enable_randoms[i] != 0, pre_rows, resident_grid(ws), st);
         if (rc != HPX_OK) return rc;
+        mark_resident_log(ws, ma.gen, resident_grid(ws));
         i = j;
         continue;
       }
@@ -2193,8 +2225,11 @@ HPX_API int hpx_terngrad_encode(int count, const float* const* ins, const int32_
       ra.bar = reinterpret_cast<uint64_t*>(ws->bar);
       ra.host_flag = expired;
       ra.spin_limit = resident_spin_limit();
+      ra.stamps = phase_stamps_for(resident_grid(ws));
+      ra.done = ws->done;
       rc = launch_resident(ra, resident_grid(ws), st);
       if (rc != HPX_OK) return rc;
+      mark_resident_log(ws, ra.gen, resident_grid(ws));
     }
   }
   if (tiled.empty()) return HPX_OK;
@@ -2274,6 +2309,14 @@ HPX_API int hpx_terngrad_encode_status(hpx_stream_t stream) {
   if (!ws->pinned) return HPX_OK;  // nothing has been encoded on this stream
   if (ws->resident_log.empty() && !hpx::barrier_expired(ws)) return HPX_OK;  // no barrier kernel is outstanding
   return settle_resident_log(ws, st);
+}
+
+HPX_API int hpx_terngrad_phase_stamps(uint64_t* device_words, int32_t workgroups) {
+  hpx::clear_error();
+  HPX_ARG(workgroups >= 0 && (device_words || workgroups == 0), "hpx_terngrad_phase_stamps: null buffer");
+  g_phase_capacity.store(device_words ? workgroups : 0, std::memory_order_relaxed);
+  g_phase_stamps.store(workgroups > 0 ? device_words : nullptr, std::memory_order_relaxed);
+  return HPX_OK;
 }
 
 HPX_API int64_t hpx_terngrad_repaired(hpx_stream_t stream) {
