@@ -514,7 +514,9 @@ def x_terngrad_resnet50(torch, np, capi, L, stream, gen, res):
     sec_tiled = timed(torch, r50_step, 50, 10)
     L.hpx_set_option(b"terngrad_resident_bucket", 1)
     msg_bytes = sum(10 + (m_ + 3) // 4 for m_ in r50)
+    phases = terngrad_phases(torch, np, L, r50_step, torch.cuda.get_device_properties(0).multi_processor_count)
     res["terngrad_resnet50_161_tensors"] = {
+        "phases_us": phases,
         "ms_per_step": round(sec * 1e3, 4), "tensors": k_, "launches_per_step": 2,
         "algorithmic_bytes": 8.5 * N_TERNGRAD, "frac_of_hbm_peak": round(8.5 * N_TERNGRAD / sec / 1e9 / HBM_PEAK_GBS, 4),
         "ms_per_step_with_the_two_launch_encode": round(sec_tiled * 1e3, 4),
@@ -550,6 +552,50 @@ def x_terngrad_resnet50(torch, np, capi, L, stream, gen, res):
         "ms": round(sec_root * 1e3, 4), "algorithmic_bytes": alg_root, "frac_of_hbm_peak": round(alg_root / sec_root / 1e9 / HBM_PEAK_GBS, 4),
         "launches_per_call": 1,
         "roofline": kernel_roofline(kt_root, {"terngrad_decode_multi_kernel": alg_root})}
+
+
+def x_terngrad_sizes(torch, np, capi, L, stream, gen, res):
+    # ---- TernGrad 2-bit encode + decode over tensor sizes: which encode a size takes (two launches; one launch
+    # with the tensor on chip; one launch with the tensor's head on chip and the rest streamed twice), kernel
+    # times, step time and fraction of the HBM peak on 8.5 B/elt.  102,760,448 is VGG-16's first fully connected layer.
+    kernels = ["terngrad_resident_kernel", "terngrad_resident_streamed_kernel", "terngrad_minmax_kernel",
+               "terngrad_quant_kernel", "terngrad_decode_kernel"]
+    table = []
+    for n in (1_000_000, 2_000_000, 4_000_000, 6_000_000, 8_000_000, 12_000_000, 16_000_000, 20_000_000, N_TERNGRAD,
+              30_000_000, 33_500_000, 34_000_000, 40_000_000, 48_000_000, 64_000_000, 80_000_000, 102_760_448,
+              128_000_000, 134_000_000, 136_000_000, 160_000_000):
+        nsets = 4 if n < 70_000_000 else 2
+        sets = []
+        for _ in range(nsets):
+            x = torch.randn(n, device="cuda", generator=gen) * 1e-2
+            msg = torch.zeros(10 + (n + 3) // 4, dtype=torch.uint8, device="cuda")
+            dec = torch.empty(n, device="cuda")
+            sets.append((x, msg, dec,
+                         Call(L.hpx_terngrad_encode, 1, capi.ptr_array([x.data_ptr()]), capi.i32_array([n]), capi.ptr_array([msg.data_ptr()]),
+                              capi.i32_array([msg.numel()]), capi.u8_array([2]), capi.i32_array([1]), capi.u64_array([0]), stream),
+                         Call(L.hpx_terngrad_decode, 1, capi.ptr_array([dec.data_ptr()]), capi.i32_array([n]), capi.ptr_array([msg.data_ptr()]),
+                              capi.i32_array([msg.numel()]), capi.i32_array([0]), stream)))
+        state = {"i": 0}
+
+        def step():
+            s_ = sets[state["i"] % nsets]
+            state["i"] += 1
+            s_[3]()
+            s_[4]()
+
+        sec = timed(torch, step, 40, 5)
+        kt = kernel_times(torch, capi, step, kernels, reps=8)
+        path = ("one launch, on chip" if kt["terngrad_resident_kernel"] else
+                "one launch, head on chip, rest streamed twice" if kt["terngrad_resident_streamed_kernel"] else "two launches")
+        enc_us = sum(v for k, v in kt.items() if v and k != "terngrad_decode_kernel") * 1e6
+        table.append({"elements": n, "encode": path, "encode_kernels_us": round(enc_us, 1),
+                      "decode_kernel_us": round((kt["terngrad_decode_kernel"] or 0) * 1e6, 1), "step_us": round(sec * 1e6, 1),
+                      "frac_of_hbm_peak": round(8.5 * n / sec / 1e9 / HBM_PEAK_GBS, 4)})
+        del sets
+        torch.cuda.empty_cache()
+    res["terngrad_size_sweep"] = table
+    big = [r for r in table if r["elements"] == 102_760_448][0]
+    res["terngrad_102M"] = dict(big, algorithmic_bytes=8.5 * 102_760_448, workload="VGG-16 fc6, 2-bit, stochastic rounding, encode + decode(write)")
 
 
 GD_KERNELS = ["gd_sample_kernel", "gd_select_kernel", "gd_threshold_kernel", "gd_stream_kernel", "gd_scan_kernel",
@@ -793,7 +839,8 @@ def x_scheduler(torch, np, capi, L, stream, gen, res):
             "GBps_of_gradient": round(4.0 * float(sum(sizes)) / float(np.median(lat)) / 1e9, 1), "errors": hp.error_count()}
 
 
-EXTRAS = {"tbq": x_tbq, "terngrad_root": x_terngrad_root, "terngrad_resnet50": x_terngrad_resnet50, "dgc": x_dgc,
+EXTRAS = {"tbq": x_tbq, "terngrad_root": x_terngrad_root, "terngrad_resnet50": x_terngrad_resnet50,
+          "terngrad_sizes": x_terngrad_sizes, "dgc": x_dgc,
           "dgc_bucket": x_dgc_bucket, "powersgd": x_powersgd, "scheduler": x_scheduler}
 
 

@@ -83,6 +83,11 @@ int hpx_release_stream(hpx_stream_t stream);
  *                             that may only use some of the CUs (a CU mask)
  *                             must set it to that number: the workgroups of a
  *                             resident launch wait for each other
+ *   "terngrad_resident_streamed" 1 (default): a tensor larger than the chip
+ *                             holds (about 33.5 M elements) also takes ONE
+ *                             launch of that kind: its head stays on chip,
+ *                             the rest is read twice by the same launch;
+ *                             0: such tensors take the two-launch encode
  *   "clock_seed"              what an encoder uses when it is called with
  *                             seeds == NULL; negative (default): the wall
  *                             clock, as the reference's bodies

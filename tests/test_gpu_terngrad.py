@@ -479,6 +479,68 @@ def test_resident_barrier_expiry_is_repaired(tg, oracle_cpu, capi, resident_from
         assert capi.load().hpx_release_workspaces() == 0
 
 
+# ---- tensors larger than the chip: one launch keeps the head on chip and streams the rest twice ----
+def _streamed_case(tg, oracle_cpu, capi, n, b, rnd, seed, expect_streamed=True):
+    gen = torch.Generator(device="cuda").manual_seed(n % 1000 + b)
+    x = torch.randn(n, device="cuda", generator=gen) * 1e-2
+    x[n // 3] = 0.75; x[n - 5] = -0.625                       # extremes in the part kept on chip and in the streamed part
+    L = capi.load()
+    L.hpx_profile_reset(); L.hpx_profile_enable(1)
+    try:
+        out = tg.encode([x], [b], [rnd], [seed])[0]
+        torch.cuda.synchronize()
+        launches = capi.profile_query("terngrad_resident_streamed_kernel")[1]
+    finally:
+        L.hpx_profile_enable(0); L.hpx_profile_reset()
+    assert launches == (1 if expect_streamed else 0), launches
+    xh = host(x)
+    rc, ref = oracle_cpu.terngrad_encode(xh, b, rnd, seed)
+    assert rc == 0
+    assert_bits_equal(host(out), ref, f"message n={n} b={b} rnd={rnd}")
+    del xh, ref
+    return x, out
+
+
+@pytest.mark.parametrize("n", [40_000_000, 64_000_000, 102_760_448])
+@pytest.mark.parametrize("b,rnd", [(2, 1), (2, 0), (8, 1), (8, 0)])
+def test_tensors_larger_than_the_chip(tg, oracle_cpu, capi, n, b, rnd):
+    # 102,760,448 elements is VGG-16's first fully connected layer
+    x, out = _streamed_case(tg, oracle_cpu, capi, n, b, rnd, seed=7 + b)
+    if n == 40_000_000:
+        dec = torch.empty(n, device="cuda")
+        tg.decode([out], [dec], [0])
+        torch.cuda.synchronize()
+        rc, dref = oracle_cpu.terngrad_decode(host(out), n)
+        assert_bits_equal(host(dec), dref, "decode of the streamed encode's message")
+
+
+@pytest.mark.parametrize("b,rnd,n", [(1, 1, 40_000_003), (1, 0, 50_000_001), (4, 1, 36_000_002), (4, 0, 34_000_001),
+                                     (2, 1, 33_554_432 + 4096 + 3), (2, 1, 134_000_001), (1, 1, 23_100_007), (2, 0, 2**27 + 2**25 + 5)])
+def test_streamed_encode_other_widths_ragged_ends_and_the_edges_of_its_range(tg, oracle_cpu, capi, b, rnd, n):
+    # just above what the chip holds (a streamed part of a few rows, most workgroups without one), several times
+    # what it holds, 1-bit codes with random rounding (fewer register rows: the chip holds 23 M), tails n % 8
+    _streamed_case(tg, oracle_cpu, capi, n, b, rnd, seed=2**32 - 9)
+
+
+def test_streamed_encode_zero_sign_and_switch(tg, oracle_cpu, capi):
+    # a zero extreme takes the sign of the FIRST zero of the tensor, wherever it lies: in the streamed part only,
+    # or in both parts; and the option that sends such tensors to the two-launch encode
+    n = 36_000_000
+    for first_zero, sign in ((35_900_017, -0.0), (1234, -0.0), (34_000_000, 0.0)):
+        x = torch.rand(n, device="cuda") * 1e-2 + 1e-3            # all positive: the minimum is the zero
+        x[first_zero] = sign
+        x[35_999_999] = 0.0
+        out = tg.encode([x], [2], [1], [11])[0]
+        torch.cuda.synchronize()
+        rc, ref = oracle_cpu.terngrad_encode(host(x), 2, 1, 11)
+        assert_bits_equal(host(out), ref, f"first zero at {first_zero}")
+    old = capi.set_option("terngrad_resident_streamed", 0)
+    try:
+        _streamed_case(tg, oracle_cpu, capi, 36_000_000, 2, 1, seed=3, expect_streamed=False)
+    finally:
+        capi.set_option("terngrad_resident_streamed", old)
+
+
 def test_repair_leaves_the_buffers_of_finished_calls_alone(tg, oracle_cpu, capi, resident_from_2m):
     # Two single-launch encodes that finish well, no status call; their buffers are then overwritten, as a caller
     # whose allocator hands the memory on would.  A third encode's barrier expires.  The repair must encode the third

@@ -218,6 +218,9 @@ enum Option {
   kOptTerngradResidentWorkgroups,  // "terngrad_resident_workgroups": workgroups of a resident launch; 0 (default) = one per CU.
                                    // For a process that may only use some of the CUs (a CU mask), which the device's CU
                                    // count does not show: a resident launch needs all its workgroups running at once.
+  kOptTerngradResidentStreamed,  // "terngrad_resident_streamed": 1 (default) = a tensor larger than the chip holds also
+                                 // takes the single launch, which keeps the tensor's head on chip and streams the
+                                 // rest twice; 0 = such tensors take the two-launch encode.
   kOptClockSeed,                // "clock_seed": what an encoder called with seeds == NULL uses in place of the wall clock
                                 // (terngrad_body.h:247-251, gd_body.h:138-140); negative (default) = read the clock.
                                 // Makes the C++ drivers, which cannot pass seeds, reproducible.

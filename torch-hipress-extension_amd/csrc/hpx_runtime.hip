@@ -196,6 +196,7 @@ const OptionDef kOptions[kOptCount] = {
     {"terngrad_barrier_ms", "HPX_TERNGRAD_BARRIER_MS", 2000},
     {"terngrad_resident_bucket", "HPX_TERNGRAD_RESIDENT_BUCKET", 1},
     {"terngrad_resident_workgroups", "HPX_TERNGRAD_RESIDENT_WORKGROUPS", 0},
+    {"terngrad_resident_streamed", "HPX_TERNGRAD_RESIDENT_STREAMED", 1},
     {"clock_seed", "HPX_CLOCK_SEED", -1},
 };
 std::atomic<int64_t> g_opt[kOptCount];

@@ -513,6 +513,9 @@ struct ResArgs {
                          // fills them, otherwise just enough of them, so that a smaller share still spreads over all waves
   uint32_t lds_rows;     // rows of kResThreads units kept in LDS
   uint32_t pre_rows;     // register rows whose random addends are prepared during pass 1: 0 or res_pre_rows(bits)
+  uint32_t stream_u0;    // a tensor larger than the chip: the first unit that is NOT kept on chip (= the workgroups'
+                         // shares together); each workgroup streams `stream_units` units from there on twice, once
+  uint32_t stream_units; // for the extremes and once to quantise them; a multiple of kWave.  0: everything is on chip
   uint32_t gen;          // generation of this launch, counted from 1: the tag of its records
   uint64_t* bar;         // exchange memory (kBarTotalWords); only ever holds (gen << 32 | key) words
   uint32_t* host_flag;   // pinned host word, set to 1 when the barrier wait expires
@@ -559,7 +562,15 @@ __device__ __forceinline__ uint32_t quant_unit_prepared(const float4 (&v)[UNIT /
 // PRE: register rows whose random addends are prepared during pass 1 (a compile-time count, so that pass 2
 // stays one straight block the scheduler can interleave across rows; a per-row branch cost as much as the
 // prepared rows saved).
-template <int B, bool RANDOM, int PRE>
+//
+// STREAMED: the tensor is larger than the chip can hold.  The workgroups' shares (the first stream_u0 units) stay on
+// chip as described; the rest is dealt out in contiguous pieces of stream_units units per workgroup and streamed
+// twice by the same launch: before the share is loaded, for its extremes, and after the share has been quantised,
+// to be quantised itself.  The tensor's head is read once, the rest twice: 4 (2 - share/n) bytes per element where
+// the two-launch encode reads 8.
+constexpr int kResStreamIters = 8;  // units per lane and round of a streaming loop (128 KiB per workgroup in flight at 2 bits)
+
+template <int B, bool RANDOM, int PRE, bool STREAMED = false>
 __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const ResArgs a) {
   constexpr int DPB = 8 / B;
   constexpr int UNIT = DPB > 4 ? DPB : 4;
@@ -604,6 +615,35 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
   float4 v[KU][H];
   float4* s_pre = s_rows + size_t(a.lds_rows) * H * kResThreads;
   float mn = __builtin_inff(), mx = -__builtin_inff(), am = __builtin_inff();
+  uint32_t fz = 0xFFFFFFFFu;
+  // The part of the tensor that does not stay on chip, first time through: extremes and first zero only.
+  const uint32_t st_u0 = STREAMED ? a.stream_u0 + blockIdx.x * a.stream_units : 0u;
+  const uint32_t st_lim = st_u0 + (STREAMED ? a.stream_units : 0u);
+  const uint32_t st_end = STREAMED ? (st_u0 >= full_units ? st_u0 : (st_lim < full_units ? st_lim : full_units)) : 0u;
+  if (STREAMED) {
+    for (uint32_t t0 = st_u0; t0 < st_end; t0 += uint32_t(kResStreamIters) * kResThreads) {
+      float4 w[kResStreamIters][H];
+#pragma unroll
+      for (int k = 0; k < kResStreamIters; k++) {
+        const uint32_t u = t0 + k * kResThreads + threadIdx.x;
+#pragma unroll
+        for (int h = 0; h < H; h++)
+          w[k][h] = u < st_end ? ld4_stream(xp + size_t(u) * UNIT + h * 4) : make_float4(qnan, qnan, qnan, qnan);
+      }
+      float amt = __builtin_inff();
+#pragma unroll
+      for (int k = 0; k < kResStreamIters; k++)
+#pragma unroll
+        for (int h = 0; h < H; h++) acc3x4(w[k][h], mn, mx, amt);
+      if (amt == 0.0f) {  // a zero among this lane's elements of the round: note where (rare)
+        float d0 = 0.f, d1 = 0.f;
+#pragma unroll
+        for (int k = 0; k < kResStreamIters; k++)
+#pragma unroll
+          for (int h = 0; h < H; h++) acc_zero4(w[k][h], (t0 + k * kResThreads + threadIdx.x) * UNIT + h * 4, d0, d1, fz);
+      }
+    }
+  }
   const bool whole_rows = wg_u0 + uint32_t(KU * kResThreads) <= wg_end;
   const uint32_t wave_lane0 = __builtin_amdgcn_readfirstlane(threadIdx.x & ~uint32_t(kWave - 1));
   for (uint32_t r = 0; r < a.lds_rows; r++) {
@@ -653,7 +693,6 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
       for (int h = 0; h < H; h++) acc3x4(s_rows[(r * H + h) * kResThreads + threadIdx.x], mn, mx, am);
     }
   }
-  uint32_t fz = 0xFFFFFFFFu;
   if (am == 0.0f) {
     float d0 = 0.f, d1 = 0.f;
 #pragma unroll
@@ -777,6 +816,48 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
       for (int jb = 0; jb < BPU; jb++) pay[size_t(u) * BPU + jb] = uint8_t(packed >> (8 * jb));
     }
   }
+  // The part of the tensor that did not stay on chip, second time through: quantise it.
+  if (STREAMED) {
+    if (RANDOM) {
+      const uint32_t x0 = a.seg.seed + (st_u0 + threadIdx.x) * BPU;
+#pragma unroll
+      for (int q = 0; q < UNIT; q++) {
+        const int jb = q / DPB, j = q % DPB;
+        draw[q] = lcg_mul(j + 2) * (x0 + jb) + lcg_add(j + 2);
+      }
+    }
+    // Two rounds in flight: the loads of the next round are requested before this round is worked on (the waves
+    // of a workgroup leave the barrier together and would otherwise all load, then all compute).
+    constexpr uint32_t kRound = uint32_t(kResStreamIters) * kResThreads;
+    float4 w0[kResStreamIters][H], w1[kResStreamIters][H];
+    auto fetch = [&](float4 (&w)[kResStreamIters][H], uint32_t t0) {
+#pragma unroll
+      for (int k = 0; k < kResStreamIters; k++) {
+        const uint32_t u = t0 + k * kResThreads + threadIdx.x;
+#pragma unroll
+        for (int h = 0; h < H; h++)
+          w[k][h] = (t0 < st_end && u < st_end) ? ld4_stream(xp + size_t(u) * UNIT + h * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+    };
+    auto emit = [&](float4 (&w)[kResStreamIters][H], uint32_t t0) {
+#pragma unroll
+      for (int k = 0; k < kResStreamIters; k++) {
+        const uint32_t u = t0 + k * kResThreads + threadIdx.x;
+        const uint32_t packed = quant_unit<B, RANDOM>(w[k], mn, gi, draw, uint32_t(kResThreads) * BPU);
+        if (u < st_end) {
+#pragma unroll
+          for (int jb = 0; jb < BPU; jb++) pay[size_t(u) * BPU + jb] = uint8_t(packed >> (8 * jb));
+        }
+      }
+    };
+    fetch(w0, st_u0);
+    for (uint32_t t0 = st_u0; t0 < st_end; t0 += 2 * kRound) {
+      fetch(w1, t0 + kRound);
+      emit(w0, t0);
+      fetch(w0, t0 + 2 * kRound);
+      if (t0 + kRound < st_end) emit(w1, t0 + kRound);
+    }
+  }
   // The unit that holds the end of the tensor, if the length is not a whole number of units.
   if (blockIdx.x == 0 && threadIdx.x == 0 && full_units * UNIT < n) {
     uint32_t d[UNIT];
@@ -798,7 +879,10 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
 // reads every tensor once.  The unit of work is a piece: `rows` rows of 64 units of
 // one tensor, held by one wave (register rows first, LDS rows after them), so the
 // tensor, its extremes and its seed are wave-uniform and the inner loops are those
-// of the single-tensor kernel.  Piece p belongs to wave p % 16 of workgroup p / 16;
+// of the single-tensor kernel.  Piece p belongs to wave p / G of workgroup p % G (G workgroups):
+// consecutive pieces go to consecutive workgroups, so every CU gets the same mix of whole pieces,
+// tensor ends and tiny tensors (with piece p on wave p % 16 of workgroup p / 16 the workgroups that
+// held sixteen whole pieces of a large tensor set the pace of both passes);
 // the host picks the smallest `rows` for which all pieces fit (every tensor has at
 // least one piece; the piece that ends a tensor also takes the 1..UNIT-1 elements
 // behind its last whole unit).
@@ -842,7 +926,7 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_multi_kernel(co
   phase_stamp(a.stamps, 0);
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x & (kWave - 1);
   const int total = a.piece_start[a.nseg];
-  const int my_piece = int(blockIdx.x) * kWaves + int(wave);
+  const int my_piece = int(wave) * int(gridDim.x) + int(blockIdx.x);
   const bool active = my_piece < total;           // wave-uniform
   const int piece = active ? my_piece : total - 1;  // an idle wave looks at the last piece and touches nothing
   const int s = __builtin_amdgcn_readfirstlane(find_segment<kCapLarge>(a.piece_start, a.nseg, piece));
@@ -1057,7 +1141,11 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_multi_kernel(co
     }
     quant_unit_ragged<B, RANDOM>(sg, mn, gi, full_units, d);
   }
-  phase_stamp(a.stamps, 3);  // the workgroup's first wave is through (the others hold pieces of the same length)
+  // the last of the workgroup's waves to get here leaves the reading (the waves hold pieces of different tensors
+  // and lengths and no barrier joins them again)
+  if (a.stamps && lane == 0)
+    __hip_atomic_fetch_max(reinterpret_cast<unsigned long long*>(a.stamps) + size_t(blockIdx.x) * 4 + 3,
+                           static_cast<unsigned long long>(wall_clock64()), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // The 4*B bits holding the codes of the 4-element group that starts at element e.
@@ -1605,18 +1693,36 @@ int resident_grid(const hpx::Workspace* ws) {
   return (cap > 0 && cap < ws->num_cus) ? int(cap) : ws->num_cus;
 }
 
-// Fills chunk_units / lds_rows when tensor (n, bits) fits the chip; false otherwise.
+// Fills chunk_units / lds_rows when tensor (n, bits) fits the chip, and the streamed part as well when it is
+// larger (the single launch then keeps the tensor's head on chip and streams the rest twice; measured against the
+// two launches of small workgroups it stays ahead at every size: 160 M elements 205 against 228 us, 260 M 342
+// against 369); false when the single launch is not to be used.
 bool resident_plan(int32_t n, int bits, bool random, const hpx::Workspace* ws, ResArgs& ra) {
   const int64_t min_elems = hpx::option(hpx::kOptTerngradResidentMin);
   if (min_elems < 0 || n < min_elems || resident_grid(ws) <= 0 || resident_grid(ws) > kBarMaxWorkgroups) return false;
   const int unit = (8 / bits) > 4 ? (8 / bits) : 4;
   const int h = unit / 4;
   const int64_t full_units = n / unit;
-  const int64_t per_wg = (full_units + resident_grid(ws) - 1) / resident_grid(ws);
+  const int64_t grid = resident_grid(ws);
+  const int64_t per_wg = (full_units + grid - 1) / grid;
   int64_t rows = (per_wg + kResThreads - 1) / kResThreads;
   if (rows < 1) rows = 1;
   const int reg_rows = res_reg_groups(bits, random) / h, lds_rows_max = kResLdsGroups / h;
-  if (rows > reg_rows + lds_rows_max) return false;
+  ra.stream_u0 = 0u;
+  ra.stream_units = 0u;
+  if (rows > reg_rows + lds_rows_max) {
+    // Larger than the chip: every workgroup keeps a full share, the rest is streamed.
+    const int64_t share = int64_t(reg_rows + lds_rows_max) * kResThreads;
+    if (hpx::option(hpx::kOptTerngradResidentStreamed) == 0) return false;
+    const int64_t rest = full_units - share * grid;
+    ra.chunk_units = static_cast<uint32_t>(share);
+    ra.reg_rows = static_cast<uint32_t>(reg_rows);
+    ra.lds_rows = static_cast<uint32_t>(lds_rows_max);
+    ra.pre_rows = 0u;
+    ra.stream_u0 = static_cast<uint32_t>(share * grid);
+    ra.stream_units = static_cast<uint32_t>(((rest + grid - 1) / grid + kWave - 1) / kWave * kWave);
+    return true;
+  }
   // The share itself is only rounded up to whole waves' worth of units, so that every CU has one (rounded to
   // whole rows, the headline tensor's 24.4 rows per workgroup became 25 rows for 250 workgroups and none for six).
   ra.chunk_units = static_cast<uint32_t>((per_wg + kWave - 1) / kWave * kWave);
@@ -1627,7 +1733,7 @@ bool resident_plan(int32_t n, int bits, bool random, const hpx::Workspace* ws, R
   return true;
 }
 
-template <int B, bool RANDOM, int PRE>
+template <int B, bool RANDOM, int PRE, bool STREAMED = false>
 int launch_resident_as(const ResArgs& ra, int num_cus, hipStream_t st) {
   constexpr int H = ((8 / B) > 4 ? (8 / B) : 4) / 4;
   // The dynamic-LDS limit is a property of the function on one device: raise it once per device.
@@ -1638,21 +1744,23 @@ int launch_resident_as(const ResArgs& ra, int num_cus, hipStream_t st) {
     HPX_HIP(hipGetDevice(&dev));
     std::lock_guard<std::mutex> g(attr_mu);
     if (dev >= 64 || !(attr_done >> dev & 1)) {
-      HPX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&terngrad_resident_kernel<B, RANDOM, PRE>),
+      HPX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&terngrad_resident_kernel<B, RANDOM, PRE, STREAMED>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize,
                                   kResLdsTotalGroups * kResThreads * int(sizeof(float4))));
       if (dev < 64) attr_done |= uint64_t(1) << dev;
     }
   }
   const size_t lds = size_t(ra.lds_rows + PRE) * H * kResThreads * sizeof(float4);
-  HPX_LAUNCH_LDS("terngrad_resident_kernel", hpx::g_prof_on, (terngrad_resident_kernel<B, RANDOM, PRE>), dim3(num_cus),
-                 dim3(kResThreads), lds, st, ra);
+  HPX_LAUNCH_LDS(STREAMED ? "terngrad_resident_streamed_kernel" : "terngrad_resident_kernel", hpx::g_prof_on,
+                 (terngrad_resident_kernel<B, RANDOM, PRE, STREAMED>), dim3(num_cus), dim3(kResThreads), lds, st, ra);
   HPX_HIP(hipGetLastError());
   return HPX_OK;
 }
 
 template <int B>
 int launch_resident_bits(const ResArgs& ra, int num_cus, hipStream_t st) {
+  if (ra.stream_units)
+    return ra.seg.random ? launch_resident_as<B, true, 0, true>(ra, num_cus, st) : launch_resident_as<B, false, 0, true>(ra, num_cus, st);
   if (!ra.seg.random) return launch_resident_as<B, false, 0>(ra, num_cus, st);
   if (ra.pre_rows) return launch_resident_as<B, true, res_pre_rows(B)>(ra, num_cus, st);
   return launch_resident_as<B, true, 0>(ra, num_cus, st);
@@ -1737,10 +1845,11 @@ bool resident_multi_plan(int count, const int32_t* in_sizes, const uint8_t* bitw
   if (rows > reg_rows + lds_rows_max) return false;
   ma.rows = static_cast<uint32_t>(rows);
   ma.lds_rows = rows > reg_rows ? static_cast<uint32_t>(rows - reg_rows) : 0u;
-  // prepared rows: the full set, or half of it when the tensors' LDS rows leave no room for more
+  // prepared rows: the full set, or three quarters or half of it when the tensors' LDS rows leave no room for more
   const int spare_rows = (kResLdsTotalGroups - int(ma.lds_rows) * h) / h;
   pre_rows = 0u;
   if (random && spare_rows >= res_pre_rows(bits)) pre_rows = static_cast<uint32_t>(res_pre_rows(bits));
+  else if (random && spare_rows >= res_pre_rows(bits) * 3 / 4) pre_rows = static_cast<uint32_t>(res_pre_rows(bits) * 3 / 4);
   else if (random && spare_rows >= res_pre_rows(bits) / 2) pre_rows = static_cast<uint32_t>(res_pre_rows(bits) / 2);
   ma.nseg = count;
   ma.piece_start[0] = 0;
@@ -1778,6 +1887,7 @@ template <int B>
 int launch_resident_multi_bits(const ResMultiArgs& ma, bool random, uint32_t pre_rows, int num_cus, hipStream_t st) {
   if (!random) return launch_resident_multi_as<B, false, 0>(ma, num_cus, st);
   if (pre_rows == uint32_t(res_pre_rows(B))) return launch_resident_multi_as<B, true, res_pre_rows(B)>(ma, num_cus, st);
+  if (pre_rows == uint32_t(res_pre_rows(B) * 3 / 4)) return launch_resident_multi_as<B, true, res_pre_rows(B) * 3 / 4>(ma, num_cus, st);
   if (pre_rows == uint32_t(res_pre_rows(B) / 2)) return launch_resident_multi_as<B, true, res_pre_rows(B) / 2>(ma, num_cus, st);
   return launch_resident_multi_as<B, true, 0>(ma, num_cus, st);
 }
