@@ -168,10 +168,29 @@ def test_more_matrices_than_one_table(psgd):
     _run_case(psgd, shapes, rng)
 
 
-def test_rank_above_limit_is_rejected(psgd):
-    n, m, r = 8, 8, 17
-    t = lambda *s: torch.zeros(*s, device="cuda")
-    psgd.encode1([t(n * m)], [t(n * m)], [t(m, r)], [t(n, m)], [t(n, r)], expect_rc=-3)
+def test_ranks_above_sixteen(psgd):
+    # The reference takes any rank (plain mm, powersgd_body.h:28,49,69; `matrix_approximation_rank`, hp_cuda.cpp:849).
+    # Here a rank above 16 goes sixteen columns per pass over the matrix: ranks that end inside a block, on its edge,
+    # several blocks, a factor too large for the LDS orthonormalisation, mixed with small ranks in one batch, with
+    # padding, over two iterations.
+    rng = np.random.default_rng(17)
+    shapes = [(300, 260, 17, 0), (257, 513, 32, 5), (700, 300, 64, 0), (128, 90, 33, 3), (40, 1200, 20, 0), (64, 64, 4, 0),
+              (1100, 70, 48, 1)]
+    _run_case(psgd, shapes, rng, iterations=2)
+    for shape in ((300, 260, 17, 0), (2048, 1024, 32, 0), (1024, 2048, 64, 7)):
+        _run_case(psgd, [shape], rng)
+
+
+def test_rank_r_matrix_of_rank_forty_is_reproduced(psgd):
+    rng = np.random.default_rng(31)
+    n, m, r = 640, 512, 40
+    Mtrue = (rng.normal(0, 1, (n, r)) @ rng.normal(0, 1, (m, r)).T).astype(np.float32)
+    g = dev(Mtrue.reshape(-1).copy()); res = torch.zeros(n * m, device="cuda")
+    Q = dev(rng.normal(0, 1, (m, r)).astype(np.float32)); M = torch.zeros(n, m, device="cuda"); P = torch.zeros(n, r, device="cuda")
+    psgd.encode1([g], [res], [Q], [M], [P]); psgd.encode2([P], [M], [Q]); psgd.decode([P], [Q], [M], [res], [g])
+    torch.cuda.synchronize()
+    assert ps.rel_fro(host(M), Mtrue) < 1e-5
+    assert float(res.norm()) < 1e-4 * float(np.linalg.norm(Mtrue))
 
 
 def test_config4_layer_set(psgd):

@@ -14,7 +14,11 @@
 // Operand layout of that instruction: A[blk][i] in lane 4*blk+i, B[blk][j] in
 // lane 4*blk+j, D[blk][i][j] in lane 4*blk+j, register i.
 //
-// Ranks up to 16 are handled as up to four column groups of four.
+// Ranks up to 16 are handled as up to four column groups of four in one pass over the data.  Larger ranks
+// (the reference takes any, powersgd_body.h:28,49,69) go sixteen columns at a time: every pass names a block
+// of columns of P and Q by an offset pointer, the block's width `r` and the factors' row stride `ld`; encode1
+// stores M in its first pass and reads it back in the others, decode builds M up over its passes and writes the
+// residual and the gradient in the last.
 #include "hpx_common.h"
 
 namespace {
@@ -42,7 +46,12 @@ struct Seg {
   int64_t numel;
   int32_t n, m, r;
   int32_t part_off;    // encode2: offset (in floats / 4) of this matrix's partials
+  int32_t ld;          // row stride of P and Q (the full rank; r is the width of the block of columns at hand)
+  int32_t mode;        // kFromM | kOntoM | kKeepGrad, for the passes of a rank above 16
 };
+constexpr int32_t kFromM = 1;    // encode1: M has been stored by an earlier pass: read it instead of grad + residual
+constexpr int32_t kOntoM = 2;    // decode: add this block's P Q^T to what M holds instead of starting from zero
+constexpr int32_t kKeepGrad = 4; // decode: more blocks follow: write M only, leave residual and gradient alone
 struct Args {
   int32_t nseg;
   int32_t tile_start[kMaxSeg + 1];
@@ -68,7 +77,8 @@ __global__ __launch_bounds__(kThreads) void psgd_encode1_kernel(const Args a) {
   const float* __restrict__ R = sg.res;
   const float* __restrict__ Q = sg.Q;
   float* __restrict__ M = sg.M;
-  const int n = sg.n, m = sg.m, r = sg.r;
+  const int n = sg.n, m = sg.m, r = sg.r, ld = sg.ld;
+  const bool from_m = (sg.mode & kFromM) != 0;
   const int64_t N = sg.numel;
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int row0 = (tile - a.tile_start[s]) * 4;
@@ -95,8 +105,8 @@ __global__ __launch_bounds__(kThreads) void psgd_encode1_kernel(const Args a) {
 #pragma unroll
       for (int u = 0; u < kUnroll; u++) {
         const int64_t f = int64_t(row) * m + k0 + 64 * u + 4 * b;
-        g4[u] = ld4_stream(G + f);
-        r4[u] = ld4_stream(R + f);
+        g4[u] = from_m ? ld4_stream(M + f) : ld4_stream(G + f);
+        r4[u] = from_m ? make_float4(0.f, 0.f, 0.f, 0.f) : ld4_stream(R + f);
       }
 #pragma unroll
       for (int u = 0; u < kUnroll; u++)
@@ -105,13 +115,13 @@ __global__ __launch_bounds__(kThreads) void psgd_encode1_kernel(const Args a) {
 #pragma unroll
           for (int c = 0; c < CG; c++) {
             const int col = c * 4 + i;  // B operand: lane 4b+j holds Q[k][j]
-            q[u][t][c] = col < r ? Q[int64_t(k0 + 64 * u + 4 * b + t) * r + col] : 0.f;
+            q[u][t][c] = col < r ? Q[int64_t(k0 + 64 * u + 4 * b + t) * ld + col] : 0.f;
           }
 #pragma unroll
       for (int u = 0; u < kUnroll; u++) {
         const int64_t f = int64_t(row) * m + k0 + 64 * u + 4 * b;
         const float4 m4 = make_float4(g4[u].x + r4[u].x, g4[u].y + r4[u].y, g4[u].z + r4[u].z, g4[u].w + r4[u].w);
-        st4_stream(M + f, m4);  // the set of M matrices is far larger than the caches: do not allocate
+        if (!from_m) st4_stream(M + f, m4);  // the set of M matrices is far larger than the caches: do not allocate
         const float v[4] = {m4.x, m4.y, m4.z, m4.w};
 #pragma unroll
         for (int t = 0; t < 4; t++)
@@ -125,9 +135,10 @@ __global__ __launch_bounds__(kThreads) void psgd_encode1_kernel(const Args a) {
     float v[4];
     if (rows_full && k0 + 64 <= m) {
       const int64_t f = int64_t(row) * m + kk;
-      const float4 g4 = ld4_stream(G + f), r4 = ld4_stream(R + f);
+      const float4 g4 = from_m ? ld4_stream(M + f) : ld4_stream(G + f);
+      const float4 r4 = from_m ? make_float4(0.f, 0.f, 0.f, 0.f) : ld4_stream(R + f);
       const float4 m4 = make_float4(g4.x + r4.x, g4.y + r4.y, g4.z + r4.z, g4.w + r4.w);
-      st4(M + f, m4);
+      if (!from_m) st4(M + f, m4);
       v[0] = m4.x; v[1] = m4.y; v[2] = m4.z; v[3] = m4.w;
     } else {
 #pragma unroll
@@ -136,7 +147,7 @@ __global__ __launch_bounds__(kThreads) void psgd_encode1_kernel(const Args a) {
         float x = 0.f;
         if (row < n && k < m) {
           const int64_t f = int64_t(row) * m + k;
-          if (f < N) {
+          if (f < N && !from_m) {
             x = G[f] + R[f];
             M[f] = x;
           } else {
@@ -152,7 +163,7 @@ __global__ __launch_bounds__(kThreads) void psgd_encode1_kernel(const Args a) {
 #pragma unroll
       for (int c = 0; c < CG; c++) {
         const int col = c * 4 + i;  // B operand: lane 4b+j holds Q[k][j]
-        const float q = (k < m && col < r) ? Q[int64_t(k) * r + col] : 0.f;
+        const float q = (k < m && col < r) ? Q[int64_t(k) * ld + col] : 0.f;
         acc[c] = mfma4(v[t], q, acc[c]);
       }
     }
@@ -176,7 +187,7 @@ __global__ __launch_bounds__(kThreads) void psgd_encode1_kernel(const Args a) {
       float x = s_p[0][c][ii][j];
 #pragma unroll
       for (int w = 1; w < kWaves; w++) x += s_p[w][c][ii][j];
-      sg.P[int64_t(row0 + ii) * r + col] = x;
+      sg.P[int64_t(row0 + ii) * ld + col] = x;
     }
   }
 }
@@ -270,7 +281,7 @@ __global__ __launch_bounds__(kThreads) void psgd_mtp_kernel(const Args a) {
   const Seg& sg = a.seg[s];
   const float* __restrict__ M = sg.M;
   const float* __restrict__ P = sg.P;
-  const int n = sg.n, m = sg.m, r = sg.r;
+  const int n = sg.n, m = sg.m, r = sg.r, ld = sg.ld;
   const int strips = (m + kStrip - 1) / kStrip;
   const int t_in = tile - a.tile_start[s];
   const int strip = t_in % strips, rblk = t_in / strips;
@@ -301,7 +312,7 @@ __global__ __launch_bounds__(kThreads) void psgd_mtp_kernel(const Args a) {
 #pragma unroll
       for (int u = 0; u < kRows; u++)
 #pragma unroll
-        for (int c = 0; c < CG; c++) p[u][c] = (c * 4 + j) < r ? P[int64_t(row + u) * r + c * 4 + j] : 0.f;
+        for (int c = 0; c < CG; c++) p[u][c] = (c * 4 + j) < r ? P[int64_t(row + u) * ld + c * 4 + j] : 0.f;
 #pragma unroll
       for (int u = 0; u < kRows; u++) {
         const float v[4] = {m4[u].x, m4[u].y, m4[u].z, m4[u].w};
@@ -324,7 +335,7 @@ __global__ __launch_bounds__(kThreads) void psgd_mtp_kernel(const Args a) {
 #pragma unroll
     for (int c = 0; c < CG; c++) {
       const int col = c * 4 + j;
-      const float p = col < r ? P[int64_t(row) * r + col] : 0.f;
+      const float p = col < r ? P[int64_t(row) * ld + col] : 0.f;
 #pragma unroll
       for (int t = 0; t < 4; t++) acc[c][t] = mfma4(v[t], p, acc[c][t]);
     }
@@ -362,7 +373,7 @@ __global__ __launch_bounds__(kThreads) void psgd_qreduce_kernel(const Args a) {
   if (e < mr) {
     float x = 0.f;
     for (int p = 0; p < nparts; p++) x += part[int64_t(p) * mr + e];
-    sg.Qout[e] = x;
+    sg.Qout[(e / sg.r) * sg.ld + e % sg.r] = x;
   }
 }
 
@@ -382,7 +393,8 @@ __global__ __launch_bounds__(kThreads) void psgd_decode_kernel(const Args a) {
   float* __restrict__ M = sg.M;
   float* __restrict__ G = const_cast<float*>(sg.grad);
   float* __restrict__ R = const_cast<float*>(sg.res);
-  const int n = sg.n, m = sg.m, r = sg.r;
+  const int n = sg.n, m = sg.m, r = sg.r, ld = sg.ld;
+  const bool onto_m = (sg.mode & kOntoM) != 0, keep_grad = (sg.mode & kKeepGrad) != 0;
   const int64_t N = sg.numel;
   const int strips = (m + kStrip - 1) / kStrip;
   const int t_in = tile - a.tile_start[s];
@@ -399,7 +411,7 @@ __global__ __launch_bounds__(kThreads) void psgd_decode_kernel(const Args a) {
 #pragma unroll
   for (int t = 0; t < 4; t++)
 #pragma unroll
-    for (int col = 0; col < CG * 4; col++) q[t][col] = (kk + t < m && col < r) ? Q[int64_t(kk + t) * r + col] : 0.f;
+    for (int col = 0; col < CG * 4; col++) q[t][col] = (kk + t < m && col < r) ? Q[int64_t(kk + t) * ld + col] : 0.f;
 
   const bool cols_full = k0 + kStrip <= m;
   for (int row0 = rbeg; row0 < rend; row0 += 4) {
@@ -412,9 +424,16 @@ __global__ __launch_bounds__(kThreads) void psgd_decode_kernel(const Args a) {
     f32x4 acc[4];
 #pragma unroll
     for (int t = 0; t < 4; t++) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (onto_m) {  // a later block of columns of a rank above 16: go on from what the earlier blocks left in M
+#pragma unroll
+      for (int ii = 0; ii < 4; ii++)
+#pragma unroll
+        for (int t = 0; t < 4; t++)
+          if (row0 + ii < rend && kk + t < m) acc[t][ii] = M[int64_t(row0 + ii) * m + kk + t];
+    }
 #pragma unroll
     for (int col = 0; col < CG * 4; col++) {
-      const float p = (row0 + i < n && col < r) ? P[int64_t(row0 + i) * r + col] : 0.f;
+      const float p = (row0 + i < n && col < r) ? P[int64_t(row0 + i) * ld + col] : 0.f;
 #pragma unroll
       for (int t = 0; t < 4; t++) acc[t] = mfma4(p, q[t][col], acc[t]);
     }
@@ -424,8 +443,10 @@ __global__ __launch_bounds__(kThreads) void psgd_decode_kernel(const Args a) {
         const int64_t f = int64_t(row0 + ii) * m + kk;
         const float4 m4 = make_float4(acc[0][ii], acc[1][ii], acc[2][ii], acc[3][ii]);
         const float4 r4 = make_float4(g4[ii].x - m4.x, g4[ii].y - m4.y, g4[ii].z - m4.z, g4[ii].w - m4.w);
-        st4_stream(R + f, r4);
-        st4_stream(G + f, m4);  // in place over the line just read
+        if (!keep_grad) {
+          st4_stream(R + f, r4);
+          st4_stream(G + f, m4);  // in place over the line just read
+        }
         st4(M + f, m4);  // plain: streaming this third store was measurably slower
       }
       continue;
@@ -439,7 +460,7 @@ __global__ __launch_bounds__(kThreads) void psgd_decode_kernel(const Args a) {
 #pragma unroll
       for (int t = 0; t < 4; t++) {
         if (kk + t < m) {
-          if (f + t < N) {
+          if (f + t < N && !keep_grad) {
             R[f + t] = G[f + t] - mv[t];
             G[f + t] = mv[t];
           }
@@ -457,18 +478,20 @@ struct Batch {
   const int32_t *ns, *ms, *rs;
 };
 
-int check_dims(const char* who, const Batch& b, int* max_cg) {
-  *max_cg = 1;
+constexpr int kPassCols = 4 * kMaxCG;  // columns of the factors one pass over the data handles
+
+int check_dims(const char* who, const Batch& b, int* max_rank) {
+  *max_rank = 1;
   for (int i = 0; i < b.count; i++) {
     HPX_ARG(b.ns[i] > 0 && b.ms[i] > 0 && b.rs[i] > 0, "%s: matrix %d has dims %d x %d rank %d", who, i, b.ns[i], b.ms[i],
             b.rs[i]);
-    HPX_ARG(b.rs[i] <= 4 * kMaxCG, "%s: matrix %d has rank %d; ranks above %d are not supported", who, i, b.rs[i],
-            4 * kMaxCG);
-    const int cg = (b.rs[i] + 3) / 4;
-    if (cg > *max_cg) *max_cg = cg;
+    if (b.rs[i] > *max_rank) *max_rank = b.rs[i];
   }
   return HPX_OK;
 }
+// The block of columns [c0, c0 + kPassCols) of a rank-r factor: its width (0: the matrix has no such block) and
+// the column groups of four it needs.
+inline int block_cols(int r, int c0) { return r <= c0 ? 0 : (r - c0 < kPassCols ? r - c0 : kPassCols); }
 
 #define PSGD_LAUNCH_CG_LDS(KERNEL, cg, grid, lds, st, args)                                                         \
   switch (cg) {                                                                                                     \
@@ -489,8 +512,8 @@ HPX_API int hpx_powersgd_encode1(int count, const float* const* grads, const int
   HPX_ARG(count >= 0, "hpx_powersgd_encode1: negative count");
   if (count == 0) return HPX_OK;
   HPX_ARG(grads && numels && residuals && Qs && Ms && Ps && ns && ms && rs, "hpx_powersgd_encode1: null argument array");
-  int cg = 1;
-  int rc = check_dims("hpx_powersgd_encode1", Batch{count, ns, ms, rs}, &cg);
+  int max_rank = 1;
+  int rc = check_dims("hpx_powersgd_encode1", Batch{count, ns, ms, rs}, &max_rank);
   if (rc != HPX_OK) return rc;
   for (int i = 0; i < count; i++) {
     HPX_ARG(grads[i] && residuals[i] && Qs[i] && Ms[i] && Ps[i], "hpx_powersgd_encode1: matrix %d has a null pointer", i);
@@ -500,20 +523,28 @@ HPX_API int hpx_powersgd_encode1(int count, const float* const* grads, const int
   hipStream_t st = static_cast<hipStream_t>(stream);
   Args a;
   a.partials = nullptr;
-  int i = 0;
-  while (i < count) {
-    a.nseg = 0;
-    a.tile_start[0] = 0;
-    while (i < count && a.nseg < kMaxSeg) {
-      const int32_t t = cdiv(ns[i], 4);
-      if (int64_t(a.tile_start[a.nseg]) + t > INT32_MAX) break;
-      a.seg[a.nseg] = Seg{grads[i], residuals[i], Qs[i], Ms[i], Ps[i], nullptr, numels[i], ns[i], ms[i], rs[i], 0};
-      a.tile_start[a.nseg + 1] = a.tile_start[a.nseg] + t;
-      a.nseg++;
-      i++;
+  for (int c0 = 0; c0 < max_rank; c0 += kPassCols) {
+    int i = 0;
+    while (i < count) {
+      a.nseg = 0;
+      a.tile_start[0] = 0;
+      int cg = 1;
+      while (i < count && a.nseg < kMaxSeg) {
+        const int rb = block_cols(rs[i], c0);
+        if (rb == 0) { i++; continue; }
+        const int32_t t = cdiv(ns[i], 4);
+        if (int64_t(a.tile_start[a.nseg]) + t > INT32_MAX) break;
+        a.seg[a.nseg] = Seg{grads[i], residuals[i], Qs[i] + c0, Ms[i], Ps[i] + c0, nullptr, numels[i], ns[i], ms[i], rb, 0,
+                            rs[i], c0 ? kFromM : 0};
+        if ((rb + 3) / 4 > cg) cg = (rb + 3) / 4;
+        a.tile_start[a.nseg + 1] = a.tile_start[a.nseg] + t;
+        a.nseg++;
+        i++;
+      }
+      if (a.nseg == 0) continue;
+      PSGD_LAUNCH_CG(psgd_encode1_kernel, cg, a.tile_start[a.nseg], st, a);
+      HPX_HIP(hipGetLastError());
     }
-    PSGD_LAUNCH_CG(psgd_encode1_kernel, cg, a.tile_start[a.nseg], st, a);
-    HPX_HIP(hipGetLastError());
   }
   return HPX_OK;
 }
@@ -524,13 +555,13 @@ HPX_API int hpx_powersgd_encode2(int count, float* const* Ps, const float* const
   HPX_ARG(count >= 0, "hpx_powersgd_encode2: negative count");
   if (count == 0) return HPX_OK;
   HPX_ARG(Ps && Ms && Qs && ns && ms && rs, "hpx_powersgd_encode2: null argument array");
-  int cg = 1;
-  int rc = check_dims("hpx_powersgd_encode2", Batch{count, ns, ms, rs}, &cg);
+  int max_rank = 1;
+  int rc = check_dims("hpx_powersgd_encode2", Batch{count, ns, ms, rs}, &max_rank);
   if (rc != HPX_OK) return rc;
-  int64_t part_quads = 0;  // partial storage in units of 4 floats
+  int64_t part_quads = 0;  // partial storage in units of 4 floats (one pass at a time uses it)
   for (int i = 0; i < count; i++) {
     HPX_ARG(Ps[i] && Ms[i] && Qs[i], "hpx_powersgd_encode2: matrix %d has a null pointer", i);
-    part_quads += (int64_t(cdiv(ns[i], kE2RowsPerBlock)) * ms[i] * rs[i] + 3) / 4;
+    part_quads += (int64_t(cdiv(ns[i], kE2RowsPerBlock)) * ms[i] * block_cols(rs[i], 0) + 3) / 4;
   }
   HPX_ARG(part_quads <= INT32_MAX, "hpx_powersgd_encode2: batch too large for one call");
   hipStream_t st = static_cast<hipStream_t>(stream);
@@ -541,29 +572,14 @@ HPX_API int hpx_powersgd_encode2(int count, float* const* Ps, const float* const
   if (rc != HPX_OK) return rc;
   Args a;
   a.partials = reinterpret_cast<float*>(ws->dev);
-  int i = 0;
-  int64_t poff = 0;
-  while (i < count) {
-    const int first = i;
+  // step 1: orthonormalise every P over all of its columns
+  for (int i = 0; i < count;) {
     a.nseg = 0;
-    a.tile_start[0] = 0;
-    int32_t red_start[kMaxSeg + 1];
-    red_start[0] = 0;
-    while (i < count && a.nseg < kMaxSeg) {
-      const int32_t t = cdiv(ms[i], kStrip) * cdiv(ns[i], kE2RowsPerBlock);
-      const int32_t tr = cdiv(int64_t(ms[i]) * rs[i], kThreads);
-      if (int64_t(a.tile_start[a.nseg]) + t > INT32_MAX || int64_t(red_start[a.nseg]) + tr > INT32_MAX) break;
-      a.seg[a.nseg] = Seg{nullptr, nullptr, nullptr, const_cast<float*>(Ms[i]), Ps[i], Qs[i], 0, ns[i], ms[i], rs[i],
-                          static_cast<int32_t>(poff)};
-      poff += (int64_t(cdiv(ns[i], kE2RowsPerBlock)) * ms[i] * rs[i] + 3) / 4;
-      a.tile_start[a.nseg + 1] = a.tile_start[a.nseg] + t;
-      red_start[a.nseg + 1] = red_start[a.nseg] + tr;
-      a.nseg++;
-      i++;
-    }
-    (void)first;
     int64_t max_nr = 0;
-    for (int k = 0; k < a.nseg; k++) max_nr = int64_t(a.seg[k].n) * a.seg[k].r > max_nr ? int64_t(a.seg[k].n) * a.seg[k].r : max_nr;
+    for (; i < count && a.nseg < kMaxSeg; i++) {
+      a.seg[a.nseg++] = Seg{nullptr, nullptr, nullptr, nullptr, Ps[i], nullptr, 0, ns[i], ms[i], rs[i], 0, rs[i], 0};
+      if (int64_t(ns[i]) * rs[i] > max_nr) max_nr = int64_t(ns[i]) * rs[i];
+    }
     if (max_nr <= kOrthLdsFloats) {
       const size_t lds = size_t(max_nr) * sizeof(float);
       HPX_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(psgd_orth_lds_kernel),
@@ -572,11 +588,40 @@ HPX_API int hpx_powersgd_encode2(int count, float* const* Ps, const float* const
     } else {
       HPX_LAUNCH("psgd_orth_kernel", psgd_orth_kernel, dim3(a.nseg), dim3(kOrthThreads), st, a);
     }
-    PSGD_LAUNCH_CG(psgd_mtp_kernel, cg, a.tile_start[a.nseg], st, a);
     HPX_HIP(hipGetLastError());
-    for (int k = 0; k <= a.nseg; k++) a.tile_start[k] = red_start[k];
-    HPX_LAUNCH("psgd_qreduce_kernel", psgd_qreduce_kernel, dim3(a.tile_start[a.nseg]), dim3(kThreads), st, a);
-    HPX_HIP(hipGetLastError());
+  }
+  // step 2: Q = M^T P, sixteen columns per pass over M
+  for (int c0 = 0; c0 < max_rank; c0 += kPassCols) {
+    int i = 0;
+    int64_t poff = 0;
+    while (i < count) {
+      a.nseg = 0;
+      a.tile_start[0] = 0;
+      int32_t red_start[kMaxSeg + 1];
+      red_start[0] = 0;
+      int cg = 1;
+      while (i < count && a.nseg < kMaxSeg) {
+        const int rb = block_cols(rs[i], c0);
+        if (rb == 0) { i++; continue; }
+        const int32_t t = cdiv(ms[i], kStrip) * cdiv(ns[i], kE2RowsPerBlock);
+        const int32_t tr = cdiv(int64_t(ms[i]) * rb, kThreads);
+        if (int64_t(a.tile_start[a.nseg]) + t > INT32_MAX || int64_t(red_start[a.nseg]) + tr > INT32_MAX) break;
+        a.seg[a.nseg] = Seg{nullptr, nullptr, nullptr, const_cast<float*>(Ms[i]), Ps[i] + c0, Qs[i] + c0, 0, ns[i], ms[i], rb,
+                            static_cast<int32_t>(poff), rs[i], 0};
+        poff += (int64_t(cdiv(ns[i], kE2RowsPerBlock)) * ms[i] * rb + 3) / 4;
+        if ((rb + 3) / 4 > cg) cg = (rb + 3) / 4;
+        a.tile_start[a.nseg + 1] = a.tile_start[a.nseg] + t;
+        red_start[a.nseg + 1] = red_start[a.nseg] + tr;
+        a.nseg++;
+        i++;
+      }
+      if (a.nseg == 0) continue;
+      PSGD_LAUNCH_CG(psgd_mtp_kernel, cg, a.tile_start[a.nseg], st, a);
+      HPX_HIP(hipGetLastError());
+      for (int k = 0; k <= a.nseg; k++) a.tile_start[k] = red_start[k];
+      HPX_LAUNCH("psgd_qreduce_kernel", psgd_qreduce_kernel, dim3(a.tile_start[a.nseg]), dim3(kThreads), st, a);
+      HPX_HIP(hipGetLastError());
+    }
   }
   return HPX_OK;
 }
@@ -588,8 +633,8 @@ HPX_API int hpx_powersgd_decode(int count, const float* const* Ps, const float* 
   HPX_ARG(count >= 0, "hpx_powersgd_decode: negative count");
   if (count == 0) return HPX_OK;
   HPX_ARG(Ps && Qs && Ms && residuals && grads && numels && ns && ms && rs, "hpx_powersgd_decode: null argument array");
-  int cg = 1;
-  int rc = check_dims("hpx_powersgd_decode", Batch{count, ns, ms, rs}, &cg);
+  int max_rank = 1;
+  int rc = check_dims("hpx_powersgd_decode", Batch{count, ns, ms, rs}, &max_rank);
   if (rc != HPX_OK) return rc;
   for (int i = 0; i < count; i++) {
     HPX_ARG(Ps[i] && Qs[i] && Ms[i] && residuals[i] && grads[i], "hpx_powersgd_decode: matrix %d has a null pointer", i);
@@ -599,23 +644,31 @@ HPX_API int hpx_powersgd_decode(int count, const float* const* Ps, const float* 
   hipStream_t st = static_cast<hipStream_t>(stream);
   Args a;
   a.partials = nullptr;
-  int i = 0;
-  while (i < count) {
-    a.nseg = 0;
-    a.tile_start[0] = 0;
-    while (i < count && a.nseg < kMaxSeg) {
-      const int32_t t = cdiv(ms[i], kStrip) * cdiv(ns[i], kDecRowsPerBlock);
-      if (int64_t(a.tile_start[a.nseg]) + t > INT32_MAX) break;
-      a.seg[a.nseg] = Seg{grads[i], residuals[i], Qs[i], Ms[i], const_cast<float*>(Ps[i]), nullptr, numels[i], ns[i], ms[i],
-                          rs[i], 0};
-      a.tile_start[a.nseg + 1] = a.tile_start[a.nseg] + t;
-      a.nseg++;
-      i++;
+  for (int c0 = 0; c0 < max_rank; c0 += kPassCols) {
+    int i = 0;
+    while (i < count) {
+      a.nseg = 0;
+      a.tile_start[0] = 0;
+      int cg = 1;
+      while (i < count && a.nseg < kMaxSeg) {
+        const int rb = block_cols(rs[i], c0);
+        if (rb == 0) { i++; continue; }
+        const int32_t t = cdiv(ms[i], kStrip) * cdiv(ns[i], kDecRowsPerBlock);
+        if (int64_t(a.tile_start[a.nseg]) + t > INT32_MAX) break;
+        const int32_t mode = (c0 ? kOntoM : 0) | (c0 + kPassCols < rs[i] ? kKeepGrad : 0);
+        a.seg[a.nseg] = Seg{grads[i], residuals[i], Qs[i] + c0, Ms[i], const_cast<float*>(Ps[i]) + c0, nullptr, numels[i], ns[i],
+                            ms[i], rb, 0, rs[i], mode};
+        if ((rb + 3) / 4 > cg) cg = (rb + 3) / 4;
+        a.tile_start[a.nseg + 1] = a.tile_start[a.nseg] + t;
+        a.nseg++;
+        i++;
+      }
+      if (a.nseg == 0) continue;
+      // One read and three writes per element: held to two workgroups per CU (LDS the kernel never touches,
+      // hpx_common.h), the 36 matrices of the configuration decode in 755 us instead of 792 (three per CU: 776).
+      PSGD_LAUNCH_CG_LDS(psgd_decode_kernel, cg, a.tile_start[a.nseg], hpx::kWriteStreamPadLds2, st, a);
+      HPX_HIP(hipGetLastError());
     }
-    // One read and three writes per element: held to two workgroups per CU (LDS the kernel never touches,
-    // hpx_common.h), the 36 matrices of the configuration decode in 755 us instead of 792 (three per CU: 776).
-    PSGD_LAUNCH_CG_LDS(psgd_decode_kernel, cg, a.tile_start[a.nseg], hpx::kWriteStreamPadLds2, st, a);
-    HPX_HIP(hipGetLastError());
   }
   return HPX_OK;
 }
