@@ -350,7 +350,10 @@ int hpx_ecq_decode(int count, const uint8_t* const* ins, const int32_t* in_sizes
 /* ---- PowerSGD: rank-r factorisation with error feedback ------------------- */
 /* The reference bodies operate on torch tensors (powersgd_body.h); here every
  * matrix is a row-major fp32 device array: M is n x m, Q is m x r, P is n x r,
- * grad/residual hold numel <= n*m elements (the flat prefix of M). */
+ * grad/residual hold numel <= n*m elements (the flat prefix of M).  Any rank
+ * r >= 1, as the reference (its bodies are plain mm, powersgd_body.h:28,49,69):
+ * up to 16 in one pass over the matrix, above that sixteen columns of the
+ * factors per pass. */
 
 /* Replaces hp_cuda_powersgd_encode1 (hp_cuda.cpp:85-92,
  * hp_cuda_kernel.cu:232-255; powersgd_body.h:10-31 as its comments state it):
