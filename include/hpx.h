@@ -88,6 +88,21 @@ int hpx_release_stream(hpx_stream_t stream);
  *                             launch of that kind: its head stays on chip,
  *                             the rest is read twice by the same launch;
  *                             0: such tensors take the two-launch encode
+ *   "gd_provisional_min_samples" a sparsifier call (hpx_gd_encode,
+ *                             hpx_dgc_encode) whose tensors' samples add up to
+ *                             at least this many (default 262144) starts its
+ *                             pass over the tensors from a provisional
+ *                             threshold taken from the first 16384 samples and
+ *                             finds the exact one afterwards among the samples
+ *                             the pass marked, instead of gathering the whole
+ *                             sample first; the message is the same.  Negative:
+ *                             never
+ *   "gd_provisional_margin"   how many times the expected number of entries
+ *                             the provisional threshold lets through (default
+ *                             3).  A tensor whose provisional threshold turns
+ *                             out not to lie below the exact one is encoded
+ *                             again through the gather path (hpx_gd_fallbacks
+ *                             counts them); 0 all but forces that
  *   "clock_seed"              what an encoder uses when it is called with
  *                             seeds == NULL; negative (default): the wall
  *                             clock, as the reference's bodies
@@ -295,6 +310,11 @@ int hpx_gd_encode(int count, const float* const* grads, const int32_t* Ns,
 int hpx_gd_decode(int count, const uint8_t* const* ins, const int32_t* in_sizes,
                   float* const* outs, const int32_t* out_sizes,
                   const int32_t* is_add_tos, hpx_stream_t stream);
+
+/* Diagnostic: tensors of sparsifier calls on `stream` so far whose provisional
+ * threshold was not below the exact one and that were therefore encoded through
+ * the gather path after all (see "gd_provisional_margin"). */
+int64_t hpx_gd_fallbacks(hpx_stream_t stream);
 
 /* ---- DGC without residual --------------------------------------------------
  * The reference holds this sparsifier as a body without a driver

@@ -31,6 +31,7 @@ SYMBOLS = (
     "hpx_terngrad_decode_status",
     "hpx_gd_encode",
     "hpx_gd_decode",
+    "hpx_gd_fallbacks",
     "hpx_dgc_encode",
     "hpx_dgc_decode",
     "hpx_ecq_encode",
@@ -100,6 +101,8 @@ def load():
     L.hpx_terngrad_repaired.argtypes = [p]
     L.hpx_terngrad_repaired.restype = C.c_int64
     L.hpx_terngrad_phase_stamps.argtypes = [p, i32]
+    L.hpx_gd_fallbacks.argtypes = [p]
+    L.hpx_gd_fallbacks.restype = C.c_int64
     L.hpx_release_stream.argtypes = [p]
     L.hpx_terngrad_decode.argtypes = [i32, pp, p, pp, p, p, p]
     L.hpx_terngrad_decode_status.argtypes = [p]

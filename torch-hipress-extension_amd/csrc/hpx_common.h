@@ -105,6 +105,7 @@ struct Workspace {
   CompletionLog<ResidentRec, ResidentMark> resident_log;
   uint32_t* done = nullptr;  // kBarMaxWorkgroups words, see ensure_barrier
   uint64_t repaired = 0;  // tensors encoded again after an expired barrier, ever
+  uint64_t gd_fallbacks = 0;  // sparsifier tensors whose provisional threshold was not below the exact one, ever
 };
 constexpr size_t kStateWords = 4096;       // 16 KiB
 constexpr size_t kStatusWord = kStateWords - 16;  // sticky flags live here
@@ -221,6 +222,12 @@ enum Option {
   kOptTerngradResidentStreamed,  // "terngrad_resident_streamed": 1 (default) = a tensor larger than the chip holds also
                                  // takes the single launch, which keeps the tensor's head on chip and streams the
                                  // rest twice; 0 = such tensors take the two-launch encode.
+  kOptGdProvisionalMinSamples,  // "gd_provisional_min_samples": a sparsifier call whose tensors' samples add up to this many
+                                // takes the path that starts its pass from a provisional threshold (hpx_gd.hip); negative:
+                                // never.  Default 262144.
+  kOptGdProvisionalMargin,      // "gd_provisional_margin": how many times the expected number of entries that threshold lets
+                                // through.  Default 3; 0 puts it at the top of its samples, which all but forces the
+                                // fall-back to the gather path (for tests of that fall-back).
   kOptClockSeed,                // "clock_seed": what an encoder called with seeds == NULL uses in place of the wall clock
                                 // (terngrad_body.h:247-251, gd_body.h:138-140); negative (default) = read the clock.
                                 // Makes the C++ drivers, which cannot pass seeds, reproducible.

@@ -51,10 +51,13 @@ constexpr int kCapLarge = 256;                   // tensors per launch table (17
 constexpr int kCapSmall = 4;                     // calls with a few tensors pass a table of a few hundred bytes
 
 struct GdState {
-  uint32_t unused0;
-  uint32_t thr_bits;  // threshold as fp32 bits
-  uint32_t pad[62];
+  uint32_t hits;      // provisional path: samples found above the provisional threshold so far
+  uint32_t thr_bits;  // threshold as fp32 bits (provisional path: the provisional one until the exact one is known)
+  uint32_t fallback;  // provisional path: 1 when the provisional threshold turned out to lie above the exact one
+  uint32_t pad[61];
 };
+constexpr uint32_t kPreSamples = 16384;  // samples the provisional threshold is taken from
+constexpr uint32_t kFallback = 0xFFFFFFFEu;  // reported in place of a count: this tensor has to take the other path
 constexpr int kScanChunk = 4096;   // per-tile counts scanned by one workgroup
 constexpr int kMaxChunks = 128;    // 2^31 elements / kTile / kScanChunk
 
@@ -125,6 +128,8 @@ template <int CAP>
 struct GdArgs {
   int32_t nseg;
   int32_t residual;             // 0: the sparsifier without residual (dgc_body.h)
+  int32_t margin;               // provisional path: how many times the expected number of entries the provisional
+                                // threshold lets through
   int32_t tile_start[CAP + 1];  // exclusive prefix of this launch's workgroups per tensor
   GdSeg seg[CAP];
   uint32_t* report;             // pinned host memory, kReportWords per tensor of this table
@@ -270,6 +275,153 @@ __global__ __launch_bounds__(kSelThreads) void gd_threshold_kernel(const GdArgs<
   find_digit<kBins2>(hist + kBins1, rank, d2, rank);
   find_digit<kBins3>(hist + kBins1 + kBins2, rank, d3, rank);
   if (threadIdx.x == 0) seg_state(sg)->thr_bits = (d1 << 21) | (d2 << 10) | d3;
+}
+
+// ---- the sampled threshold without the full gather (provisional path) -----------------------------------------
+// The reference's threshold is the thr_index-th largest of a 1 % sample drawn at random positions: gathering it
+// costs a 128-byte line of G and one of R per sample, a fifth of the traffic of the pass over the tensor itself,
+// and it has to be finished before that pass can start.  This path starts the pass from a PROVISIONAL threshold
+// instead - taken from the first kPreSamples samples only and set low enough (`margin` times the expected
+// number of entries above it) that it all but certainly lies below the exact one - so the pass marks a superset
+// of the candidates.  Every sample whose value exceeds the provisional threshold is then one whose bit the pass
+// has set, so the exact threshold (the thr_index-th largest of ALL samples) is found among the samples whose bit is
+// set: a gather over the bit mask (1 bit per element, cache-resident) and the values of the few that hit.  A last
+// small pass clears the bits of the elements that do not exceed the exact threshold; scan and expand go on as
+// ever.  Should fewer than thr_index + 1 samples exceed the provisional threshold (it was not below the exact one,
+// or they tie), the tensor is reported as kFallback and the host sends it through the gather path, on the residual
+// the pass has already updated.
+//
+// Rank `rank` (0-based from the top) of `count` keys in global memory, by one workgroup of kSelThreads lanes:
+// three histogram passes of 11 + 11 + 10 bits in LDS.  Every lane returns the key.
+__device__ __forceinline__ uint32_t select_rank(const uint32_t* __restrict__ keys, uint32_t count, uint32_t rank,
+                                                uint32_t* s_hist) {
+  uint32_t prefix = 0;
+#pragma unroll 1
+  for (int pass = 1; pass <= 3; pass++) {
+    for (int i = threadIdx.x; i < kBins1; i += kSelThreads) s_hist[i] = 0;
+    __syncthreads();
+    for (uint32_t x = threadIdx.x; x < count; x += kSelThreads) {
+      const uint32_t key = keys[x];
+      if (pass == 1) atomicAdd(&s_hist[key >> 21], 1u);
+      else if (pass == 2) { if ((key >> 21) == prefix) atomicAdd(&s_hist[(key >> 10) & 2047u], 1u); }
+      else if ((key >> 10) == prefix) atomicAdd(&s_hist[key & 1023u], 1u);
+    }
+    __syncthreads();
+    uint32_t d;
+    if (pass == 3) find_digit<kBins3>(s_hist, rank, d, rank); else find_digit<kBins1>(s_hist, rank, d, rank);
+    prefix = pass == 1 ? d : pass == 2 ? ((prefix << 11) | d) : ((prefix << 10) | d);
+  }
+  return prefix;
+}
+
+// One workgroup per tensor: the provisional threshold.
+template <int CAP>
+__global__ __launch_bounds__(kSelThreads) void gd_presample_kernel(const GdArgs<CAP> a) {
+  __shared__ uint32_t s_hist[kBins1];
+  const GdSeg& sg = a.seg[blockIdx.x];
+  const GdLayout l = gd_layout(sg.n, sg.sample_cnt);
+  uint32_t* samples = reinterpret_cast<uint32_t*>(sg.ws + l.samples);
+  const uint32_t s0 = sg.sample_cnt < kPreSamples ? sg.sample_cnt : kPreSamples;
+  for (uint32_t x = threadIdx.x; x < s0; x += kSelThreads) {
+    const uint32_t i = sample_index(sg.seed, x, sg.n);
+    samples[x] = __float_as_uint(__builtin_fabsf(a.residual ? sg.g[i] + sg.r[i] : sg.g[i]));
+  }
+  __syncthreads();
+  // rank of the provisional threshold among the s0 samples: `margin` times where the exact one is expected
+  uint64_t kp = 0;
+  if (a.margin > 0) kp = (uint64_t(a.margin) * (uint64_t(sg.thr_index) + 1) * s0 + sg.sample_cnt - 1) / sg.sample_cnt + 8;
+  if (kp > s0 - 1) kp = s0 - 1;
+  const uint32_t key = select_rank(samples, s0, uint32_t(kp), s_hist);
+  if (threadIdx.x == 0) {
+    GdState* st = seg_state(sg);
+    st->thr_bits = key;
+    st->hits = 0;
+    st->fallback = 0;
+  }
+}
+
+// All samples against the bit mask the pass left: the values of those whose bit is set are listed.
+template <int CAP>
+__global__ __launch_bounds__(kThreads) void gd_resample_kernel(const GdArgs<CAP> a) {
+  const int tile = blockIdx.x;
+  const int s = find_segment<CAP>(a.tile_start, a.nseg, tile);
+  const GdSeg& sg = a.seg[s];
+  const GdLayout l = gd_layout(sg.n, sg.sample_cnt);
+  const uint64_t* __restrict__ masks = reinterpret_cast<const uint64_t*>(sg.ws + l.masks);
+  uint32_t* hits = reinterpret_cast<uint32_t*>(sg.ws + l.samples);
+  GdState* st = seg_state(sg);
+  const uint32_t x = uint32_t(tile - a.tile_start[s]) * kThreads + threadIdx.x;
+  bool hit = false;
+  uint32_t i = 0;
+  if (x < sg.sample_cnt) {
+    i = sample_index(sg.seed, x, sg.n);
+    hit = (masks[i >> 6] >> (i & 63u)) & 1ull;
+  }
+  const uint64_t m = __ballot(hit);
+  if (m == 0) return;
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  uint32_t base = 0;
+  if (lane == uint32_t(__builtin_ctzll(m))) base = atomicAdd(&st->hits, uint32_t(__popcll(m)));
+  base = __shfl(base, __builtin_ctzll(m), kWave);
+  if (hit) hits[base + uint32_t(__popcll(m & ((1ull << lane) - 1ull)))] = __float_as_uint(__builtin_fabsf(sg.r[i]));
+}
+
+// One workgroup per tensor: the exact threshold from the listed values, or the call for the other path.
+template <int CAP>
+__global__ __launch_bounds__(kSelThreads) void gd_exact_kernel(const GdArgs<CAP> a) {
+  __shared__ uint32_t s_hist[kBins1];
+  const GdSeg& sg = a.seg[blockIdx.x];
+  const GdLayout l = gd_layout(sg.n, sg.sample_cnt);
+  GdState* st = seg_state(sg);
+  const uint32_t found = st->hits;
+  if (found <= sg.thr_index) {
+    if (threadIdx.x == 0) st->fallback = 1;
+    return;
+  }
+  const uint32_t key = select_rank(reinterpret_cast<const uint32_t*>(sg.ws + l.samples), found, sg.thr_index, s_hist);
+  if (threadIdx.x == 0) st->thr_bits = key;
+}
+
+// The bits of the elements that exceed the provisional threshold but not the exact one are cleared, the tiles'
+// counts corrected: a wave per tile, a mask word per lane, the value of a word's first set bit loaded for all
+// lanes together.
+template <int CAP>
+__global__ __launch_bounds__(kThreads) void gd_recount_kernel(const GdArgs<CAP> a) {
+  const int blk = blockIdx.x;
+  const int s = find_segment<CAP>(a.tile_start, a.nseg, blk);
+  const GdSeg& sg = a.seg[s];
+  const GdState* st = seg_state(sg);
+  if (st->fallback) return;
+  const GdLayout l = gd_layout(sg.n, sg.sample_cnt);
+  uint64_t* __restrict__ masks = reinterpret_cast<uint64_t*>(sg.ws + l.masks);
+  uint32_t* __restrict__ cnt = reinterpret_cast<uint32_t*>(sg.ws + l.cnt);
+  const float* __restrict__ r = sg.r;
+  const uint32_t ntiles = cdiv(sg.n, kTile);
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  const uint32_t tile = uint32_t(blk - a.tile_start[s]) * (kThreads / kWave) + threadIdx.x / kWave;
+  if (tile >= ntiles) return;
+  if (cnt[tile] == 0) return;  // wave-uniform
+  const float thr = __uint_as_float(st->thr_bits), nthr = -thr;
+  const uint64_t old = masks[size_t(tile) * kWave + lane];
+  const uint32_t e0 = tile * uint32_t(kTile) + lane * kWave;
+  uint64_t m = old, keep = 0;
+  const uint32_t b1 = m ? uint32_t(__builtin_ctzll(m)) : 0u;
+  const float v1 = m ? r[e0 + b1] : 0.0f;
+  if (m) {
+    if (v1 > thr || v1 < nthr) keep |= 1ull << b1;
+    m &= m - 1;
+  }
+  while (m) {
+    const uint32_t b = uint32_t(__builtin_ctzll(m));
+    m &= m - 1;
+    const float v = r[e0 + b];
+    if (v > thr || v < nthr) keep |= 1ull << b;
+  }
+  if (keep != old) masks[size_t(tile) * kWave + lane] = keep;
+  uint32_t c = uint32_t(__popcll(keep));
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) c += __shfl_xor(c, o, kWave);
+  if (lane == 0) cnt[tile] = c;
 }
 
 // The one pass over the tensors.  Lane l of wave w handles elements
@@ -459,6 +611,16 @@ __global__ __launch_bounds__(kThreads) void gd_expand_kernel(const GdArgs<CAP> a
   }
   const uint32_t total = __builtin_amdgcn_readlane(inc2, kWave - 1);
   const uint32_t ex0 = inc2 - a0 - a1, ex1 = ex0 + a0;  // exclusive prefixes of chunks 2 * lane and 2 * lane + 1
+  if (a.margin >= 0 && st->fallback) {
+    // the provisional threshold was not below the exact one: nothing of what the masks hold may be used
+    if (tile0 == 0 && a.report != nullptr && lane == 0) {
+      uint32_t* rep = a.report + size_t(s) * kReportWords;
+      __hip_atomic_store(rep + 0, kFallback, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      __hip_atomic_store(rep + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      __hip_atomic_store(rep + 2, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+    return;
+  }
   if (tile0 == 0 && a.report != nullptr) {
     // Pinned host words the host polls (no copy command, no wait for the stream).  The host waits for each
     // of the three words to change, so plain system-scope stores do (a release would write the whole L2 back).
@@ -900,12 +1062,15 @@ struct Plan {
   int index;  // position in the call
 };
 
-// The six phases for up to CAP tensors: six launch sequences, no host wait.
+// The phases for up to CAP tensors, no host wait.  margin < 0: the threshold from the full gathered sample
+// (sample, three histogram passes, rank search), then the pass, scan and expand.  margin >= 0: the provisional
+// path (above): provisional threshold, the pass, the samples against the mask, exact threshold, recount, scan, expand.
 template <int CAP>
-int launch_phases(const Plan* plans, int count, bool residual, uint32_t* report, hipStream_t st) {
+int launch_phases(const Plan* plans, int count, bool residual, int margin, uint32_t* report, hipStream_t st) {
   GdArgs<CAP> a;
   a.nseg = count;
   a.residual = residual ? 1 : 0;
+  a.margin = margin;
   a.report = report;
   for (int i = 0; i < count; i++) a.seg[i] = plans[i].seg;
   auto tiles = [&](auto per_tensor) {
@@ -917,18 +1082,32 @@ int launch_phases(const Plan* plans, int count, bool residual, uint32_t* report,
     const uint32_t b = cdiv(sg.sample_cnt, kSelThreads * 8);
     return b > uint32_t(kSelBlocksMax) ? uint32_t(kSelBlocksMax) : b;
   };
-  dim3 grid = tiles([](const GdSeg& sg) { return cdiv(sg.sample_cnt > uint32_t(kHistWords) ? sg.sample_cnt : uint32_t(kHistWords), kThreads); });
-  HPX_LAUNCH("gd_sample_kernel", gd_sample_kernel<CAP>, grid, dim3(kThreads), st, a);
-  grid = tiles(sel_blocks);
-  HPX_LAUNCH("gd_select_kernel", (gd_select_kernel<1, CAP>), grid, dim3(kSelThreads), st, a);
-  HPX_LAUNCH("gd_select_kernel", (gd_select_kernel<2, CAP>), grid, dim3(kSelThreads), st, a);
-  HPX_LAUNCH("gd_select_kernel", (gd_select_kernel<3, CAP>), grid, dim3(kSelThreads), st, a);
-  HPX_LAUNCH("gd_threshold_kernel", gd_threshold_kernel<CAP>, dim3(uint32_t(count)), dim3(kSelThreads), st, a);
-  grid = tiles([](const GdSeg& sg) { return cdiv(sg.n, kTile); });
-  if (residual)
-    HPX_LAUNCH("gd_stream_kernel", (gd_stream_kernel<true, CAP>), grid, dim3(kThreads), st, a);
-  else
-    HPX_LAUNCH("gd_stream_kernel", (gd_stream_kernel<false, CAP>), grid, dim3(kThreads), st, a);
+  auto stream_pass = [&]() {
+    const dim3 g = tiles([](const GdSeg& sg) { return cdiv(sg.n, kTile); });
+    if (residual)
+      HPX_LAUNCH("gd_stream_kernel", (gd_stream_kernel<true, CAP>), g, dim3(kThreads), st, a);
+    else
+      HPX_LAUNCH("gd_stream_kernel", (gd_stream_kernel<false, CAP>), g, dim3(kThreads), st, a);
+  };
+  dim3 grid;
+  if (margin < 0) {
+    grid = tiles([](const GdSeg& sg) { return cdiv(sg.sample_cnt > uint32_t(kHistWords) ? sg.sample_cnt : uint32_t(kHistWords), kThreads); });
+    HPX_LAUNCH("gd_sample_kernel", gd_sample_kernel<CAP>, grid, dim3(kThreads), st, a);
+    grid = tiles(sel_blocks);
+    HPX_LAUNCH("gd_select_kernel", (gd_select_kernel<1, CAP>), grid, dim3(kSelThreads), st, a);
+    HPX_LAUNCH("gd_select_kernel", (gd_select_kernel<2, CAP>), grid, dim3(kSelThreads), st, a);
+    HPX_LAUNCH("gd_select_kernel", (gd_select_kernel<3, CAP>), grid, dim3(kSelThreads), st, a);
+    HPX_LAUNCH("gd_threshold_kernel", gd_threshold_kernel<CAP>, dim3(uint32_t(count)), dim3(kSelThreads), st, a);
+    stream_pass();
+  } else {
+    HPX_LAUNCH("gd_presample_kernel", gd_presample_kernel<CAP>, dim3(uint32_t(count)), dim3(kSelThreads), st, a);
+    stream_pass();
+    grid = tiles([](const GdSeg& sg) { return cdiv(sg.sample_cnt, kThreads); });
+    HPX_LAUNCH("gd_resample_kernel", gd_resample_kernel<CAP>, grid, dim3(kThreads), st, a);
+    HPX_LAUNCH("gd_exact_kernel", gd_exact_kernel<CAP>, dim3(uint32_t(count)), dim3(kSelThreads), st, a);
+    grid = tiles([](const GdSeg& sg) { return cdiv(cdiv(sg.n, kTile), kThreads / kWave); });
+    HPX_LAUNCH("gd_recount_kernel", gd_recount_kernel<CAP>, grid, dim3(kThreads), st, a);
+  }
   grid = tiles([](const GdSeg& sg) { return cdiv(cdiv(sg.n, kTile), kScanChunk); });
   HPX_LAUNCH("gd_scan_kernel", gd_scan_kernel<CAP>, grid, dim3(kSelThreads), st, a);
   HPX_HIP(hipGetLastError());
@@ -1029,20 +1208,60 @@ int gd_encode_batch(int count, float* const* grads, const int32_t* Ns, float* co
   }
   volatile uint32_t* report = reinterpret_cast<volatile uint32_t*>(ws->pinned);
   const int total = int(plans.size());
-  for (int first = 0; first < total; first += kMaxPerWait) {
-    const int batch = total - first < kMaxPerWait ? total - first : kMaxPerWait;
-    for (int t = 0; t < batch; t++)
+  // The provisional path pays where the gather of the full sample is long: from a few hundred thousand samples on.
+  uint64_t all_samples = 0;
+  for (const Plan& p : plans) all_samples += p.seg.sample_cnt;
+  const int64_t prov_min = hpx::option(hpx::kOptGdProvisionalMinSamples);
+  const int64_t prov_margin = hpx::option(hpx::kOptGdProvisionalMargin);
+  const int margin = (prov_min >= 0 && all_samples >= uint64_t(prov_min) && prov_margin >= 0) ? int(prov_margin > 1000 ? 1000 : prov_margin) : -1;
+  auto reset_reports = [&](int n_) {
+    for (int t = 0; t < n_; t++)
       for (int w = 0; w < 3; w++) report[size_t(t) * kReportWords + w] = kNotReported;
     __atomic_thread_fence(__ATOMIC_RELEASE);
+  };
+  for (int first = 0; first < total; first += kMaxPerWait) {
+    const int batch = total - first < kMaxPerWait ? total - first : kMaxPerWait;
+    reset_reports(batch);
     for (int k = 0; k < batch; k += kCapLarge) {
       const int m = batch - k < kCapLarge ? batch - k : kCapLarge;
       uint32_t* rep = const_cast<uint32_t*>(report) + size_t(k) * kReportWords;
-      rc = m <= kCapSmall ? launch_phases<kCapSmall>(&plans[first + k], m, residuals != nullptr, rep, st)
-                          : launch_phases<kCapLarge>(&plans[first + k], m, residuals != nullptr, rep, st);
+      rc = m <= kCapSmall ? launch_phases<kCapSmall>(&plans[first + k], m, residuals != nullptr, margin, rep, st)
+                          : launch_phases<kCapLarge>(&plans[first + k], m, residuals != nullptr, margin, rep, st);
       if (rc != HPX_OK) return rc;
     }
     rc = wait_reports(report, batch, st);
     if (rc != HPX_OK) return rc;
+    // What the tensors reported, kept on the host: the pinned words serve again below.
+    std::vector<uint32_t> rep_host(size_t(batch) * kReportWords);
+    for (size_t w = 0; w < rep_host.size(); w++) rep_host[w] = report[w];
+    if (margin >= 0) {
+      // Tensors whose provisional threshold was not below the exact one: through the gather path, on the array
+      // the pass has already updated (it holds G + R now: sampled and thresholded as it is, nothing added again).
+      std::vector<int> fb;
+      for (int t = 0; t < batch; t++)
+        if (rep_host[size_t(t) * kReportWords] == kFallback) fb.push_back(t);
+      if (!fb.empty()) {
+        std::vector<Plan> again;
+        for (int t : fb) {
+          Plan p = plans[first + t];
+          p.seg.g = p.seg.r;
+          again.push_back(p);
+        }
+        ws->gd_fallbacks += fb.size();
+        reset_reports(int(again.size()));
+        for (size_t k = 0; k < again.size(); k += kCapLarge) {
+          const int m = int(again.size() - k < size_t(kCapLarge) ? again.size() - k : size_t(kCapLarge));
+          uint32_t* rep = const_cast<uint32_t*>(report) + k * kReportWords;
+          rc = m <= kCapSmall ? launch_phases<kCapSmall>(&again[k], m, false, -1, rep, st)
+                              : launch_phases<kCapLarge>(&again[k], m, false, -1, rep, st);
+          if (rc != HPX_OK) return rc;
+        }
+        rc = wait_reports(report, int(again.size()), st);
+        if (rc != HPX_OK) return rc;
+        for (size_t j = 0; j < fb.size(); j++)
+          for (int w = 0; w < kReportWords; w++) rep_host[size_t(fb[j]) * kReportWords + w] = report[j * kReportWords + w];
+      }
+    }
     // More candidates than `expected`: order them by |r| descending and keep the first `expected`
     // (gd_body.h:176-187), all such tensors of the batch together.
     std::vector<CutJob> jobs;
@@ -1050,9 +1269,9 @@ int gd_encode_batch(int count, float* const* grads, const int32_t* Ns, float* co
     size_t aux_need = 0;
     for (int t = 0; t < batch; t++) {
       const GdSeg& sg = plans[first + t].seg;
-      const uint32_t found = report[size_t(t) * kReportWords];
+      const uint32_t found = rep_host[size_t(t) * kReportWords];
       if (found <= sg.limit) continue;
-      const uint32_t thr_bits = report[size_t(t) * kReportWords + 1], max_bits = report[size_t(t) * kReportWords + 2];
+      const uint32_t thr_bits = rep_host[size_t(t) * kReportWords + 1], max_bits = rep_host[size_t(t) * kReportWords + 2];
       // keys are |r| bits minus threshold bits: the largest tells how many byte digits are in use
       const uint32_t max_key = max_bits > thr_bits ? max_bits - thr_bits : 0u;
       CutJob job;
@@ -1095,6 +1314,7 @@ int gd_encode_batch(int count, float* const* grads, const int32_t* Ns, float* co
         GdArgs<kCapSmall> a;
         a.nseg = 1;
         a.residual = residuals != nullptr;
+        a.margin = -1;
         a.report = nullptr;  // the host has its report
         a.seg[0] = plan.seg;
         a.seg[0].cut = cut;
@@ -1137,6 +1357,14 @@ HPX_API int hpx_gd_encode(int count, const float* const* grads, const int32_t* N
   std::vector<double> kept(count);
   for (int i = 0; i < count; i++) kept[i] = 1 - drop_ratios[i];  // s_percent, gd_body.h:112
   return gd_encode_batch(count, const_cast<float* const*>(grads), Ns, residuals, outs, sample_rates, kept.data(), seeds, ws, st);
+}
+
+HPX_API int64_t hpx_gd_fallbacks(hpx_stream_t stream) {
+  hpx::clear_error();
+  hpx::Workspace* ws = hpx::workspace_record(static_cast<hipStream_t>(stream));
+  if (!ws) return -1;
+  std::lock_guard<std::mutex> lock(ws->mu);
+  return int64_t(ws->gd_fallbacks);
 }
 
 namespace {
