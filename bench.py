@@ -598,7 +598,8 @@ def x_terngrad_sizes(torch, np, capi, L, stream, gen, res):
     res["terngrad_102M"] = dict(big, algorithmic_bytes=8.5 * 102_760_448, workload="VGG-16 fc6, 2-bit, stochastic rounding, encode + decode(write)")
 
 
-GD_KERNELS = ["gd_sample_kernel", "gd_select_kernel", "gd_threshold_kernel", "gd_stream_kernel", "gd_scan_kernel",
+GD_KERNELS = ["gd_sample_kernel", "gd_select_kernel", "gd_threshold_kernel", "gd_presample_kernel", "gd_provisional_kernel", "gd_stream_kernel",
+              "gd_resample_kernel", "gd_exact_kernel", "gd_recount_kernel", "gd_scan_kernel",
               "gd_expand_kernel", "gd_sort_count_kernel", "gd_sort_pass_kernel", "gd_gather_kernel"]
 
 

@@ -90,13 +90,14 @@ int hpx_release_stream(hpx_stream_t stream);
  *                             0: such tensors take the two-launch encode
  *   "gd_provisional_min_samples" a sparsifier call (hpx_gd_encode,
  *                             hpx_dgc_encode) whose tensors' samples add up to
- *                             at least this many (default 262144) starts its
+ *                             at least this many (default -1: none) starts its
  *                             pass over the tensors from a provisional
  *                             threshold taken from the first 16384 samples and
  *                             finds the exact one afterwards among the samples
  *                             the pass marked, instead of gathering the whole
  *                             sample first; the message is the same.  Negative:
- *                             never
+ *                             never.  Off by default: measured on a 138 M
+ *                             element tensor it is 3 % slower than the gather
  *   "gd_provisional_margin"   how many times the expected number of entries
  *                             the provisional threshold lets through (default
  *                             3).  A tensor whose provisional threshold turns

@@ -44,8 +44,8 @@ def gd(capi):
 @pytest.fixture(autouse=True, scope="module", params=["gather", "provisional", "provisional_fall_back"])
 def threshold_path(request, capi):
     """Every test of this module runs three times: with the threshold taken from the gathered sample before the
-    pass; with the pass started from a provisional threshold and the exact one found afterwards (by default only
-    calls with 262144 samples and more take that path); and with the provisional threshold put at the top of its
+    pass; with the pass started from a provisional threshold and the exact one found afterwards (an option, off by
+    default); and with the provisional threshold put at the top of its
     samples, so that it lies above the exact one and every tensor falls back to the gather path after the pass has
     updated the residual.  The messages are the same bit for bit."""
     mode = request.param

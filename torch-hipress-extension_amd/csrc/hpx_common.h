@@ -223,8 +223,11 @@ enum Option {
                                  // takes the single launch, which keeps the tensor's head on chip and streams the
                                  // rest twice; 0 = such tensors take the two-launch encode.
   kOptGdProvisionalMinSamples,  // "gd_provisional_min_samples": a sparsifier call whose tensors' samples add up to this many
-                                // takes the path that starts its pass from a provisional threshold (hpx_gd.hip); negative:
-                                // never.  Default 262144.
+                                // takes the path that starts its pass from a provisional threshold (hpx_gd.hip); negative
+                                // (the default): never.  Measured on the 138 M-element configuration it does not pay:
+                                // 355-363 us against 346 for the gather path (the gather's lines warm the cache for the
+                                // pass, which runs 25 us longer without them, and the single-workgroup selections and the
+                                // recount cost what the gather saved).
   kOptGdProvisionalMargin,      // "gd_provisional_margin": how many times the expected number of entries that threshold lets
                                 // through.  Default 3; 0 puts it at the top of its samples, which all but forces the
                                 // fall-back to the gather path (for tests of that fall-back).

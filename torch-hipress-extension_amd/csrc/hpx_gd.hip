@@ -56,6 +56,7 @@ struct GdState {
   uint32_t fallback;  // provisional path: 1 when the provisional threshold turned out to lie above the exact one
   uint32_t pad[61];
 };
+constexpr int kHitWays = 128;             // parts of the list of samples above the provisional threshold
 constexpr uint32_t kPreSamples = 16384;  // samples the provisional threshold is taken from
 constexpr uint32_t kFallback = 0xFFFFFFFEu;  // reported in place of a count: this tensor has to take the other path
 constexpr int kScanChunk = 4096;   // per-tile counts scanned by one workgroup
@@ -66,7 +67,7 @@ __host__ __device__ constexpr uint32_t cdiv(uint64_t a, uint64_t b) { return sta
 
 // Where the pieces of one tensor's workspace block lie (the same arithmetic on the host and in the kernels).
 struct GdLayout {
-  size_t state, hist, samples, masks, cnt, mx, off, ctot, cmax, coff, end;
+  size_t state, hist, samples, hitlist, masks, coarse, cnt, mx, off, ctot, cmax, coff, end;
 };
 __host__ __device__ inline GdLayout gd_layout(uint32_t n, uint32_t sample_cnt) {
   const size_t ntiles = cdiv(n, kTile);
@@ -75,7 +76,9 @@ __host__ __device__ inline GdLayout gd_layout(uint32_t n, uint32_t sample_cnt) {
   l.state = at;   at += align256(sizeof(GdState));
   l.hist = at;    at += align256(sizeof(uint32_t) * kHistWords);
   l.samples = at; at += align256(sizeof(uint32_t) * size_t(sample_cnt));
+  l.hitlist = at; at += align256(sizeof(uint32_t) * (size_t(sample_cnt) + size_t(256) * 128));  // provisional path, see gd_resample_kernel
   l.masks = at;   at += align256(sizeof(uint64_t) * ntiles * kWave);      // one bit per element
+  l.coarse = at;  at += align256(sizeof(uint64_t) * ntiles);              // one bit per mask word: whether it has a bit set
   l.cnt = at;     at += align256(sizeof(uint32_t) * ntiles);              // candidates per tile
   l.mx = at;      at += align256(sizeof(uint32_t) * ntiles);              // largest |r| per tile, as bits
   l.off = at;     at += align256(sizeof(uint32_t) * ntiles);              // exclusive prefix within the chunk
@@ -314,24 +317,38 @@ __device__ __forceinline__ uint32_t select_rank(const uint32_t* __restrict__ key
   return prefix;
 }
 
-// One workgroup per tensor: the provisional threshold.
+// The first kPreSamples samples, one per lane over many workgroups (one workgroup's gathers into arrays of
+// hundreds of megabytes are bound by its CU's address translation: 16384 of them took it 90 us).
 template <int CAP>
-__global__ __launch_bounds__(kSelThreads) void gd_presample_kernel(const GdArgs<CAP> a) {
-  __shared__ uint32_t s_hist[kBins1];
-  const GdSeg& sg = a.seg[blockIdx.x];
+__global__ __launch_bounds__(kThreads) void gd_presample_kernel(const GdArgs<CAP> a) {
+  const int tile = blockIdx.x;
+  const int s = find_segment<CAP>(a.tile_start, a.nseg, tile);
+  const GdSeg& sg = a.seg[s];
   const GdLayout l = gd_layout(sg.n, sg.sample_cnt);
   uint32_t* samples = reinterpret_cast<uint32_t*>(sg.ws + l.samples);
   const uint32_t s0 = sg.sample_cnt < kPreSamples ? sg.sample_cnt : kPreSamples;
-  for (uint32_t x = threadIdx.x; x < s0; x += kSelThreads) {
+  const uint32_t x = uint32_t(tile - a.tile_start[s]) * kThreads + threadIdx.x;
+  if (x < s0) {
     const uint32_t i = sample_index(sg.seed, x, sg.n);
     samples[x] = __float_as_uint(__builtin_fabsf(a.residual ? sg.g[i] + sg.r[i] : sg.g[i]));
   }
-  __syncthreads();
+}
+
+// One workgroup per tensor: the provisional threshold from those samples; clears what the later phases count in.
+template <int CAP>
+__global__ __launch_bounds__(kSelThreads) void gd_provisional_kernel(const GdArgs<CAP> a) {
+  __shared__ uint32_t s_hist[kBins1];
+  const GdSeg& sg = a.seg[blockIdx.x];
+  const GdLayout l = gd_layout(sg.n, sg.sample_cnt);
+  const uint32_t* samples = reinterpret_cast<const uint32_t*>(sg.ws + l.samples);
+  const uint32_t s0 = sg.sample_cnt < kPreSamples ? sg.sample_cnt : kPreSamples;
   // rank of the provisional threshold among the s0 samples: `margin` times where the exact one is expected
   uint64_t kp = 0;
   if (a.margin > 0) kp = (uint64_t(a.margin) * (uint64_t(sg.thr_index) + 1) * s0 + sg.sample_cnt - 1) / sg.sample_cnt + 8;
   if (kp > s0 - 1) kp = s0 - 1;
   const uint32_t key = select_rank(samples, s0, uint32_t(kp), s_hist);
+  uint32_t* ways = reinterpret_cast<uint32_t*>(sg.ws + l.hist);
+  if (threadIdx.x < uint32_t(kHitWays)) ways[threadIdx.x] = 0;
   if (threadIdx.x == 0) {
     GdState* st = seg_state(sg);
     st->thr_bits = key;
@@ -340,7 +357,13 @@ __global__ __launch_bounds__(kSelThreads) void gd_presample_kernel(const GdArgs<
   }
 }
 
-// All samples against the bit mask the pass left: the values of those whose bit is set are listed.
+// All samples against the bit mask the pass left: the values of those whose bit is set are listed.  The list is
+// kept in kHitWays parts, workgroup b appending to part b % kHitWays (one counter for all would take the few
+// thousand appends one after the other, 37 ns each); a part has room for every sample its workgroups look at.
+__host__ __device__ inline uint32_t hit_way_room(uint32_t sample_cnt) {
+  const uint32_t blocks = cdiv(sample_cnt, kThreads);
+  return cdiv(blocks, kHitWays) * uint32_t(kThreads);
+}
 template <int CAP>
 __global__ __launch_bounds__(kThreads) void gd_resample_kernel(const GdArgs<CAP> a) {
   const int tile = blockIdx.x;
@@ -348,37 +371,59 @@ __global__ __launch_bounds__(kThreads) void gd_resample_kernel(const GdArgs<CAP>
   const GdSeg& sg = a.seg[s];
   const GdLayout l = gd_layout(sg.n, sg.sample_cnt);
   const uint64_t* __restrict__ masks = reinterpret_cast<const uint64_t*>(sg.ws + l.masks);
-  uint32_t* hits = reinterpret_cast<uint32_t*>(sg.ws + l.samples);
-  GdState* st = seg_state(sg);
-  const uint32_t x = uint32_t(tile - a.tile_start[s]) * kThreads + threadIdx.x;
+  const uint32_t blk = uint32_t(tile - a.tile_start[s]);
+  const uint32_t way = blk % uint32_t(kHitWays);
+  uint32_t* hits = reinterpret_cast<uint32_t*>(sg.ws + l.hitlist) + size_t(way) * hit_way_room(sg.sample_cnt);
+  uint32_t* counter = reinterpret_cast<uint32_t*>(sg.ws + l.hist) + way;
+  const uint32_t x = blk * kThreads + threadIdx.x;
   bool hit = false;
   uint32_t i = 0;
   if (x < sg.sample_cnt) {
     i = sample_index(sg.seed, x, sg.n);
-    hit = (masks[i >> 6] >> (i & 63u)) & 1ull;
+    // first whether the element's mask word has any bit at all (one bit per word: the whole map stays in cache),
+    // and only then the word itself
+    const uint64_t* __restrict__ coarse = reinterpret_cast<const uint64_t*>(sg.ws + l.coarse);
+    if ((coarse[i >> 12] >> ((i >> 6) & 63u)) & 1ull) hit = (masks[i >> 6] >> (i & 63u)) & 1ull;
   }
   const uint64_t m = __ballot(hit);
   if (m == 0) return;
   const uint32_t lane = threadIdx.x & (kWave - 1);
   uint32_t base = 0;
-  if (lane == uint32_t(__builtin_ctzll(m))) base = atomicAdd(&st->hits, uint32_t(__popcll(m)));
+  if (lane == uint32_t(__builtin_ctzll(m))) base = atomicAdd(counter, uint32_t(__popcll(m)));
   base = __shfl(base, __builtin_ctzll(m), kWave);
   if (hit) hits[base + uint32_t(__popcll(m & ((1ull << lane) - 1ull)))] = __float_as_uint(__builtin_fabsf(sg.r[i]));
 }
 
-// One workgroup per tensor: the exact threshold from the listed values, or the call for the other path.
+// One workgroup per tensor: the parts of the list are drawn together (into the samples' block, free by now), then
+// the exact threshold is taken from them, or the other path called for.
 template <int CAP>
 __global__ __launch_bounds__(kSelThreads) void gd_exact_kernel(const GdArgs<CAP> a) {
   __shared__ uint32_t s_hist[kBins1];
+  __shared__ uint32_t s_off[kHitWays + 1];
   const GdSeg& sg = a.seg[blockIdx.x];
   const GdLayout l = gd_layout(sg.n, sg.sample_cnt);
   GdState* st = seg_state(sg);
-  const uint32_t found = st->hits;
+  const uint32_t* ways = reinterpret_cast<const uint32_t*>(sg.ws + l.hist);
+  if (threadIdx.x == 0) {
+    uint32_t run = 0;
+    for (int w = 0; w < kHitWays; w++) { s_off[w] = run; run += ways[w]; }
+    s_off[kHitWays] = run;
+  }
+  __syncthreads();
+  const uint32_t found = s_off[kHitWays];
   if (found <= sg.thr_index) {
     if (threadIdx.x == 0) st->fallback = 1;
     return;
   }
-  const uint32_t key = select_rank(reinterpret_cast<const uint32_t*>(sg.ws + l.samples), found, sg.thr_index, s_hist);
+  const uint32_t* parts = reinterpret_cast<const uint32_t*>(sg.ws + l.hitlist);
+  uint32_t* keys = reinterpret_cast<uint32_t*>(sg.ws + l.samples);
+  const uint32_t room = hit_way_room(sg.sample_cnt);
+  for (int w = threadIdx.x / kWave; w < kHitWays; w += kSelThreads / kWave) {
+    const uint32_t c = s_off[w + 1] - s_off[w];
+    for (uint32_t k = threadIdx.x & (kWave - 1); k < c; k += kWave) keys[s_off[w] + k] = parts[size_t(w) * room + k];
+  }
+  __syncthreads();
+  const uint32_t key = select_rank(keys, found, sg.thr_index, s_hist);
   if (threadIdx.x == 0) st->thr_bits = key;
 }
 
@@ -491,14 +536,18 @@ __global__ __launch_bounds__(kThreads) void gd_stream_kernel(const GdArgs<CAP> a
     }
   }
   if (lane < kPerLane) masks[(size_t(wbase) >> 6) + lane] = (uint64_t(hi) << 32) | lo;
+  // which of the wave's sixteen mask words have a bit set (lanes beyond the sixteenth hold zeros)
+  const uint32_t any16 = uint32_t(__ballot((lo | hi) != 0u));
   uint32_t bigb = __float_as_uint(big);  // non-negative floats order like their bit patterns; a NaN is not an input
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) { const uint32_t v = __shfl_xor(bigb, o, kWave); bigb = v > bigb ? v : bigb; }
-  __shared__ uint32_t s_cnt[kThreads / kWave], s_big[kThreads / kWave];
-  if (lane == 0) { s_cnt[wave] = cnt; s_big[wave] = bigb; }
+  __shared__ uint32_t s_cnt[kThreads / kWave], s_big[kThreads / kWave], s_any[kThreads / kWave];
+  if (lane == 0) { s_cnt[wave] = cnt; s_big[wave] = bigb; s_any[wave] = any16; }
   __syncthreads();
   if (threadIdx.x == 0) {
     reinterpret_cast<uint32_t*>(sg.ws + l.cnt)[t] = s_cnt[0] + s_cnt[1] + s_cnt[2] + s_cnt[3];
+    reinterpret_cast<uint64_t*>(sg.ws + l.coarse)[t] =
+        uint64_t(s_any[0]) | (uint64_t(s_any[1]) << 16) | (uint64_t(s_any[2]) << 32) | (uint64_t(s_any[3]) << 48);
     const uint32_t m01 = s_big[0] > s_big[1] ? s_big[0] : s_big[1], m23 = s_big[2] > s_big[3] ? s_big[2] : s_big[3];
     reinterpret_cast<uint32_t*>(sg.ws + l.mx)[t] = m01 > m23 ? m01 : m23;
   }
@@ -1100,7 +1149,9 @@ int launch_phases(const Plan* plans, int count, bool residual, int margin, uint3
     HPX_LAUNCH("gd_threshold_kernel", gd_threshold_kernel<CAP>, dim3(uint32_t(count)), dim3(kSelThreads), st, a);
     stream_pass();
   } else {
-    HPX_LAUNCH("gd_presample_kernel", gd_presample_kernel<CAP>, dim3(uint32_t(count)), dim3(kSelThreads), st, a);
+    grid = tiles([](const GdSeg& sg) { return cdiv(sg.sample_cnt < kPreSamples ? sg.sample_cnt : kPreSamples, kThreads); });
+    HPX_LAUNCH("gd_presample_kernel", gd_presample_kernel<CAP>, grid, dim3(kThreads), st, a);
+    HPX_LAUNCH("gd_provisional_kernel", gd_provisional_kernel<CAP>, dim3(uint32_t(count)), dim3(kSelThreads), st, a);
     stream_pass();
     grid = tiles([](const GdSeg& sg) { return cdiv(sg.sample_cnt, kThreads); });
     HPX_LAUNCH("gd_resample_kernel", gd_resample_kernel<CAP>, grid, dim3(kThreads), st, a);

@@ -197,7 +197,7 @@ const OptionDef kOptions[kOptCount] = {
     {"terngrad_resident_bucket", "HPX_TERNGRAD_RESIDENT_BUCKET", 1},
     {"terngrad_resident_workgroups", "HPX_TERNGRAD_RESIDENT_WORKGROUPS", 0},
     {"terngrad_resident_streamed", "HPX_TERNGRAD_RESIDENT_STREAMED", 1},
-    {"gd_provisional_min_samples", "HPX_GD_PROVISIONAL_MIN_SAMPLES", 262144},
+    {"gd_provisional_min_samples", "HPX_GD_PROVISIONAL_MIN_SAMPLES", -1},
     {"gd_provisional_margin", "HPX_GD_PROVISIONAL_MARGIN", 3},
     {"clock_seed", "HPX_CLOCK_SEED", -1},
 };
