@@ -36,11 +36,11 @@ N_DGC = 138_357_544
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, each scaled by what the same
 # counter reads for a plain copy of known size.
-MEASURED_TRAFFIC_BYTES = {  # profiles/terngrad_25M_pmc_fetch_write.txt (FETCH x1.99942 + WRITE x1.0, KiB -> bytes)
-    "terngrad_resident_kernel": int((52081.1 * 1.99942 + 8295.5) * 1024),  # includes the grid-wide exchange's polls and records
-    "terngrad_minmax_kernel": int((49939.7 * 1.99942 + 390.2) * 1024),
-    "terngrad_quant_kernel": int((49990.4 * 1.99942 + 6434.5) * 1024),
-    "terngrad_decode_kernel": int((3574.9 * 1.99942 + 99906.6) * 1024),
+MEASURED_TRAFFIC_BYTES = {  # profiles/terngrad_pmc_fetch_write.txt (FETCH x1.99992 + WRITE x1.0, KiB -> bytes)
+    "terngrad_resident_kernel": int((52046.1 * 1.99992 + 8303.5) * 1024),  # includes the grid-wide exchange's polls and records
+    "terngrad_minmax_kernel": int((49939.1 * 1.99992 + 390.1) * 1024),
+    "terngrad_quant_kernel": int((49993.9 * 1.99992 + 6434.5) * 1024),
+    "terngrad_decode_kernel": int((3563.9 * 1.99992 + 99879.2) * 1024),
 }
 
 
@@ -257,7 +257,7 @@ def main():
     roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(dom),
                 "traffic_is": "not read in this run: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, scaled by a plain "
-                              "copy's readings, from profiles/terngrad_25M_pmc_fetch_write.txt",
+                              "copy's readings, from profiles/terngrad_pmc_fetch_write.txt",
                 "algorithmic_bytes_per_launch": alg_bytes[dom], "avg_launch_us": round(kt[dom] * 1e6, 2),
                 "kernel_us": {k: (round(v * 1e6, 2) if v else None) for k, v in kt.items()}}
     path_alg = 8.5 * n  # x once in, codes out; codes in, fp32 out
