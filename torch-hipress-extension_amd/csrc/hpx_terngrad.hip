@@ -772,6 +772,21 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
       draw[q] = lcg_mul(j + 2) * (x0 + jb) + lcg_add(j + 2);
     }
   }
+  // STREAMED: the first two rounds of the streamed part are requested as soon as the register rows are done and
+  // their registers free, so that memory works while the LDS rows of the share are quantised.  (Requesting them
+  // earlier, between the register rows, made the compiler spill.)
+  constexpr int SW = STREAMED ? kResStreamIters / H : 1;  // float4 per lane and round: the same at every width
+  constexpr uint32_t kRound = uint32_t(SW) * kResThreads;
+  float4 w0[SW][H], w1[SW][H];
+  auto fetch = [&](float4 (&w)[SW][H], uint32_t t0) {
+#pragma unroll
+    for (int k = 0; k < SW; k++) {
+      const uint32_t u = t0 + k * kResThreads + threadIdx.x;
+#pragma unroll
+      for (int h = 0; h < H; h++)
+        w[k][h] = (STREAMED && u < st_end) ? ld4_stream(xp + size_t(u) * UNIT + h * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+  };
   // A workgroup whose register rows are all whole (every one but the last with a share) stores
   // without a bounds check per row: the checks cost a branch each.
   auto register_rows = [&](auto whole) {
@@ -794,6 +809,10 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
     }
   };
   if (whole_rows) register_rows(std::true_type{}); else register_rows(std::false_type{});
+  if (STREAMED) {
+    fetch(w0, st_u0);
+    fetch(w1, st_u0 + kRound);
+  }
   if (RANDOM) {
     uint32_t x0 = a.seg.seed + l0 * BPU;
     // Keeps the compiler from preparing these draws before the register rows are
@@ -827,21 +846,11 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
       }
     }
     // Two rounds in flight: the loads of the next round are requested before this round is worked on (the waves
-    // of a workgroup leave the barrier together and would otherwise all load, then all compute).
-    constexpr uint32_t kRound = uint32_t(kResStreamIters) * kResThreads;
-    float4 w0[kResStreamIters][H], w1[kResStreamIters][H];
-    auto fetch = [&](float4 (&w)[kResStreamIters][H], uint32_t t0) {
+    // of a workgroup leave the barrier together and would otherwise all load, then all compute).  The first two
+    // rounds have been on their way since the register rows.
+    auto emit = [&](float4 (&w)[SW][H], uint32_t t0) {
 #pragma unroll
-      for (int k = 0; k < kResStreamIters; k++) {
-        const uint32_t u = t0 + k * kResThreads + threadIdx.x;
-#pragma unroll
-        for (int h = 0; h < H; h++)
-          w[k][h] = (t0 < st_end && u < st_end) ? ld4_stream(xp + size_t(u) * UNIT + h * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
-      }
-    };
-    auto emit = [&](float4 (&w)[kResStreamIters][H], uint32_t t0) {
-#pragma unroll
-      for (int k = 0; k < kResStreamIters; k++) {
+      for (int k = 0; k < SW; k++) {
         const uint32_t u = t0 + k * kResThreads + threadIdx.x;
         const uint32_t packed = quant_unit<B, RANDOM>(w[k], mn, gi, draw, uint32_t(kResThreads) * BPU);
         if (u < st_end) {
@@ -850,12 +859,11 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
         }
       }
     };
-    fetch(w0, st_u0);
     for (uint32_t t0 = st_u0; t0 < st_end; t0 += 2 * kRound) {
-      fetch(w1, t0 + kRound);
       emit(w0, t0);
       fetch(w0, t0 + 2 * kRound);
       if (t0 + kRound < st_end) emit(w1, t0 + kRound);
+      fetch(w1, t0 + 3 * kRound);
     }
   }
   // The unit that holds the end of the tensor, if the length is not a whole number of units.
