@@ -6,7 +6,7 @@ import pytest
 import torch
 
 from gpu_util import assert_bits_equal, dev, host, stream_ptr
-from test_oracle_ecq import ECQ_DECODED, ECQ_G, ECQ_H1, ECQ_MSG, _same_floats
+from test_oracle_ecq import ECQ_DECODED, ECQ_G, ECQ_H1, ECQ_LONG, ECQ_MSG, _same_floats
 
 pytestmark = pytest.mark.gpu
 
@@ -46,6 +46,16 @@ def test_hand_derived_message(ecq):
     assert host(out).tobytes() == ECQ_MSG, host(out).tobytes().hex()
     assert_bits_equal(host(dh), ECQ_H1, "history")
     assert_bits_equal(host(dec), ECQ_DECODED, "decoded")
+
+
+@pytest.mark.parametrize("bitwidth,G,want,h_want", ECQ_LONG, ids=["8bit", "4bit"])
+def test_hand_derived_messages_that_reread_the_scratch(ecq, bitwidth, G, want, h_want):
+    dg, dh = dev(G), torch.zeros(G.size, device="cuda")
+    out = torch.full((len(want),), 0xEE, dtype=torch.uint8, device="cuda")
+    ecq.encode([dg], [dh], [out], [1.0], [0.5], [bitwidth], [0])
+    torch.cuda.synchronize()
+    assert host(out).tobytes() == want, host(out).tobytes().hex()
+    assert_bits_equal(host(dh), h_want, "history")
 
 
 @pytest.mark.parametrize("bitwidth", [2, 4, 8])

@@ -89,6 +89,52 @@ ECQ_H1 = np.array([-0.5, 0.25, -0.25, 0.0, 0, 0, 0, 0], np.float32)
 ECQ_DECODED = np.array([1, 0, 1, 1, 2, 2, 2, -1], np.float32)
 
 
+# Two longer messages, derived by hand in the same way, that reach the places where the body reads its scratch back
+# with payload bytes in it (ecq_body.h:171,180: the scratch GH starts at out[0], the payload Q at out[10]).  In both,
+# max |G| = s, so gap = gap_inverse = 1 and f = |G| + s; alpha = 1, beta = 0.5, H = 0, seed 0; slot j of byte x draws
+# u = float(X / 4294967295.0) with X = A_{j+2} (x) + C_{j+2} mod 2^32, (A_2, C_2) = (3265436265, 3554416254),
+# (A_3, C_3) = (2155723957, 2802067423)  (naive_random.hpp:15-69, one discarded draw after srand(t + x)).
+#
+# 8 bits (s = 127, one element per byte), N = 20, M = 20, the loop covers bytes 0..18:
+#   byte 0: f = 254,    u = 3554416254/(2^32-1) = 0.82758 -> code 254 = FE  -> out[10], byte 2 of GH[2]
+#   byte 1: f = 128.5,  u = 2524885223/(2^32-1) = 0.58787 -> 129.09 -> 81   -> out[11], byte 3 of GH[2];  H[1] = 128.5 - 129 = -0.5
+#   byte 2: GH[2] was 0.5 = 3F000000 and now reads 81FE0000 = -9.3e-38: f = 127 - 9.3e-38 = 127, u = 0.34816 -> 7F -> out[12],
+#           byte 0 of GH[3];  H[2] = 0
+#   byte 3: GH[3] was 2.25 = 40100000 and now reads 4010007F = 2.25 + 127 * 2^-22: f = 129.2500303 rounds to 129.25 + 2 * 2^-16,
+#           u = 0.10846 -> 81;  H[3] = f - 129 = 0.250030517578125
+#   bytes 4..18: untouched scratch, e.g. byte 8: f = 127.25, u = 3908102598/(2^32-1) = 0.90993 -> 128.16 -> 80, H[8] = -0.75
+#   byte 19 is never written: it keeps out[29], byte 1 of GH[7] = 1 + 2^-15 = 3F800100 -> 01;  H[19] stays
+#   header: int32 30 | 127.0f | 8 | 0
+ECQ8_G = np.array([127.0, -1.5, 0.5, -2.25, 3.0, 10.75, -100.0, 1 + 2.0 ** -15, 0.25, 7.0, -31.5, 63.0, -0.125, 90.0, 5.5, -12.0,
+                   126.0, 1.0, -2.0, 33.0], np.float32)
+ECQ8_MSG = bytes([30, 0, 0, 0]) + np.float32(127.0).tobytes() + bytes([8, 0]) + bytes.fromhex("fe817f81828ae38080869ebe80d9848bfd808101")
+ECQ8_H1 = np.array([0.0, -0.5, 0.0, 0.250030517578125, 0.0, -0.25, 0.0, 2.0 ** -15, -0.75, 0.0, 0.5, 0.0, -0.875, 0.0, 0.5, 0.0,
+                    0.0, 0.0, 0.0, 0.0], np.float32)
+# 4 bits (s = 7, two elements per byte), N = 36, M = 18, the loop covers bytes 0..16:
+#   byte 0: elements 0, 1: f = 14, 7.5; u = 0.82758, 2802067423/(2^32-1) = 0.65241 -> codes 14, 8 -> 8E -> out[10], byte 2 of GH[2]
+#   byte 1: element 2 was 1.0 = 3F800000 and now reads 3F8E0000 = 1.109375: f = 8.109375, u = 0.58787 -> 8, H[2] = 0.109375;
+#           element 3: f = 9.25, u = 662824084/(2^32-1) = 0.15433 -> 9, H[3] = 0.25 -> 98
+#   byte 2 onwards: untouched scratch (byte x reads out[8x .. 8x+7] and writes out[10 + x])
+#   byte 17 is never written: it keeps out[27], byte 3 of GH[6] = 1.5 + 2^-10 = 3FC02000 -> 3F;  H[34], H[35] stay
+#   header: int32 28 | 7.0f | 4 | 0
+ECQ4_G = np.array([7.0, -0.5, 1.0, 2.25, -3.0, 4.75, 1.5 + 2.0 ** -10, 0.25, 6.0, -6.5, 0.0, 3.5, -1.25, 5.0, 2.0, -2.75, 0.75, 4.0,
+                   -5.25, 1.0, 3.0, 0.5, -6.0, 2.5, 1.75, -0.25, 5.5, 4.25, -3.75, 0.125, 6.75, 2.0, -1.0, 3.25, 0.5, -4.5], np.float32)
+ECQ4_MSG = bytes([28, 0, 0, 0]) + np.float32(7.0).tobytes() + bytes([4, 0]) + bytes.fromhex("8e98ca78eda7c899b88c8a9d79bd7b9da83f")
+ECQ4_H1 = np.array([0.0, -0.5, 0.109375, 0.25, 0.0, -0.25, 0.5009765625, 0.25, 0.0, -0.5, 0.0, 0.5, 0.25, 0.0, 0.0, 0.75, -0.25, 0.0,
+                    0.25, 0.0, 0.0, -0.5, 0.0, 0.5, -0.25, 0.25, -0.5, 0.25, -0.25, 0.125, 0.75, 0.0, 0.0, 0.25, 0.0, 0.0], np.float32)
+ECQ_LONG = ((8, ECQ8_G, ECQ8_MSG, ECQ8_H1), (4, ECQ4_G, ECQ4_MSG, ECQ4_H1))
+
+
+@pytest.mark.parametrize("bitwidth,G,want,h_want", ECQ_LONG, ids=["8bit", "4bit"])
+def test_hand_derived_messages_that_reread_the_scratch(oracle_cpu, bitwidth, G, want, h_want):
+    h = np.zeros(G.size, np.float32)
+    rc, msg, defined = oracle_cpu.ecq_encode(G.copy(), h, 1.0, 0.5, bitwidth, 0)
+    assert rc == 0 and defined and msg.tobytes() == want, msg.tobytes().hex()
+    assert np.array_equal(h, h_want), h
+    m, h2, d = _model_encode(G, np.zeros(G.size, np.float32), 1.0, 0.5, bitwidth, 0)
+    assert m.tobytes() == want and np.array_equal(h2, h_want) and d
+
+
 def test_hand_derived_message(oracle_cpu):
     h = np.zeros(8, np.float32)
     rc, msg, defined = oracle_cpu.ecq_encode(ECQ_G.copy(), h, 1.0, 0.5, 2, 0)
