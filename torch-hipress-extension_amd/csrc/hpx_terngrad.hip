@@ -197,6 +197,25 @@ __device__ __forceinline__ void ld4_stream_to_lds(const float* p, float4* lds_wa
 // Waits for every vector-memory load of the wave, LDS-bound ones included.
 __device__ __forceinline__ void wait_vector_loads() { __asm__ volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
+// A row of a register ring: requested into the very registers that held the row before (the operand is tied, so the
+// register allocator has no choice to make and nothing to spill), and waited for by count.  The compiler does not
+// know that the registers are written later than the request: between ring_request(row) and ring_wait(row) the row
+// must not be touched, and ring_wait's count must not exceed the number of vector-memory instructions that are
+// certain to have been issued after the request (loads and stores complete in the order of their issue).
+typedef float ring_f32x4 __attribute__((ext_vector_type(4)));
+template <int OFFSET>
+__device__ __forceinline__ void ring_request(float4& row, const float* uniform_base, uint32_t byte_offset) {
+  ring_f32x4 t = {row.x, row.y, row.z, row.w};
+  __asm__ volatile("global_load_dwordx4 %0, %1, %2 offset:%3 nt ; ring request" : "+v"(t) : "v"(byte_offset), "s"(uniform_base), "n"(OFFSET) : "memory");
+  row = make_float4(t.x, t.y, t.z, t.w);
+}
+template <int COUNT>
+__device__ __forceinline__ void ring_wait(float4& row) {
+  ring_f32x4 t = {row.x, row.y, row.z, row.w};
+  __asm__ volatile("s_waitcnt vmcnt(%1) ; ring wait %0" : "+v"(t) : "n"(COUNT) : "memory");
+  row = make_float4(t.x, t.y, t.z, t.w);
+}
+
 // min, max and min |x| over four elements: six instructions.
 __device__ __forceinline__ void acc3x4(const float4& v, float& mn, float& mx, float& am) {
   mn = vmin3(mn, v.x, v.y); mx = vmax3(mx, v.x, v.y); am = vmin3_abs(am, v.x, v.y);
@@ -565,9 +584,11 @@ __device__ __forceinline__ uint32_t quant_unit_prepared(const float4 (&v)[UNIT /
 //
 // STREAMED: the tensor is larger than the chip can hold.  The workgroups' shares (the first stream_u0 units) stay on
 // chip as described; the rest is dealt out in contiguous pieces of stream_units units per workgroup and streamed
-// twice by the same launch: before the share is loaded, for its extremes, and after the share has been quantised,
-// to be quantised itself.  The tensor's head is read once, the rest twice: 4 (2 - share/n) bytes per element where
-// the two-launch encode reads 8.
+// twice by the same launch: before the share is loaded, for its extremes, and again to be quantised.  The second
+// time round it passes through a ring made of the first sixteen register rows themselves: a row is requested for
+// the streamed part the moment its row of the share has been quantised, so memory is busy again from the first
+// row of pass 2 on, while the rest of the share (arithmetic only) is still being worked on.  The tensor's head is
+// read once, the rest twice: 4 (2 - share/n) bytes per element where the two-launch encode reads 8.
 constexpr int kResStreamIters = 8;  // units per lane and round of a streaming loop (128 KiB per workgroup in flight at 2 bits)
 
 template <int B, bool RANDOM, int PRE, bool STREAMED = false>
@@ -612,7 +633,16 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
   // rows' work is left when the last byte has landed.  This is one straight block per case - a
   // workgroup whose register rows are all whole, and the others - because behind a join of the
   // two the compiler no longer knows the order of the loads and waits for all of them at once.
-  float4 v[KU][H];
+  // STREAMED: pass 2 streams through two buffers of SW float4 per lane.  They are the first 2 SW register rows
+  // themselves: a row is requested again, for the streamed part, as soon as its share of the head has been quantised,
+  // so that memory works through the whole of pass 2 and the buffers cost no registers of their own.
+  constexpr int SW = STREAMED ? kResStreamIters / H : 1;  // float4 per lane and round: the same at every width
+  constexpr int KV = (STREAMED && 2 * SW > KU) ? 2 * SW : KU;
+  float4 v[KV][H];
+#pragma unroll
+  for (int k = KU; k < KV; k++)
+#pragma unroll
+    for (int h = 0; h < H; h++) v[k][h] = make_float4(0.f, 0.f, 0.f, 0.f);
   float4* s_pre = s_rows + size_t(a.lds_rows) * H * kResThreads;
   float mn = __builtin_inff(), mx = -__builtin_inff(), am = __builtin_inff();
   uint32_t fz = 0xFFFFFFFFu;
@@ -772,20 +802,20 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
       draw[q] = lcg_mul(j + 2) * (x0 + jb) + lcg_add(j + 2);
     }
   }
-  // STREAMED: the first two rounds of the streamed part are requested as soon as the register rows are done and
-  // their registers free, so that memory works while the LDS rows of the share are quantised.  (Requesting them
-  // earlier, between the register rows, made the compiler spill.)
-  constexpr int SW = STREAMED ? kResStreamIters / H : 1;  // float4 per lane and round: the same at every width
   constexpr uint32_t kRound = uint32_t(SW) * kResThreads;
-  float4 w0[SW][H], w1[SW][H];
-  auto fetch = [&](float4 (&w)[SW][H], uint32_t t0) {
-#pragma unroll
-    for (int k = 0; k < SW; k++) {
-      const uint32_t u = t0 + k * kResThreads + threadIdx.x;
-#pragma unroll
-      for (int h = 0; h < H; h++)
-        w[k][h] = (STREAMED && u < st_end) ? ld4_stream(xp + size_t(u) * UNIT + h * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
-    }
+  // STREAMED: rows 0 .. 2 SW - 1 of `v` are a ring for the streamed part.  A row's address is a uniform pointer plus
+  // a 32-bit lane offset, and the request is unconditional: a lane past the end of the workgroup's piece reads the
+  // piece's last unit (any unit of the tensor, for a workgroup without a piece) and the value is never stored.
+  constexpr int RG = 2 * SW;
+  const uint32_t lane_off = threadIdx.x * (UNIT * 4);
+  const uint32_t st_last = (st_end > st_u0 ? st_end : full_units) - 1u;  // uniform; STREAMED tensors have units
+  auto fetch_row = [&](int k, uint32_t r0) {  // r0, uniform: the row's first unit
+    const uint32_t b0 = r0 < st_last ? r0 : st_last;
+    const uint32_t room = (st_last - b0) * (UNIT * 4);
+    const float* rowp = xp + size_t(b0) * UNIT;
+    const uint32_t off = lane_off < room ? lane_off : room;
+    ring_request<0>(v[k][0], rowp, off);
+    if (H > 1) ring_request<16>(v[k][H - 1], rowp, off);
   };
   // A workgroup whose register rows are all whole (every one but the last with a share) stores
   // without a bounds check per row: the checks cost a branch each.
@@ -806,12 +836,14 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
 #pragma unroll
         for (int jb = 0; jb < BPU; jb++) pay[size_t(u) * BPU + jb] = uint8_t(packed >> (8 * jb));
       }
+      if (STREAMED && k < RG) fetch_row(k, st_u0 + uint32_t(k) * kResThreads);  // the row is free: first trip of the ring
     }
   };
-  if (whole_rows) register_rows(std::true_type{}); else register_rows(std::false_type{});
+  // (a tensor that is streamed fills every workgroup's share)
+  if (STREAMED || whole_rows) register_rows(std::true_type{}); else register_rows(std::false_type{});
   if (STREAMED) {
-    fetch(w0, st_u0);
-    fetch(w1, st_u0 + kRound);
+#pragma unroll
+    for (int k = KU; k < RG; k++) fetch_row(k, st_u0 + uint32_t(k) * kResThreads);
   }
   if (RANDOM) {
     uint32_t x0 = a.seg.seed + l0 * BPU;
@@ -845,26 +877,33 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
         draw[q] = lcg_mul(j + 2) * (x0 + jb) + lcg_add(j + 2);
       }
     }
-    // Two rounds in flight: the loads of the next round are requested before this round is worked on (the waves
-    // of a workgroup leave the barrier together and would otherwise all load, then all compute).  The first two
-    // rounds have been on their way since the register rows.
-    auto emit = [&](float4 (&w)[SW][H], uint32_t t0) {
+    // One trip round the ring per iteration: a row is waited for, quantised, stored and requested again for the
+    // next trip.  Of the rows requested after it, RG - 1 are certain to have been issued when a row is waited for
+    // (the stores between them are not counted: a wave none of whose lanes stores skips the instruction).
+    auto half = [&](auto base, uint32_t t0) {
 #pragma unroll
-      for (int k = 0; k < SW; k++) {
+      for (int k = decltype(base)::value; k < decltype(base)::value + SW; k++) {
         const uint32_t u = t0 + k * kResThreads + threadIdx.x;
-        const uint32_t packed = quant_unit<B, RANDOM>(w[k], mn, gi, draw, uint32_t(kResThreads) * BPU);
+#pragma unroll
+        for (int h = 0; h < H; h++) ring_wait<(RG - 1) * H>(v[k][h]);
+        const uint32_t packed = quant_unit<B, RANDOM>(v[k], mn, gi, draw, uint32_t(kResThreads) * BPU);
         if (u < st_end) {
 #pragma unroll
           for (int jb = 0; jb < BPU; jb++) pay[size_t(u) * BPU + jb] = uint8_t(packed >> (8 * jb));
         }
+        fetch_row(k, t0 + uint32_t(RG + k) * kResThreads);
       }
     };
     for (uint32_t t0 = st_u0; t0 < st_end; t0 += 2 * kRound) {
-      emit(w0, t0);
-      fetch(w0, t0 + 2 * kRound);
-      if (t0 + kRound < st_end) emit(w1, t0 + kRound);
-      fetch(w1, t0 + 3 * kRound);
+      half(std::integral_constant<int, 0>{}, t0);
+      if (t0 + kRound >= st_end) break;
+      half(std::integral_constant<int, SW>{}, t0);
     }
+    // Requests of the last trips are still on their way: the ring's registers stay taken until they have landed.
+#pragma unroll
+    for (int k = 0; k < RG; k++)
+#pragma unroll
+      for (int h = 0; h < H; h++) ring_wait<0>(v[k][h]);
   }
   // The unit that holds the end of the tensor, if the length is not a whole number of units.
   if (blockIdx.x == 0 && threadIdx.x == 0 && full_units * UNIT < n) {
