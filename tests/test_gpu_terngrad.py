@@ -737,6 +737,55 @@ def test_resident_bucket_many_rows_and_full_table(tg, oracle_cpu, capi, bucket_f
         assert_bits_equal(host(outs[i]), ref, f"message[{i}] n={x.size}")
 
 
+def _resnet50_sizes():
+    sizes = [64 * 3 * 7 * 7, 64, 64]
+    inp = 64
+    for planes, blocks in ((64, 3), (128, 4), (256, 6), (512, 3)):
+        for blk in range(blocks):
+            sizes += [planes * inp, planes, planes, planes * planes * 9, planes, planes, planes * 4 * planes, planes * 4, planes * 4]
+            if blk == 0:
+                sizes += [planes * 4 * inp, planes * 4, planes * 4]
+            inp = planes * 4
+    return sizes + [1000 * 2048, 1000]
+
+
+@pytest.mark.parametrize("b,rnd", [(2, 1), (2, 0), (1, 1), (8, 1)])
+def test_resident_bucket_of_resnet50s_tensors(tg, oracle_cpu, capi, bucket_forced, b, rnd):
+    """The 161 parameter tensors of ResNet-50 (25 557 032 elements; 107 of them biases and normalisation parameters of
+    at most 2048 elements, which the waves without a piece encode on their own) in one launch, every message against
+    the oracle."""
+    sizes = _resnet50_sizes()
+    assert len(sizes) == 161 and sum(sizes) == 25_557_032
+    rng = np.random.default_rng(3300 + b)
+    xs = [rng.normal(0, 1e-2, n).astype(np.float32) for n in sizes]
+    xs[1][:] = 0.0; xs[2][3] = -0.0; xs[2][7] = 0.0; xs[2] = np.abs(xs[2]); xs[2][3] = -0.0   # tiny tensors with zero extremes
+    dx = [dev(x) for x in xs]
+    seeds = [int(v) for v in rng.integers(0, 2**63, len(sizes))]
+    before = _bucket_launches(capi)
+    outs = tg.encode(dx, [b] * len(xs), [rnd] * len(xs), seeds)
+    torch.cuda.synchronize()
+    # (one bit with stochastic rounding keeps fewer rows in registers: the list then takes two launches)
+    assert _bucket_launches(capi) == before + (2 if (b, rnd) == (1, 1) else 1)
+    for i, x in enumerate(xs):
+        rc, ref = oracle_cpu.terngrad_encode(x, b, rnd, seeds[i])
+        assert rc == 0
+        assert_bits_equal(host(outs[i]), ref, f"message[{i}] n={x.size}")
+
+
+def test_resident_bucket_of_nothing_but_tiny_tensors(tg, oracle_cpu, capi, bucket_forced):
+    rng = np.random.default_rng(35)
+    for b in (1, 2, 4, 8):
+        unit = max(4, 8 // b)
+        sizes = [1, unit - 1, unit, 63, 64, 1000, 2048, 8 * 64 * unit, 8 * 64 * unit - 1] + [int(v) for v in rng.integers(1, 8 * 64 * unit, 40)]
+        xs = [rng.normal(0, 1e-2, n).astype(np.float32) for n in sizes]
+        before = _bucket_launches(capi)
+        _check(tg, oracle_cpu, xs, [b] * len(xs), [1] * len(xs), [int(v) for v in rng.integers(0, 2**63, len(xs))], [0] * len(xs), rng)
+        assert _bucket_launches(capi) == before + 1
+        # one tensor just above the limit among them: the others ride on the waves it leaves free
+        xs.append(rng.normal(0, 1e-2, 8 * 64 * unit + unit).astype(np.float32))
+        _check(tg, oracle_cpu, xs, [b] * len(xs), [1] * len(xs), [int(v) for v in rng.integers(0, 2**63, len(xs))], [0] * len(xs), rng)
+
+
 def test_resident_bucket_groups_of_a_large_call(tg, oracle_cpu, capi, bucket_forced):
     # 77 M elements: more than the chip holds, so the call becomes three resident launches (5 + 5 + 3 tensors);
     # then a call whose widths change half way: two launches

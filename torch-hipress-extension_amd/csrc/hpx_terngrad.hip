@@ -934,14 +934,22 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
 // least one piece; the piece that ends a tensor also takes the 1..UNIT-1 elements
 // behind its last whole unit).
 //
+// Tiny tensors (at most 2048 elements: the biases and normalisation parameters that make up two thirds of a
+// convolutional network's tensor list) get no piece - each would cost a wave that could hold `rows` rows.  They are
+// dealt out to the waves that are left without a piece, which encode them start to finish on their own (a wave's
+// reduction gives the tensor's extremes; no slots, no barrier) while the others load.
+//
 // The extremes travel through the epoch-tagged slots of the tiled kernels: a wave
 // folds its piece into way (piece index % kSlotWays) of its tensor's three slots with
 // atomic max operations whose results it waits for, the grid meets at the barrier of
 // grid_exchange (its payload unused), and every wave then folds the ways of its
 // tensor.
+// A tensor of at most this many rows of 64 units is "tiny": 2048 elements at every width.
+constexpr int tiny_rows(int bits) { return bits == 1 ? 4 : 8; }
+constexpr int kTinyPerWave = 2;  // tiny tensors a left-over wave takes at a time
 struct ResMultiArgs {
   int32_t nseg;
-  int32_t piece_start[kCapLarge + 1];
+  int32_t piece_start[kCapLarge + 1];  // (a tiny tensor's entry equals the next one's)
   EncSeg seg[kCapLarge];
   uint64_t* slots;
   uint32_t epoch;
@@ -953,8 +961,112 @@ struct ResMultiArgs {
   uint64_t spin_limit;
   uint64_t* stamps;    // measurement aid, normally null (phase_stamp)
   uint32_t* done;      // pinned host words, one per workgroup: set to `gen` by a workgroup that got through the barrier
+  int32_t ntiny;       // tensors without a piece: the waves without a piece encode them on their own
+  int16_t tiny[kCapLarge];  // their indices
 };
 static_assert(sizeof(ResMultiArgs) <= 9600, "kernel-argument budget");
+
+// One wave encodes kTinyPerWave whole tensors of at most tiny_rows * 64 units each (plus the elements behind their
+// last whole units), in two steps.  tiny_request asks for the tensors' rows, into the registers the wave would
+// hold a piece in, when the kernel starts: the requests queue behind those of the fifteen waves beside it and
+// land about when their pieces have (a CU serves its waves' requests in order).  tiny_finish does the rest behind
+// the grid's barrier, when memory is idle and the other waves quantise: the tensors' extremes from the wave's own
+// reduction, the header, the codes.
+template <int B>
+struct TinyShape {
+  static constexpr int DPB = 8 / B;
+  static constexpr int UNIT = DPB > 4 ? DPB : 4;
+  static constexpr int H = UNIT / 4;
+  static constexpr int BPU = UNIT / DPB;
+  static constexpr int ROWS = tiny_rows(B);
+};
+template <int B, int KV>
+__device__ __forceinline__ void tiny_request(const ResMultiArgs& a, int t0, int step, uint32_t lane, float4 (&v)[KV][TinyShape<B>::H]) {
+  using S = TinyShape<B>;
+  static_assert(kTinyPerWave * S::ROWS <= KV, "the tiny tensors' rows must fit the wave's register rows");
+  const float qnan = __builtin_nanf("");
+#pragma unroll
+  for (int i = 0; i < kTinyPerWave; i++) {
+    const bool have = t0 + i * step < a.ntiny;  // wave-uniform
+    const EncSeg& sg = a.seg[a.tiny[have ? t0 + i * step : t0]];
+    const uint32_t full_units = have ? static_cast<uint32_t>(sg.n) / S::UNIT : 0u;
+#pragma unroll
+    for (int k = 0; k < S::ROWS; k++) {
+      const uint32_t u = k * kWave + lane;
+#pragma unroll
+      for (int h = 0; h < S::H; h++)
+        v[i * S::ROWS + k][h] = u < full_units ? ld4_stream(sg.x + (u * S::UNIT + h * 4)) : make_float4(qnan, qnan, qnan, qnan);
+    }
+  }
+}
+template <int B, bool RANDOM, int KV>
+__device__ __forceinline__ void tiny_finish(const ResMultiArgs& a, int t0, int step, uint32_t lane, const float4 (&v)[KV][TinyShape<B>::H]) {
+  using S = TinyShape<B>;
+  constexpr int DPB = S::DPB, UNIT = S::UNIT, H = S::H, BPU = S::BPU, ROWS = S::ROWS;
+  constexpr uint32_t stride_bytes = uint32_t(kWave) * BPU;
+#pragma unroll
+  for (int i = 0; i < kTinyPerWave; i++) {
+    if (t0 + i * step >= a.ntiny) break;  // wave-uniform
+    const EncSeg& sg = a.seg[a.tiny[t0 + i * step]];
+    const float* __restrict__ xp = sg.x;
+    const uint32_t n = static_cast<uint32_t>(sg.n);
+    const uint32_t full_units = n / UNIT;
+    float mn = __builtin_inff(), mx = -__builtin_inff(), am = __builtin_inff();
+#pragma unroll
+    for (int k = 0; k < ROWS; k++)
+#pragma unroll
+      for (int h = 0; h < H; h++) acc3x4(v[i * ROWS + k][h], mn, mx, am);
+    uint32_t fz = 0xFFFFFFFFu;
+    if (am == 0.0f) {
+      float d0 = 0.f, d1 = 0.f;
+#pragma unroll
+      for (int k = 0; k < ROWS; k++)
+#pragma unroll
+        for (int h = 0; h < H; h++) acc_zero4(v[i * ROWS + k][h], (k * kWave + lane) * UNIT + h * 4, d0, d1, fz);
+    }
+    if (lane == 0)
+      for (uint32_t e = full_units * UNIT; e < n; e++) acc_zero(xp[e], e, mn, mx, fz);
+    mn = wave_min(mn);
+    mx = wave_max(mx);
+    fz = wave_min_u32(fz);
+    if ((mn == 0.0f || mx == 0.0f) && fz != 0xFFFFFFFFu) {  // a zero extreme carries the sign of the tensor's first zero
+      const float zv = xp[fz];
+      if (mn == 0.0f) mn = zv;
+      if (mx == 0.0f) mx = zv;
+    }
+    const float gi = inverse_gap(mn, mx, B);
+    if (lane == 0) write_header(sg.out, B, n, mn, mx);
+    uint8_t* __restrict__ pay = sg.out + 10;
+    uint32_t draw[UNIT];
+    if (RANDOM) {
+      const uint32_t x0 = sg.seed + lane * BPU;
+#pragma unroll
+      for (int q = 0; q < UNIT; q++) {
+        const int jb = q / DPB, j = q % DPB;
+        draw[q] = lcg_mul(j + 2) * (x0 + jb) + lcg_add(j + 2);
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < ROWS; k++) {
+      if (uint32_t(k) * kWave >= full_units) break;  // wave-uniform: most tiny tensors are a row or two
+      const uint32_t u = k * kWave + lane;
+      const uint32_t packed = quant_unit<B, RANDOM>(v[i * ROWS + k], mn, gi, draw, stride_bytes);
+      if (u < full_units) {
+#pragma unroll
+        for (int jb = 0; jb < BPU; jb++) pay[u * BPU + jb] = uint8_t(packed >> (8 * jb));
+      }
+    }
+    if (lane == 0 && full_units * UNIT < n) {
+      uint32_t d[UNIT];
+#pragma unroll
+      for (int q = 0; q < UNIT; q++) {
+        const int jb = q / DPB, j = q % DPB;
+        d[q] = lcg_mul(j + 2) * (sg.seed + full_units * BPU + jb) + lcg_add(j + 2);
+      }
+      quant_unit_ragged<B, RANDOM>(sg, mn, gi, full_units, d);
+    }
+  }
+}
 
 template <int B, bool RANDOM, int PRE>
 __global__ __launch_bounds__(kResThreads) void terngrad_resident_multi_kernel(const ResMultiArgs a) {
@@ -996,9 +1108,14 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_multi_kernel(co
   // As in the single-tensor kernel: all loads at once (the LDS rows, straight into LDS, ahead of the register rows), the
   // random addends of the first PRE rows while they are in flight, then every row reduced as it arrives,
   // one straight block per case.
-  float4 v[KU][H];
+  constexpr int KV = kTinyPerWave * tiny_rows(B) > KU ? kTinyPerWave * tiny_rows(B) : KU;
+  float4 v[KV][H];
   float mn = __builtin_inff(), mx = -__builtin_inff(), am = __builtin_inff();
   const bool whole_rows = u_beg + uint32_t(KU * kWave) <= u_end;
+  // A wave without a piece may have tiny tensors to encode (the host leaves at least ntiny / kTinyPerWave such
+  // waves: wave total + t takes tensors t and t + nidle of the list).
+  const int nidle = int(gridDim.x) * kWaves - total;
+  const bool has_tiny = !active && my_piece - total < a.ntiny;
   const uint32_t ul0 = u0 + uint32_t(KU) * kWave;  // this lane's unit in the first LDS row
   for (uint32_t r = 0; r < a.lds_rows; r++) {
     const uint32_t u = ul0 + r * kWave;
@@ -1039,7 +1156,9 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_multi_kernel(co
 #pragma unroll
       for (int h = 0; h < H; h++) acc3x4(v[k][h], mn, mx, am);
   };
-  if (whole_rows) pass1(std::true_type{}); else pass1(std::false_type{});
+  if (whole_rows) pass1(std::true_type{});
+  else if (!has_tiny) pass1(std::false_type{});
+  else tiny_request<B>(a, my_piece - total, nidle, lane, v);
   if (a.lds_rows > 0) wait_vector_loads();
   for (uint32_t r = 0; r < a.lds_rows; r++) {
     if (ul0 + r * kWave < u_end) {
@@ -1095,7 +1214,15 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_multi_kernel(co
   for (int q = 0; q < kBarWaves; q++) oks &= s_ok[q];
   if (oks == 0u) return;
   if (threadIdx.x == 0) __hip_atomic_store(a.done + blockIdx.x, a.gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-  if (!active) return;
+  if (!active) {
+    if (has_tiny) {
+      tiny_finish<B, RANDOM>(a, my_piece - total, nidle, lane, v);
+      if (a.stamps && lane == 0)
+        __hip_atomic_fetch_max(reinterpret_cast<unsigned long long*>(a.stamps) + size_t(blockIdx.x) * 4 + 3,
+                               static_cast<unsigned long long>(wall_clock64()), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    return;
+  }
   phase_stamp(a.stamps, 2);
 
   // ---- pass 2: the tensor's extremes, then quantise from registers ----------------
@@ -1879,15 +2006,23 @@ bool resident_multi_plan(int count, const int32_t* in_sizes, const uint8_t* bitw
   const int64_t waves = int64_t(resident_grid(ws)) * (kResThreads / kWave);
   int64_t total_units = 0;
   for (int i = 0; i < count; i++) total_units += in_sizes[i] / unit;
+  // Tiny tensors take no piece; kTinyPerWave of them share a wave that has none.  (With nothing but tiny tensors
+  // there would be no piece at all: then they are tensors like any other.)
+  int ntiny = 0;
+  for (int i = 0; i < count; i++) ntiny += in_sizes[i] / unit <= tiny_rows(bits) * kWave ? 1 : 0;
+  if (ntiny == count) ntiny = 0;
+  const bool riders = ntiny > 0;
+  auto is_tiny = [&](int i) { return riders && in_sizes[i] / unit <= tiny_rows(bits) * kWave; };
+  const int64_t tiny_waves = (ntiny + kTinyPerWave - 1) / kTinyPerWave;
   int64_t rows = (total_units + waves * kWave - 1) / (waves * kWave);
   if (rows < 1) rows = 1;
   for (; rows <= reg_rows + lds_rows_max; rows++) {
     int64_t pieces = 0;
     for (int i = 0; i < count; i++) {
       const int64_t p = (in_sizes[i] / unit + rows * kWave - 1) / (rows * kWave);
-      pieces += p < 1 ? 1 : p;
+      pieces += is_tiny(i) ? 0 : (p < 1 ? 1 : p);
     }
-    if (pieces <= waves) break;
+    if (pieces + tiny_waves <= waves) break;
   }
   if (rows > reg_rows + lds_rows_max) return false;
   ma.rows = static_cast<uint32_t>(rows);
@@ -1899,10 +2034,12 @@ bool resident_multi_plan(int count, const int32_t* in_sizes, const uint8_t* bitw
   else if (random && spare_rows >= res_pre_rows(bits) * 3 / 4) pre_rows = static_cast<uint32_t>(res_pre_rows(bits) * 3 / 4);
   else if (random && spare_rows >= res_pre_rows(bits) / 2) pre_rows = static_cast<uint32_t>(res_pre_rows(bits) / 2);
   ma.nseg = count;
+  ma.ntiny = 0;
   ma.piece_start[0] = 0;
   for (int i = 0; i < count; i++) {
     const int64_t p = (in_sizes[i] / unit + rows * kWave - 1) / (rows * kWave);
-    ma.piece_start[i + 1] = ma.piece_start[i] + static_cast<int32_t>(p < 1 ? 1 : p);
+    ma.piece_start[i + 1] = ma.piece_start[i] + (is_tiny(i) ? 0 : static_cast<int32_t>(p < 1 ? 1 : p));
+    if (is_tiny(i)) ma.tiny[ma.ntiny++] = static_cast<int16_t>(i);
   }
   return true;
 }
