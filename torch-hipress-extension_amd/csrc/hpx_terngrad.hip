@@ -927,23 +927,25 @@ __global__ __launch_bounds__(kResThreads) void terngrad_resident_kernel(const Re
 // one tensor, held by one wave (register rows first, LDS rows after them), so the
 // tensor, its extremes and its seed are wave-uniform and the inner loops are those
 // of the single-tensor kernel.  Piece p belongs to wave p / G of workgroup p % G (G workgroups):
-// consecutive pieces go to consecutive workgroups, so every CU gets the same mix of whole pieces,
-// tensor ends and tiny tensors (with piece p on wave p % 16 of workgroup p / 16 the workgroups that
+// consecutive pieces go to consecutive workgroups, so every CU gets the same mix of whole pieces
+// and tensor ends (with piece p on wave p % 16 of workgroup p / 16 the workgroups that
 // held sixteen whole pieces of a large tensor set the pace of both passes);
-// the host picks the smallest `rows` for which all pieces fit (every tensor has at
+// the host picks the smallest `rows` for which all pieces fit (every tensor that is not tiny has at
 // least one piece; the piece that ends a tensor also takes the 1..UNIT-1 elements
 // behind its last whole unit).
 //
 // Tiny tensors (at most 2048 elements: the biases and normalisation parameters that make up two thirds of a
 // convolutional network's tensor list) get no piece - each would cost a wave that could hold `rows` rows.  They are
-// dealt out to the waves that are left without a piece, which encode them start to finish on their own (a wave's
-// reduction gives the tensor's extremes; no slots, no barrier) while the others load.
+// dealt out to the waves that are left without a piece, two to a wave, which request them at the start and encode
+// them start to finish on their own behind the barrier, while the others quantise (a wave's reduction gives a
+// tensor's extremes: no slots).
 //
 // The extremes travel through the epoch-tagged slots of the tiled kernels: a wave
 // folds its piece into way (piece index % kSlotWays) of its tensor's three slots with
 // atomic max operations whose results it waits for, the grid meets at the barrier of
 // grid_exchange (its payload unused), and every wave then folds the ways of its
 // tensor.
+
 // A tensor of at most this many rows of 64 units is "tiny": 2048 elements at every width.
 constexpr int tiny_rows(int bits) { return bits == 1 ? 4 : 8; }
 constexpr int kTinyPerWave = 2;  // tiny tensors a left-over wave takes at a time
