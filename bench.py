@@ -91,10 +91,11 @@ def settle(torch, fn, seconds=None):
         torch.cuda.synchronize()
 
 
-def timed(torch, fn, steps, warmup):
+def timed(torch, fn, steps, warmup, settled=True):
     for _ in range(warmup):
         fn()
-    settle(torch, fn)
+    if settled:
+        settle(torch, fn)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
@@ -245,6 +246,9 @@ def main():
 
     for _ in range(args.copy_calibration):
         sets[0][2].copy_(sets[0][0])  # reads 4*N bytes, writes 4*N bytes
+    # the same K steps once more, first, straight after the W warm-up steps of a process that has done nothing yet:
+    # reported beside the settled figure (path_roofline.cold_start_ms_per_step), never as `value`
+    sec_cold = timed(torch, step, args.steps, args.warmup, settled=False)
     sec = timed(torch, step, args.steps, args.warmup)
     value = 4.0 * n / sec / 1e9
 
@@ -289,6 +293,8 @@ def main():
             "warm_cache_ms_per_step": round(sec_warm * 1e3, 4), "encode_ms": round(sec_enc * 1e3, 4),
             "decode_ms": round(sec_dec * 1e3, 4), "buffer_sets": len(sets),
             "wall_clock_mean_ms_per_step": round(sec * 1e3, 5),
+            "cold_start_ms_per_step": round(sec_cold * 1e3, 5),
+            "cold_start_frac_of_hbm_peak": round(path_alg / sec_cold / 1e9 / HBM_PEAK_GBS, 4),
             "event_pair_ms_per_step": quantiles(pairs), "event_pair_encode_ms": quantiles(pairs_enc),
             "event_pair_decode_ms": quantiles(pairs_dec),
             "frac_of_hbm_peak_event_pair_median": round(path_alg / quantiles(pairs, 1.0, 9)["median"] / 1e9 / HBM_PEAK_GBS, 4)}
